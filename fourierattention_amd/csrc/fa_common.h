@@ -1,0 +1,76 @@
+// Shared host/device helpers for the gfx950 Fourier-attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/fourier_attn_hip.h"
+
+#define FA_WAVE 64
+
+// ---- error reporting --------------------------------------------------------
+void fa_set_error(const char* fmt, ...);
+int fa_check_launch(const char* what);
+
+#define FA_REQUIRE(cond, code, ...)      \
+  do {                                   \
+    if (!(cond)) {                       \
+      fa_set_error(__VA_ARGS__);         \
+      return (code);                     \
+    }                                    \
+  } while (0)
+
+static inline hipStream_t fa_hip_stream(fa_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+static inline int fa_cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+static inline size_t fa_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---- element types ----------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float fa_to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+__device__ __forceinline__ float fa_to_float(f16_t x) { return (float)x.v; }
+__device__ __forceinline__ float fa_to_float(float x) { return x; }
+
+// round-to-nearest-even float -> bf16 bits (NaN kept quiet)
+__device__ __forceinline__ uint16_t fa_f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float fa_round_through(float v, int dtype) {
+  if (dtype == FA_BF16) return __uint_as_float(((uint32_t)fa_f32_to_bf16_bits(v)) << 16);
+  if (dtype == FA_FP16) return (float)(_Float16)v;
+  return v;
+}
+
+// ---- exact Fourier phases ---------------------------------------------------
+// cos/sin of 2*pi*((a*b) mod T)/T; the product is reduced in integers so the
+// angle handed to the float unit is always inside one period.
+__device__ __forceinline__ void fa_sincos_phase(int64_t a, int64_t b, int T, float* s, float* c) {
+  int64_t r = (a * b) % (int64_t)T;
+  float x = 2.0f * (float)r / (float)T;  // in [0, 2)
+  sincospif(x, s, c);
+}
+
+// ---- wave / block reductions ------------------------------------------------
+__device__ __forceinline__ float fa_wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, FA_WAVE);
+  return v;
+}
+__device__ __forceinline__ float fa_wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, FA_WAVE));
+  return v;
+}
+__device__ __forceinline__ float fa_wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, FA_WAVE));
+  return v;
+}

@@ -1,0 +1,574 @@
+// Decode attention over [sink ; local window ; mid rows], any shape (generic path).
+//
+// The compressed dims of the mid rows are never rebuilt.  With s = scale,
+// a = avg_u - avg_d * s and F[l, n] = cos / sin(2 pi n l / T):
+//   score[l]  = F[l, :] . w + q_c . a + q_n . K_mn[l, :],  w = (1/N) K_coef (q_c * s)
+//   out_c     = s_v * ((1/N) V_coef^T (F^T p) - avg_d_v * P) + avg_u_v * P,  P = sum_l p[l]
+// so one pass over the coefficients before (prep) and one after (merge) replace the
+// per-token reconstruction, and the token loop only touches the stored dims.
+// All exponentials are base 2 (scores carry log2(e)).
+#include "fa_common.h"
+
+namespace {
+
+constexpr int kGMax = 8;      // query heads per KV head handled by the generic kernels
+constexpr int kTile = 256;    // tokens per tile = threads per block
+constexpr int kFreqIters = 4; // frequencies per thread in the g accumulation (N <= 1024)
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct Seg {
+  const void* k;
+  const void* v;
+  int rows;
+  int64_t bs, rs;
+};
+
+// ---------------------------------------------------------------------------
+// prep: W[b, hq, n] = (sm*log2e/N) sum_j coef[b, n, kc0 + j] q[b, hq, d_j] s[b, kc0 + j]
+//       c0[b, hq]   = sm*log2e * sum_j q[b, hq, d_j] (avg_u - avg_d s)[b, kc0 + j]
+// ---------------------------------------------------------------------------
+template <typename E>
+__global__ __launch_bounds__(256) void decode_prep_kernel(
+    const E* __restrict__ q, const float* __restrict__ k_mc, const float* __restrict__ avg_u,
+    const float* __restrict__ avg_d, const float* __restrict__ scale, const int32_t* __restrict__ kc_list,
+    const int32_t* __restrict__ kc_h, float* __restrict__ W, float* __restrict__ c0, int Hq, int Hkv, int D,
+    int N, int Ck, float sm_log2e, int rows_per_block) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int G = Hq / Hkv;
+  const int kc0 = kc_h[h], kc_len = kc_h[h + 1] - kc0;
+  float qs[kGMax][2], qa[kGMax][2];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) qs[g][0] = qs[g][1] = qa[g][0] = qa[g][1] = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj) {
+    int j = lane + 64 * jj;
+    if (j < kc_len) {
+      int d = kc_list[kc0 + j] - h * D;
+      float s = scale[(int64_t)b * Ck + kc0 + j];
+      float a = avg_u[(int64_t)b * Ck + kc0 + j] - avg_d[(int64_t)b * Ck + kc0 + j] * s;
+#pragma unroll
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) {
+          float qv = fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + d]);
+          qs[g][jj] = qv * s;
+          qa[g][jj] = qv * a;
+        }
+    }
+  }
+  if (blockIdx.x == 0 && w == 0) {
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) {
+        float v = fa_wave_sum(qa[g][0] + qa[g][1]);
+        if (lane == 0) c0[(int64_t)b * Hq + h * G + g] = v * sm_log2e;
+      }
+  }
+  const float mul = sm_log2e / (float)N;
+  const int n_beg = blockIdx.x * rows_per_block;
+  const int n_end = min(2 * N, n_beg + rows_per_block);
+  for (int n = n_beg + w; n < n_end; n += 4) {
+    const float* row = k_mc + ((int64_t)b * 2 * N + n) * Ck + kc0;
+    float v0 = lane < kc_len ? row[lane] : 0.f;
+    float v1 = lane + 64 < kc_len ? row[lane + 64] : 0.f;
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) {
+        float v = fa_wave_sum(v0 * qs[g][0] + v1 * qs[g][1]);
+        if (lane == 0) W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = v * mul;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// sink + local window: one tile of up to 256 full-width rows per block
+// ---------------------------------------------------------------------------
+template <typename E>
+__global__ __launch_bounds__(256) void decode_il_kernel(
+    const E* __restrict__ q, Seg s0, Seg s1, float* __restrict__ pm, float* __restrict__ pd,
+    float* __restrict__ po, int Hq, int Hkv, int D, int n_split, float sm_log2e) {
+  extern __shared__ float smem[];
+  const int G = Hq / Hkv;
+  float* s_q = smem;                 // [G][D]
+  float* s_p = s_q + G * D;          // [G][kTile]
+  float* s_red = s_p + G * kTile;    // [4][kGMax]
+  float* s_o = s_red + 4 * kGMax;    // [G][D] (second half accumulators)
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int n_il = s0.rows + s1.rows;
+  for (int e = tid; e < G * D; e += 256)
+    s_q[e] = fa_to_float(q[((int64_t)b * Hq + h * G) * D + e]) * sm_log2e;
+  __syncthreads();
+
+  const int i = split * kTile + tid;
+  const bool ok = i < n_il;
+  const E* krow = nullptr;
+  if (ok) {
+    krow = (i < s0.rows) ? (const E*)s0.k + (int64_t)b * s0.bs + (int64_t)i * s0.rs
+                         : (const E*)s1.k + (int64_t)b * s1.bs + (int64_t)(i - s0.rows) * s1.rs;
+    krow += h * D;
+  }
+  float sc[kGMax];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) sc[g] = 0.f;
+  if (ok) {
+    for (int d = 0; d < D; ++d) {
+      float kv = fa_to_float(krow[d]);
+#pragma unroll
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) sc[g] = fmaf(kv, s_q[g * D + d], sc[g]);
+    }
+  }
+  // tile max
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) {
+    float v = fa_wave_max(ok ? sc[g] : -INFINITY);
+    if (lane == 0) s_red[w * kGMax + g] = v;
+  }
+  __syncthreads();
+  float mx[kGMax];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g)
+    mx[g] = fmaxf(fmaxf(s_red[g], s_red[kGMax + g]), fmaxf(s_red[2 * kGMax + g], s_red[3 * kGMax + g]));
+  __syncthreads();
+  float dsum[kGMax];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) {
+    float p = (ok && g < G) ? exp2f(sc[g] - mx[g]) : 0.f;
+    if (g < G) s_p[g * kTile + tid] = p;
+    float v = fa_wave_sum(p);
+    if (lane == 0) s_red[w * kGMax + g] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g)
+    dsum[g] = s_red[g] + s_red[kGMax + g] + s_red[2 * kGMax + g] + s_red[3 * kGMax + g];
+
+  // PV: thread = (dim, half of the tile)
+  const int dim = tid % 128, half = tid / 128;
+  float o[kGMax];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) o[g] = 0.f;
+  const int t_end = min(kTile, n_il - split * kTile);
+  if (dim < D) {
+    for (int tt = half; tt < t_end; tt += 2) {
+      int ii = split * kTile + tt;
+      const E* vrow = (ii < s0.rows) ? (const E*)s0.v + (int64_t)b * s0.bs + (int64_t)ii * s0.rs
+                                     : (const E*)s1.v + (int64_t)b * s1.bs + (int64_t)(ii - s0.rows) * s1.rs;
+      float vv = fa_to_float(vrow[h * D + dim]);
+#pragma unroll
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) o[g] = fmaf(s_p[g * kTile + tt], vv, o[g]);
+    }
+  }
+  if (half == 1 && dim < D) {
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) s_o[g * D + dim] = o[g];
+  }
+  __syncthreads();
+  if (half == 0 && dim < D) {
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) {
+        int64_t r = ((int64_t)b * Hq + h * G + g) * n_split + split;
+        po[r * D + dim] = o[g] + s_o[g * D + dim];
+      }
+  }
+  if (tid < G) {
+    int64_t r = ((int64_t)b * Hq + h * G + tid) * n_split + split;
+    float m = -INFINITY, dd = 0.f;
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g == tid) {
+        m = mx[g];
+        dd = dsum[g];
+      }
+    pm[r] = m;
+    pd[r] = dd;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// mid rows: split over tokens; per split partial (m, d, g[2N], o_n[vn_len])
+// ---------------------------------------------------------------------------
+template <typename E>
+__global__ __launch_bounds__(256) void decode_mid_kernel(
+    const E* __restrict__ q, const E* __restrict__ k_mn, int64_t k_bs, int64_t k_rs,
+    const E* __restrict__ v_mn, int64_t v_bs, int64_t v_rs, const float* __restrict__ W,
+    const float* __restrict__ c0, const int32_t* __restrict__ kn_list, const int32_t* __restrict__ kn_h,
+    const int32_t* __restrict__ vn_h, float* __restrict__ pm, float* __restrict__ pd,
+    float* __restrict__ pg, float* __restrict__ pon, int Hq, int Hkv, int D, int N, int L_m, int T,
+    int n_split, int tiles_per_split, float sm_log2e) {
+  extern __shared__ float smem[];
+  const int G = Hq / Hkv;
+  float* s_w = smem;                   // [G][2N]
+  float* s_qn = s_w + G * 2 * N;       // [G][D]
+  float* s_p = s_qn + G * D;           // [G][kTile]
+  float* s_red = s_p + G * kTile;      // [4][kGMax]
+  float* s_o = s_red + 4 * kGMax;      // [G][D]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int kn0 = kn_h[h], kn_len = kn_h[h + 1] - kn0;
+  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
+
+  for (int e = tid; e < G * 2 * N; e += 256) s_w[e] = W[((int64_t)b * Hq + h * G) * 2 * N + e];
+  for (int e = tid; e < G * D; e += 256) {
+    int g = e / D, j = e % D;
+    float v = 0.f;
+    if (j < kn_len) v = fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + (kn_list[kn0 + j] - h * D)]) * sm_log2e;
+    s_qn[e] = v;
+  }
+  float cz[kGMax], m_run[kGMax], d_run[kGMax];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) {
+    cz[g] = g < G ? c0[(int64_t)b * Hq + h * G + g] : 0.f;
+    m_run[g] = -INFINITY;
+    d_run[g] = 0.f;
+  }
+  float gc[kFreqIters][kGMax], gs[kFreqIters][kGMax], on[kGMax];
+#pragma unroll
+  for (int i = 0; i < kFreqIters; ++i)
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) gc[i][g] = gs[i][g] = 0.f;
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) on[g] = 0.f;
+  __syncthreads();
+
+  const int l_beg = split * tiles_per_split * kTile;
+  const int l_end = min(L_m, l_beg + tiles_per_split * kTile);
+  const E* kb = k_mn + (int64_t)b * k_bs + kn0;
+  const E* vb = v_mn + (int64_t)b * v_bs + vn0;
+  const int dim = tid % 128, half = tid / 128;
+
+  for (int l0 = l_beg; l0 < l_end; l0 += kTile) {
+    const int t_len = min(kTile, l_end - l0);
+    // ---- phase 1: scores, thread = token --------------------------------
+    const int l = l0 + tid;
+    const bool ok = tid < t_len;
+    float sc[kGMax];
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) sc[g] = cz[g];
+    if (ok) {
+      float sr, si, zr = 1.f, zi = 0.f;
+      fa_sincos_phase(l, 1, T, &si, &sr);
+      for (int n = 0; n < N; ++n) {
+        if ((n & 63) == 0) fa_sincos_phase(l, n, T, &zi, &zr);
+#pragma unroll
+        for (int g = 0; g < kGMax; ++g)
+          if (g < G) sc[g] = fmaf(zr, s_w[g * 2 * N + n], fmaf(zi, s_w[g * 2 * N + N + n], sc[g]));
+        float nr = zr * sr - zi * si;
+        float ni = zr * si + zi * sr;
+        zr = nr;
+        zi = ni;
+      }
+      const E* krow = kb + (int64_t)l * k_rs;
+      for (int j = 0; j < kn_len; ++j) {
+        float kv = fa_to_float(krow[j]);
+#pragma unroll
+        for (int g = 0; g < kGMax; ++g)
+          if (g < G) sc[g] = fmaf(kv, s_qn[g * D + j], sc[g]);
+      }
+    }
+    // ---- phase 2: online softmax over the tile --------------------------
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) {
+      float v = fa_wave_max(ok ? sc[g] : -INFINITY);
+      if (lane == 0) s_red[w * kGMax + g] = v;
+    }
+    __syncthreads();
+    float alpha[kGMax];
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) {
+      float tm = fmaxf(fmaxf(s_red[g], s_red[kGMax + g]), fmaxf(s_red[2 * kGMax + g], s_red[3 * kGMax + g]));
+      float mn = fmaxf(m_run[g], tm);
+      alpha[g] = (m_run[g] == -INFINITY) ? 0.f : exp2f(m_run[g] - mn);
+      m_run[g] = mn;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) {
+      float p = (ok && g < G) ? exp2f(sc[g] - m_run[g]) : 0.f;
+      if (g < G) s_p[g * kTile + tid] = p;
+      float v = fa_wave_sum(p);
+      if (lane == 0) s_red[w * kGMax + g] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      d_run[g] = d_run[g] * alpha[g] + (s_red[g] + s_red[kGMax + g] + s_red[2 * kGMax + g] + s_red[3 * kGMax + g]);
+    // ---- phase 3: g[n] += sum_t p[t] e^{i theta n (l0 + t)}, thread = frequency
+#pragma unroll
+    for (int i = 0; i < kFreqIters; ++i) {
+      const int n = tid + 256 * i;
+      if (n < N) {
+#pragma unroll
+        for (int g = 0; g < kGMax; ++g) {
+          gc[i][g] *= alpha[g];
+          gs[i][g] *= alpha[g];
+        }
+        float sr, si, zr, zi;
+        fa_sincos_phase(n, 1, T, &si, &sr);
+        for (int tt = 0; tt < t_len; ++tt) {
+          if ((tt & 63) == 0) fa_sincos_phase(n, l0 + tt, T, &zi, &zr);
+#pragma unroll
+          for (int g = 0; g < kGMax; ++g)
+            if (g < G) {
+              float p = s_p[g * kTile + tt];
+              gc[i][g] = fmaf(p, zr, gc[i][g]);
+              gs[i][g] = fmaf(p, zi, gs[i][g]);
+            }
+          float nr = zr * sr - zi * si;
+          float ni = zr * si + zi * sr;
+          zr = nr;
+          zi = ni;
+        }
+      }
+    }
+    // ---- phase 4: stored V dims, thread = (dim, tile half) ----------------
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) on[g] *= alpha[g];
+    if (dim < vn_len) {
+      for (int tt = half; tt < t_len; tt += 2) {
+        float vv = fa_to_float(vb[(int64_t)(l0 + tt) * v_rs + dim]);
+#pragma unroll
+        for (int g = 0; g < kGMax; ++g)
+          if (g < G) on[g] = fmaf(s_p[g * kTile + tt], vv, on[g]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- write the split's partials ---------------------------------------
+  if (half == 1 && dim < vn_len) {
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) s_o[g * D + dim] = on[g];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) {
+    if (g >= G) continue;
+    const int64_t r = ((int64_t)b * Hq + h * G + g) * n_split + split;
+    if (half == 0 && dim < vn_len) pon[r * D + dim] = on[g] + s_o[g * D + dim];
+#pragma unroll
+    for (int i = 0; i < kFreqIters; ++i) {
+      const int n = tid + 256 * i;
+      if (n < N) {
+        pg[r * 2 * N + n] = gc[i][g];
+        pg[r * 2 * N + N + n] = gs[i][g];
+      }
+    }
+    if (tid == 0) {
+      pm[r] = m_run[g];
+      pd[r] = d_run[g];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// merge: one block per (b, hq)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void decode_merge_kernel(
+    const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
+    const float* __restrict__ md_m, const float* __restrict__ md_d, const float* __restrict__ md_g,
+    const float* __restrict__ md_on, int n_mid_split, const float* __restrict__ v_mc,
+    const float* __restrict__ avg_u, const float* __restrict__ avg_d, const float* __restrict__ scale,
+    const int32_t* __restrict__ vc_list, const int32_t* __restrict__ vc_h, const int32_t* __restrict__ vn_list,
+    const int32_t* __restrict__ vn_h, float* __restrict__ out, int Hq, int Hkv, int D, int N, int Cv) {
+  extern __shared__ float smem[];
+  float* s_g = smem;              // [2N]
+  float* s_o = s_g + 2 * N;       // [D]
+  float* s_part = s_o + D;        // [2][128]
+  float* s_w = s_part + 256;      // [n_il_split + n_mid_split]
+  const int tid = threadIdx.x;
+  const int hq = blockIdx.x, b = blockIdx.y;
+  const int G = Hq / Hkv, h = hq / G;
+  const int64_t r = (int64_t)b * Hq + hq;
+  const int n_all = n_il_split + n_mid_split;
+
+  float mstar = -INFINITY;
+  for (int s = 0; s < n_il_split; ++s) mstar = fmaxf(mstar, il_m[r * n_il_split + s]);
+  for (int s = 0; s < n_mid_split; ++s) mstar = fmaxf(mstar, md_m[r * n_mid_split + s]);
+  for (int s = tid; s < n_all; s += 256) {
+    float m = s < n_il_split ? il_m[r * n_il_split + s] : md_m[r * n_mid_split + (s - n_il_split)];
+    s_w[s] = (m == -INFINITY) ? 0.f : exp2f(m - mstar);
+  }
+  for (int d = tid; d < D; d += 256) s_o[d] = 0.f;
+  __syncthreads();
+  float dsum = 0.f, pmid = 0.f;
+  for (int s = 0; s < n_il_split; ++s) dsum += s_w[s] * il_d[r * n_il_split + s];
+  for (int s = 0; s < n_mid_split; ++s) pmid += s_w[n_il_split + s] * md_d[r * n_mid_split + s];
+  dsum += pmid;
+
+  for (int n = tid; n < 2 * N; n += 256) {
+    float a = 0.f;
+    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[n_il_split + s], md_g[(r * n_mid_split + s) * 2 * N + n], a);
+    s_g[n] = a;
+  }
+  __syncthreads();
+
+  // stored dims of V
+  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
+  for (int j = tid; j < vn_len; j += 256) {
+    float a = 0.f;
+    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[n_il_split + s], md_on[(r * n_mid_split + s) * D + j], a);
+    s_o[vn_list[vn0 + j] - h * D] = a;
+  }
+  // compressed dims of V: g . V_coef
+  const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
+  {
+    const int j = tid % 128, part = tid / 128;
+    float a = 0.f;
+    if (j < vc_len && n_mid_split > 0) {
+      const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + j;
+      for (int n = part; n < 2 * N; n += 2) a = fmaf(s_g[n], vp[(int64_t)n * Cv], a);
+    }
+    s_part[part * 128 + j] = a;
+  }
+  __syncthreads();
+  for (int j = tid; j < vc_len; j += 256) {
+    float a = (s_part[j] + s_part[128 + j]) / (float)N;
+    int64_t o = (int64_t)b * Cv + vc0 + j;
+    float v = n_mid_split > 0 ? scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid : 0.f;
+    s_o[vc_list[vc0 + j] - h * D] = v;
+  }
+  __syncthreads();
+  for (int d = tid; d < D; d += 256) {
+    float a = s_o[d];
+    for (int s = 0; s < n_il_split; ++s) a = fmaf(s_w[s], il_o[(r * n_il_split + s) * D + d], a);
+    out[r * D + d] = a / dsum;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct Plan {
+  int n_il_split, n_mid_split, tiles_per_split;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, total;
+};
+
+Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m) {
+  Plan p{};
+  p.n_il_split = fa_cdiv(n_il, kTile);
+  const int tiles = fa_cdiv(L_m, kTile);
+  int want = fa_cdiv(1024, (int64_t)B * Hkv);
+  if (want < 1) want = 1;
+  int ns = tiles < want ? tiles : want;
+  if (ns > 64) ns = 64;
+  p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
+  p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+  const size_t rows = (size_t)B * Hq;
+  size_t o = 0;
+  auto take = [&](size_t n_float) {
+    size_t at = o;
+    o += fa_align_up(n_float * sizeof(float), 256);
+    return at;
+  };
+  p.off_W = take(rows * 2 * N);
+  p.off_c0 = take(rows);
+  p.off_ilm = take(rows * p.n_il_split);
+  p.off_ild = take(rows * p.n_il_split);
+  p.off_ilo = take(rows * p.n_il_split * D);
+  p.off_mm = take(rows * p.n_mid_split);
+  p.off_md = take(rows * p.n_mid_split);
+  p.off_mg = take(rows * p.n_mid_split * 2 * N);
+  p.off_mon = take(rows * p.n_mid_split * D);
+  p.total = o;
+  return p;
+}
+
+template <typename E>
+int launch_generic(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream_t st) {
+  char* ws = (char*)a.workspace;
+  float* W = (float*)(ws + p.off_W);
+  float* c0 = (float*)(ws + p.off_c0);
+  float* ilm = (float*)(ws + p.off_ilm);
+  float* ild = (float*)(ws + p.off_ild);
+  float* ilo = (float*)(ws + p.off_ilo);
+  float* mm = (float*)(ws + p.off_mm);
+  float* md = (float*)(ws + p.off_md);
+  float* mg = (float*)(ws + p.off_mg);
+  float* mon = (float*)(ws + p.off_mon);
+  const int G = a.Hq / a.Hkv;
+  const float sm_log2e = sm_scale * kLog2e;
+  if (p.n_mid_split > 0) {
+    const int rows_per_block = 64;
+    decode_prep_kernel<E><<<dim3(fa_cdiv(2 * a.N, rows_per_block), a.Hkv, a.B), 256, 0, st>>>(
+        (const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0, a.Hq, a.Hkv, a.D,
+        a.N, a.Ck, sm_log2e, rows_per_block);
+    size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_mid_kernel<E>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
+    }
+    decode_mid_kernel<E><<<dim3(p.n_mid_split, a.Hkv, a.B), 256, lds, st>>>(
+        (const E*)a.q, (const E*)a.k_mn, a.k_mn_batch_stride, a.k_mn_row_stride, (const E*)a.v_mn,
+        a.v_mn_batch_stride, a.v_mn_row_stride, W, c0, a.kn_list, a.kn_h_list, a.vn_h_list, mm, md, mg, mon, a.Hq,
+        a.Hkv, a.D, a.N, a.L_m, a.T, p.n_mid_split, p.tiles_per_split, sm_log2e);
+  }
+  if (p.n_il_split > 0) {
+    Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
+    Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
+    size_t lds = (2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
+    decode_il_kernel<E><<<dim3(p.n_il_split, a.Hkv, a.B), 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq,
+                                                                          a.Hkv, a.D, p.n_il_split, sm_log2e);
+  }
+  size_t lds = ((size_t)2 * a.N + a.D + 256 + p.n_il_split + p.n_mid_split) * sizeof(float);
+  decode_merge_kernel<<<dim3(a.Hq, a.B), 256, lds, st>>>(ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split,
+                                                         a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v, a.vc_list,
+                                                         a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D,
+                                                         a.N, a.Cv);
+  return fa_check_launch("fa_decode_attn");
+}
+
+}  // namespace
+
+extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || N < 0 || il_rows_total < 0 || L_m < 0) return 0;
+  return make_plan(B, Hq, Hkv, D, N > 0 ? N : 1, il_rows_total, L_m).total;
+}
+
+extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
+  FA_REQUIRE(a, FA_ERR_NULL_POINTER, "fa_decode_attn: null argument block");
+  FA_REQUIRE(a->q_len == 1, FA_ERR_BAD_SHAPE, "fa_decode_attn: q_len = %d, decode needs exactly one query row", a->q_len);
+  FA_REQUIRE(a->B > 0 && a->Hq > 0 && a->Hkv > 0 && a->D > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: bad B/Hq/Hkv/D");
+  FA_REQUIRE(a->Hq % a->Hkv == 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: Hq %d not a multiple of Hkv %d", a->Hq, a->Hkv);
+  FA_REQUIRE(a->il_rows[0] >= 0 && a->il_rows[1] >= 0 && a->L_m >= 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: negative row count");
+  FA_REQUIRE(a->il_rows[0] + a->il_rows[1] + a->L_m > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: no keys");
+  FA_REQUIRE(a->q && a->out, FA_ERR_NULL_POINTER, "fa_decode_attn: q/out null");
+  FA_REQUIRE(a->dtype == FA_BF16 || a->dtype == FA_FP16 || a->dtype == FA_FP32, FA_ERR_BAD_DTYPE, "fa_decode_attn: dtype %d", a->dtype);
+  for (int i = 0; i < 2; ++i)
+    FA_REQUIRE(a->il_rows[i] == 0 || (a->k_il[i] && a->v_il[i]), FA_ERR_NULL_POINTER, "fa_decode_attn: il segment %d null", i);
+  const int G = a->Hq / a->Hkv;
+  FA_REQUIRE(G <= kGMax, FA_ERR_UNSUPPORTED, "fa_decode_attn: %d query heads per KV head (max %d)", G, kGMax);
+  FA_REQUIRE(a->D <= 128, FA_ERR_UNSUPPORTED, "fa_decode_attn: head_dim %d (max 128)", a->D);
+  if (a->L_m > 0) {
+    FA_REQUIRE(a->N > 0 && a->T > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: N=%d T=%d", a->N, a->T);
+    FA_REQUIRE(a->N <= 256 * kFreqIters, FA_ERR_UNSUPPORTED, "fa_decode_attn: N=%d (max %d)", a->N, 256 * kFreqIters);
+    FA_REQUIRE(a->Ck >= 0 && a->Cv >= 0 && a->Cnk >= 0 && a->Cnv >= 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: negative dim count");
+    FA_REQUIRE(a->Ck + a->Cnk == a->Hkv * a->D && a->Cv + a->Cnv == a->Hkv * a->D, FA_ERR_BAD_SHAPE,
+               "fa_decode_attn: compressed + stored dims must equal Hkv*D");
+    FA_REQUIRE(a->kc_h_list && a->kn_h_list && a->vc_h_list && a->vn_h_list, FA_ERR_NULL_POINTER,
+               "fa_decode_attn: per-head offset list null");
+    FA_REQUIRE((a->Ck == 0 || a->kc_list) && (a->Cnk == 0 || a->kn_list) && (a->Cv == 0 || a->vc_list) &&
+                   (a->Cnv == 0 || a->vn_list), FA_ERR_NULL_POINTER, "fa_decode_attn: index list null");
+    FA_REQUIRE((a->Ck == 0 || (a->k_mc && a->avg_k_u && a->avg_k_d && a->scale_k)) &&
+                   (a->Cv == 0 || (a->v_mc && a->avg_v_u && a->avg_v_d && a->scale_v)),
+               FA_ERR_NULL_POINTER, "fa_decode_attn: coefficient/statistics pointer null");
+    FA_REQUIRE((a->Cnk == 0 || a->k_mn) && (a->Cnv == 0 || a->v_mn), FA_ERR_NULL_POINTER, "fa_decode_attn: k_mn/v_mn null");
+  }
+  const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m);
+  FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
+             a->workspace_bytes, p.total);
+  FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");
+  const float sm = a->sm_scale > 0.f ? a->sm_scale : 1.0f / sqrtf((float)a->D);
+  hipStream_t st = fa_hip_stream(stream);
+  switch (a->dtype) {
+    case FA_BF16: return launch_generic<bf16_t>(*a, p, sm, st);
+    case FA_FP16: return launch_generic<f16_t>(*a, p, sm, st);
+    default: return launch_generic<float>(*a, p, sm, st);
+  }
+}

@@ -1,0 +1,275 @@
+"""Operator-level mirror of the reference's kernel entry points, backed by the HIP library.
+
+Same names, argument meaning and error behaviour as
+``fourier_attn_triton/fourier_triton_valid4_v2.py``:
+
+* ``mat_fourier_triton``            (lines 81-102)
+* ``mat_avg_std_triton``            (lines 433-461)
+* ``mat_fourier_avg_std_triton``    (lines 285-326)
+* ``triton_fourier_attn``           (lines 684-779)  - also exported as ``fourier_attn``
+* ``mat_fourier_inv_torch``         (lines 782-791)  - as ``mat_fourier_inv``
+* ``MultiDimHiPPO2``                (lines 840-865)
+
+The names keep the reference's ``_triton`` suffix so call sites need no edit; nothing
+here uses Triton.  Tensors must live on the GPU; PyTorch only provides the memory and
+the current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import FA_BF16, FA_FP16, FA_FP32, DecodeArgs, check
+
+_DTYPE_CODE = {torch.bfloat16: FA_BF16, torch.float16: FA_FP16, torch.float32: FA_FP32}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor: the HIP kernels are the only implementation")
+
+
+_workspaces: Dict[Tuple[int, str], torch.Tensor] = {}
+
+
+def workspace(device: torch.device, nbytes: int, tag: str = "default") -> torch.Tensor:
+    """A per-device scratch buffer that only grows.  Work that shares a tag must be issued on
+    one stream (kernels of consecutive calls then run in order and may reuse it)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def as_i32(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.int32 else t.to(torch.int32)
+
+
+# --------------------------------------------------------------------------- K1
+def mat_fourier(a: torch.Tensor, N: int, T: int, K_start: int = 0, cols: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None, accumulate: bool = False, K: Optional[int] = None) -> torch.Tensor:
+    """``c[b, n, m] (+)= sum_k cos(2 pi (k + K_start) n / T) a[b, k, cols[m]]`` and the sin rows.
+
+    ``a (B, K, width)`` may be a strided view as long as its last dim is contiguous; ``cols``
+    (int32, GPU) selects columns; ``K`` limits the rows read."""
+    _require_gpu(a, "a")
+    assert a.dim() == 3 and a.stride(2) == 1, "a must be (B, K, M) with a contiguous last dim"
+    B, rows, width = a.shape
+    K = rows if K is None else min(int(K), rows)
+    Mc = width if cols is None else cols.numel()
+    if out is None:
+        assert not accumulate
+        out = torch.empty((B, 2 * N, Mc), device=a.device, dtype=torch.float32)
+    assert out.is_contiguous() and out.dtype == torch.float32 and tuple(out.shape) == (B, 2 * N, Mc)
+    if Mc == 0 or B == 0:
+        return out
+    lib = _lib.load()
+    check(lib.fa_mat_fourier(a.data_ptr(), dtype_code(a.dtype), a.stride(0), a.stride(1), _ptr(cols), out.data_ptr(), B, K,
+                             Mc, N, int(T), int(K_start), int(accumulate), _stream(a.device)))
+    return out
+
+
+def mat_fourier_triton(a: torch.Tensor, N: int, T: int, K_start: int = 0) -> torch.Tensor:
+    assert a.is_contiguous(), "Matrix A must be contiguous"  # TRI:82
+    return mat_fourier(a, N, T, K_start)
+
+
+# --------------------------------------------------------------------------- K2
+def mat_avg_std(a: torch.Tensor, cols: Optional[torch.Tensor] = None, round_dtype: Optional[torch.dtype] = None):
+    """fp32 ``(avg, max_dev)`` of the columns of ``a (B, K, width)``, each rounded through
+    ``round_dtype`` when given."""
+    _require_gpu(a, "a")
+    assert a.dim() == 3 and a.stride(2) == 1
+    B, K, width = a.shape
+    Mc = width if cols is None else cols.numel()
+    avg = torch.empty((B, Mc), device=a.device, dtype=torch.float32)
+    dev = torch.empty((B, Mc), device=a.device, dtype=torch.float32)
+    if Mc == 0 or B == 0:
+        return avg, dev
+    lib = _lib.load()
+    nbytes = lib.fa_stats_workspace_bytes(B, Mc, K)
+    ws = workspace(a.device, nbytes)
+    rd = FA_FP32 if round_dtype is None else dtype_code(round_dtype)
+    check(lib.fa_mat_avg_std(a.data_ptr(), dtype_code(a.dtype), a.stride(0), a.stride(1), _ptr(cols), avg.data_ptr(),
+                             dev.data_ptr(), B, K, Mc, rd, ws.data_ptr(), ws.numel(), _stream(a.device)))
+    return avg, dev
+
+
+def mat_avg_std_triton(a: torch.Tensor):
+    assert a.is_cuda and a.is_contiguous(), "Input tensor must be a contiguous CUDA tensor"  # TRI:438
+    assert a.dim() == 3, "Input tensor must be 3-dimensional"
+    avg, dev = mat_avg_std(a, round_dtype=a.dtype)
+    return avg.to(a.dtype), dev.to(a.dtype)  # TRI:461
+
+
+# --------------------------------------------------------------------------- K3
+def mat_fourier_avg_std(c: torch.Tensor, K: int, T: int, round_dtype: Optional[torch.dtype] = torch.float16):
+    _require_gpu(c, "c")
+    assert c.is_contiguous() and c.dtype == torch.float32 and c.dim() == 3
+    B, N2, Mc = c.shape
+    avg = torch.empty((B, Mc), device=c.device, dtype=torch.float32)
+    dev = torch.empty((B, Mc), device=c.device, dtype=torch.float32)
+    if Mc == 0 or B == 0:
+        return avg, dev
+    lib = _lib.load()
+    nbytes = lib.fa_stats_workspace_bytes(B, Mc, int(K))
+    ws = workspace(c.device, nbytes)
+    rd = FA_FP32 if round_dtype is None else dtype_code(round_dtype)
+    check(lib.fa_mat_fourier_avg_std(c.data_ptr(), avg.data_ptr(), dev.data_ptr(), B, N2 // 2, Mc, int(K), int(T), rd,
+                                     ws.data_ptr(), ws.numel(), _stream(c.device)))
+    return avg, dev
+
+
+def mat_fourier_avg_std_triton(c: torch.Tensor, K: int, T: int):
+    assert c.is_contiguous(), "Matrix C must be contiguous"  # TRI:286
+    avg, dev = mat_fourier_avg_std(c.float() if c.dtype != torch.float32 else c, K, T, torch.float16)
+    return avg.to(torch.float16), dev.to(torch.float16)  # TRI:326
+
+
+# ------------------------------------------------------------------ reconstruction
+def mat_fourier_inv(c: torch.Tensor, K: int, T: int, avg_u=None, avg_d=None, scale=None) -> torch.Tensor:
+    """``(B, K, Mc)`` fp32 reconstruction (TRI:782-791), optionally through the affine statistics."""
+    _require_gpu(c, "c")
+    assert c.is_contiguous() and c.dtype == torch.float32 and c.dim() == 3
+    B, N2, Mc = c.shape
+    r = torch.empty((B, int(K), Mc), device=c.device, dtype=torch.float32)
+    if r.numel() == 0:
+        return r
+    f = lambda t: None if t is None else t.float().contiguous()
+    au, ad, sc = f(avg_u), f(avg_d), f(scale)
+    check(_lib.load().fa_reconstruct(c.data_ptr(), _ptr(au), _ptr(ad), _ptr(sc), r.data_ptr(), B, N2 // 2, Mc, int(K), int(T),
+                                     _stream(c.device)))
+    return r
+
+
+# -------------------------------------------------------------------- rank-1 update
+def coeff_update_(c: torch.Tensor, row: torch.Tensor, cols: Optional[torch.Tensor], p: int, T: int) -> torch.Tensor:
+    """In place ``c[b, n, j] += cos(2 pi p n / T) row[b, cols[j]]`` (+ sin rows).  ``row (B, width)``
+    may be a strided view with a contiguous last dim."""
+    _require_gpu(c, "c")
+    assert c.is_contiguous() and c.dtype == torch.float32 and c.dim() == 3
+    assert row.dim() == 2 and row.stride(1) == 1
+    B, N2, Mc = c.shape
+    if Mc == 0 or B == 0:
+        return c
+    check(_lib.load().fa_coeff_update(c.data_ptr(), row.data_ptr(), dtype_code(row.dtype), row.stride(0), _ptr(cols), B,
+                                      N2 // 2, Mc, int(p), int(T), _stream(c.device)))
+    return c
+
+
+class MultiDimHiPPO2(torch.nn.Module):
+    """Same call contract as the reference class (TRI:840-865): without ``slice_input`` the
+    whole ``base_input (B, L, C)`` is projected (period and length ``int(1/dt)``: longer inputs
+    are cut, shorter ones behave as zero-padded); with ``slice_input (B, 1, C)`` the result is
+    ``base_input + transform(slice_input)`` entering at phase ``token_num``."""
+
+    def __init__(self, N, input_dim, method="legt", dt=1.0, T=1.0, discretization="bilinear", scale=False, c=0.0):
+        super().__init__()
+        self.method, self.N, self.input_dim, self.dt, self.T, self.c = method, N, input_dim, dt, T, c
+        self.base_N = N // input_dim
+
+    def forward(self, base_input, token_num, slice_input=None, fast=False):
+        base_N = self.N // self.input_dim // 2
+        period = int(1 / self.dt)
+        if slice_input is not None:
+            out = base_input.clone()
+            return coeff_update_(out, slice_input[:, 0, :], None, token_num, period)
+        return mat_fourier(base_input, base_N, period, 0, K=period)
+
+
+# ------------------------------------------------------------------ decode attention
+def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
+                    T, sm_scale=-1.0, out=None):
+    """Thin call into ``fa_decode_attn``.
+
+    ``il_segments``: up to two ``(k, v)`` pairs of ``(B, rows, Hkv*D)`` views (last dim contiguous).
+    ``stats_*``: ``(avg_u, avg_d, scale)`` fp32 ``(B, C)``.  ``lists``: the eight int32 tensors
+    ``kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h`` (``*_h`` with the leading 0)."""
+    _require_gpu(q, "q")
+    B, q_len, feat = q.shape
+    D = feat // num_head_q
+    a = DecodeArgs()
+    assert q.is_contiguous()
+    a.q = q.data_ptr()
+    total_il = 0
+    for i in range(2):
+        if i < len(il_segments) and il_segments[i] is not None and il_segments[i][0].shape[1] > 0:
+            k, v = il_segments[i]
+            assert k.stride(2) == 1 and v.stride(2) == 1 and k.stride() == v.stride() and k.shape == v.shape
+            assert k.dtype == q.dtype and v.dtype == q.dtype
+            a.k_il[i], a.v_il[i] = k.data_ptr(), v.data_ptr()
+            a.il_rows[i], a.il_batch_stride[i], a.il_row_stride[i] = k.shape[1], k.stride(0), k.stride(1)
+            total_il += k.shape[1]
+    kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h = lists
+    a.Ck, a.Cnk, a.Cv, a.Cnv = kc.numel(), kn.numel(), vc.numel(), vn.numel()
+    N = 0
+    if seq_len_m > 0:
+        N = (k_mc.shape[1] if a.Ck else v_mc.shape[1]) // 2
+        for t in (k_mc, v_mc):
+            assert t.dtype == torch.float32 and t.is_contiguous()
+        for t in (k_mn, v_mn):
+            assert t.stride(2) == 1 and t.dtype == q.dtype
+        a.k_mc, a.v_mc = _ptr(k_mc), _ptr(v_mc)
+        a.k_mn, a.v_mn = _ptr(k_mn), _ptr(v_mn)
+        a.k_mn_batch_stride, a.k_mn_row_stride = k_mn.stride(0), k_mn.stride(1)
+        a.v_mn_batch_stride, a.v_mn_row_stride = v_mn.stride(0), v_mn.stride(1)
+        a.avg_k_u, a.avg_k_d, a.scale_k = (_ptr(t) for t in stats_k)
+        a.avg_v_u, a.avg_v_d, a.scale_v = (_ptr(t) for t in stats_v)
+        for t in (*stats_k, *stats_v):
+            assert t.dtype == torch.float32 and t.is_contiguous()
+    a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()
+    a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list = vc.data_ptr(), vc_h.data_ptr(), vn.data_ptr(), vn_h.data_ptr()
+    if out is None:
+        out = torch.empty((B, num_head_q, 1, D), device=q.device, dtype=torch.float32)
+    a.out = out.data_ptr()
+    a.B, a.Hq, a.Hkv, a.D = B, num_head_q, num_head_kv, D
+    a.q_len, a.N, a.L_m, a.T = q_len, N, int(seq_len_m), int(T)
+    a.sm_scale = float(sm_scale)
+    a.dtype = dtype_code(q.dtype)
+    lib = _lib.load()
+    nbytes = lib.fa_decode_attn_workspace_bytes(B, num_head_q, num_head_kv, D, N, total_il, int(seq_len_m))
+    ws = workspace(q.device, nbytes, "decode")
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    check(lib.fa_decode_attn(ctypes.byref(a), _stream(q.device)))
+    return out
+
+
+def triton_fourier_attn(q, k_il, v_il, k_mc, v_mc, k_mn, v_mn,
+                        avg_k_u, avg_k_d, scale_k, avg_v_u, avg_v_d, scale_v,
+                        kc_list, kc_h_list, kn_list, kn_h_list,
+                        vc_list, vc_h_list, vn_list, vn_h_list,
+                        num_head_q, num_head_kv, seq_len_m, T, sm_scale=-1):
+    """Drop-in for the reference function of the same name (TRI:684-779): returns
+    ``(B, Hq, 1, D)`` float32."""
+    batch_size, seq_len_q, feature_dim = q.shape
+    assert seq_len_q == 1, f"{q.shape = }"  # TRI:692
+    f32 = lambda t: t.float().contiguous()
+    lists = tuple(as_i32(t) for t in (kc_list, kc_h_list, kn_list, kn_h_list, vc_list, vc_h_list, vn_list, vn_h_list))
+    k_mc = k_mc if k_mc.dtype == torch.float32 else k_mc.float()
+    v_mc = v_mc if v_mc.dtype == torch.float32 else v_mc.float()
+    return decode_attn_raw(q.contiguous(), [(k_il, v_il)], k_mc.contiguous(), v_mc.contiguous(), k_mn, v_mn,
+                           (f32(avg_k_u), f32(avg_k_d), f32(scale_k)), (f32(avg_v_u), f32(avg_v_d), f32(scale_v)),
+                           lists, num_head_q, num_head_kv, seq_len_m, T, sm_scale)
+
+
+fourier_attn = triton_fourier_attn

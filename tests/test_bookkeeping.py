@@ -1,0 +1,150 @@
+"""Host logic without a GPU: the integer state machine against the CPU restatement of the
+reference cache (shapes and counters after every call), the period pair, and the C ABI's
+exports and argument validation (no kernel is launched)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from fourierattention_amd import _lib
+from fourierattention_amd.bookkeeping import Action, CacheBook, periods
+from fourierattention_amd.cache import ExtraConfig
+from fourierattention_amd import masks as pm
+from oracle import fourier_oracle as fo
+from oracle.cache_oracle import OracleCache
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_periods_match_oracle():
+    for mt in list(range(30, 3000, 7)) + [131072, 131072 + 512, 32768 + 128]:
+        assert periods(mt, 4, 20) == fo.periods(mt, 4, 20)
+    assert periods(131072, 4, 1024)[0::2] == (130044, 130043)
+
+
+TRACES = [
+    # I, W, M, max_new, max_pos, B, prompt, steps
+    (4, 16, 16, 10, 4096, 2, 103, 8),      # compressed, streaming
+    (4, 16, 16, 10, 4096, 2, 30, 12),      # short prompt: window only, forever
+    (4, 16, 16, 10, 113, 2, 120, 5),       # maxtokens clamped by max_position_embeddings
+    (4, 64, 8, 8, 4096, 1, 88, 4),         # short mid: append branch of a compressed layer
+    (4, 512, 256, 64, 131072, 1, 2048, 3),  # BASELINE config 1 geometry
+    (0, 8, 4, 4, 4096, 3, 40, 5),          # no sink tokens
+]
+
+
+@pytest.mark.parametrize("I,W,M,max_new,max_pos,B,prompt,steps", TRACES)
+def test_state_machine_trace_matches_reference_restatement(I, W, M, max_new, max_pos, B, prompt, steps):
+    Hkv, D, layers = 2, 8, 3
+    masks = pm.synthetic_masks(layers, Hkv, D, 3, 5, seed=1)
+    cfg = ExtraConfig(numinittokens=I, maxlocallen=W, maxmidstates=M, non_critical_dims_path=None, max_position_embeddings=max_pos,
+                      num_key_value_heads=Hkv, max_new_tokens=max_new)
+    cpu = OracleCache(cfg, masks=masks, model_dtype="fp32")
+    book = CacheBook(layers, I, W, M, max_new, max_pos)
+    r = np.random.default_rng(0)
+
+    def check(l, step):
+        lb = book.layers[l]
+        kc = cpu.key_cache[l]
+        assert (lb.n_init, lb.n_coef_rows, lb.n_mid, lb.n_local) == (
+            kc["k_init"].shape[1], kc["k_compressed"].shape[1], kc["k_uncompressed"].shape[1], kc["k_local"].shape[1])
+        assert lb.seq_length == cpu.get_seq_length(l)
+        assert lb.curr_tokennum == cpu.curr_tokennum[l]
+        assert book.seen_tokens == cpu._seen_tokens and book.maxtokens == cpu.maxtokens
+        assert (book.t_x, book.t_c) == (cpu._t_x(), cpu.t_c)
+
+    for l in range(layers):
+        k = r.standard_normal((B, Hkv, prompt, D))
+        kd, _ = cpu.update(k, k, l)
+        st = book.step(l, B, prompt)
+        assert st.action in (Action.PREFILL_COMPRESS, Action.PREFILL_LOCAL)
+        assert (st.action is Action.PREFILL_COMPRESS) == (cpu.key_cache[l]["k_compressed"].shape[1] > 0)
+        if st.action is Action.PREFILL_COMPRESS:
+            assert st.mid_rows == cpu.key_cache[l]["k_uncompressed"].shape[1] and st.fft_rows == min(st.mid_rows, cpu.t_c)
+        check(l, st)
+    for s in range(steps):
+        for l in range(layers):
+            k = r.standard_normal((B, Hkv, 1, D))
+            before = cpu.curr_tokennum[l]
+            kd, _ = cpu.update(k, k, l)
+            st = book.step(l, B, 1)
+            assert (st.action is Action.STREAM) == (kd["k_init"] is not None)
+            if st.action is Action.STREAM:
+                assert st.phase == before + 1 == cpu.curr_tokennum[l]
+                # phase runs one ahead of the row index of the evicted token
+                assert st.phase == book.layers[l].n_mid
+            check(l, st)
+
+
+def test_layer_zero_must_come_first_and_stream_needs_one_token():
+    book = CacheBook(2, 4, 16, 16, 10, 4096)
+    with pytest.raises(RuntimeError):
+        book.step(1, 1, 100)
+    book.step(0, 1, 100)
+    book.step(1, 1, 100)
+    with pytest.raises(ValueError):
+        book.step(0, 1, 2)
+
+
+def test_missing_layer_key_raises_value_error():
+    masks = pm.synthetic_masks(3, 2, 8, 3)
+    del masks["Layer_1"]
+    masks["Layer_7"] = masks["Layer_0"]
+    cfg = ExtraConfig(numinittokens=4, maxlocallen=16, maxmidstates=16, non_critical_dims_path=None, non_critical_dims=masks,
+                      max_position_embeddings=4096, num_key_value_heads=2, max_new_tokens=4)
+    with pytest.raises(ValueError):
+        OracleCache(cfg, masks=masks)
+    from fourierattention_amd import DynamicCache
+    with pytest.raises(ValueError):
+        DynamicCache(cfg, device="cpu")
+
+
+# ----------------------------------------------------------------- C ABI ------
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "fourier_attn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_functions()
+    assert len(declared) >= 10
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert set(declared) == set(_lib.EXPORTED), set(declared) ^ set(_lib.EXPORTED)
+    assert lib.fa_abi_version() >= 1
+    assert lib.fa_decode_args_size() == ctypes.sizeof(_lib.DecodeArgs)
+
+
+def test_argument_validation_returns_codes_without_a_gpu():
+    lib = _lib.load()
+    assert lib.fa_decode_attn(None, None) == -1
+    a = _lib.DecodeArgs()
+    a.q_len = 2
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -2 and b"q_len" in lib.fa_last_error_string()
+    a.q_len, a.B, a.Hq, a.Hkv, a.D = 1, 1, 6, 4, 64
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -2          # Hq not a multiple of Hkv
+    a.Hq, a.Hkv = 8, 2
+    a.il_rows[0] = 4
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -1          # q / out null
+    buf = ctypes.create_string_buffer(1 << 16)
+    p = ctypes.addressof(buf)
+    a.q = a.out = p
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -1          # il segment null
+    a.k_il[0] = a.v_il[0] = p
+    a.dtype = 9
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -3
+    a.dtype = 0
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -4          # workspace missing
+    a.Hq, a.Hkv = 64, 2
+    assert lib.fa_decode_attn(ctypes.byref(a), None) == -5          # 32 query heads per KV head
+    assert lib.fa_mat_fourier(None, 0, 0, 0, None, None, 1, 1, 1, 1, 1, 0, 0, None) == -1
+    assert lib.fa_mat_fourier(p, 0, 0, 0, None, p, 1, 1, 1, 0, 1, 0, 0, None) == -2
+    assert lib.fa_mat_fourier(p, 7, 0, 0, None, p, 1, 1, 1, 1, 1, 0, 0, None) == -3
+    assert lib.fa_mat_avg_std(p, 0, 0, 0, None, p, p, 1, 4, 4, 2, None, 0, None) == -4
+    assert lib.fa_coeff_update(p, None, 0, 0, None, 1, 1, 1, 0, 1, None) == -1
+    assert lib.fa_stats_workspace_bytes(2, 10, 1000) == 3 * 2 * 4 * 10 * 4
+    assert lib.fa_decode_attn_workspace_bytes(8, 32, 8, 128, 512, 1028, 31740) > 0

@@ -1,0 +1,169 @@
+"""The cache object end to end on the GPU against the CPU restatement of the reference's
+state machine: part shapes / counters / stored rows bit-exact, floating point within the
+stated tolerances."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fourier_oracle as fo
+from oracle.cache_oracle import OracleCache
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(masks, **kw):
+    from fourierattention_amd import ExtraConfig
+    base = dict(numinittokens=4, maxlocallen=16, maxmidstates=16, non_critical_dims=masks, non_critical_dims_path=None,
+                max_position_embeddings=4096, num_key_value_heads=2, max_new_tokens=10, model_type="llama")
+    base.update(kw)
+    return ExtraConfig(**base)
+
+
+def _masks(layers, Hkv, D, kcounts, vcounts, seed=0):
+    from fourierattention_amd import masks as pm
+    rng = np.random.default_rng(seed)
+    out = {}
+    for i in range(layers):
+        kc, _, _, _ = H.ragged_mask(rng, Hkv, D, kcounts)
+        vc, _, _, _ = H.ragged_mask(rng, Hkv, D, vcounts)
+        out[f"Layer_{i}"] = pm.layer_from_compressed(kc.tolist(), vc.tolist(), Hkv, D)
+    return out
+
+
+def _compare_parts(kp, kw, tag, dtype):
+    for part in ("init", "compressed", "uncompressed", "local"):
+        g, w = kp[f"{tag}_{part}"], kw[f"{tag}_{part}"]
+        assert tuple(g.shape) == tuple(w.shape), (tag, part, g.shape, w.shape)
+        if part == "compressed":
+            assert g.dtype == torch.float32
+            if w.size:
+                err = np.linalg.norm(g.cpu().numpy() - w) / np.linalg.norm(w)
+                assert err <= 1e-3, err       # stated bound; fp32 accumulation gives ~1e-6
+                assert err <= 2e-5, err
+        else:
+            assert g.dtype == dtype
+            np.testing.assert_array_equal(g.float().cpu().numpy(), w.astype(np.float32))  # stored rows are copies
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("prompt,max_new,max_pos,expect_T", [
+    (103, 10, 4096, (93, 92)),      # int(1/dt) = T_x - 1, mid (83 rows) shorter than the period
+    (120, 10, 113, (93, 92)),       # maxtokens clamped: mid (100 rows) longer than T_c -> tail dropped by the transform
+    (110, 20, 4096, (110, 110)),
+])
+def test_cache_prefill_and_streaming(dtype, prompt, max_new, max_pos, expect_T):
+    from fourierattention_amd import DynamicCache, CacheParts
+    B, Hq, Hkv, D, layers, steps = 2, 8, 2, 64, 2, 6
+    masks = _masks(layers, Hkv, D, [40, 17], [64, 0])
+    cfg = _cfg(masks, max_new_tokens=max_new, max_position_embeddings=max_pos)
+    gpu = DynamicCache(cfg)
+    cpu = OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
+    r = np.random.default_rng(11)
+    k0 = H.to_dtype_np(r.standard_normal((layers, B, Hkv, prompt, D)), dtype)
+    v0 = H.to_dtype_np(r.standard_normal((layers, B, Hkv, prompt, D)) * 1.5 + 0.2, dtype)
+    for l in range(layers):
+        kp, vp = gpu.update(H.to_gpu(k0[l], dtype), H.to_gpu(v0[l], dtype), l)
+        kw, vw = cpu.update(k0[l], v0[l], l)
+        assert kp["k_init"] is None and kp["k_compressed"] is None and kp["k_uncompressed"] is None
+        assert tuple(kp["k_local"].shape) == tuple(kw["k_local"].shape) == (B, prompt, Hkv * D)
+    assert (gpu._book.t_x, gpu._book.t_c) == (cpu._t_x(), cpu.t_c) == expect_T
+    assert gpu.maxtokens == cpu.maxtokens and gpu._seen_tokens == cpu._seen_tokens == prompt
+    assert len(gpu) == len(cpu) == layers and gpu.get_seq_length() == cpu.get_seq_length() == prompt
+    assert gpu.curr_tokennum == cpu.curr_tokennum
+    for l in range(layers):
+        _compare_parts(gpu.key_cache[l], cpu.key_cache[l], "k", dtype)
+        _compare_parts(gpu.value_cache[l], cpu.value_cache[l], "v", dtype)
+        for name, tol in (("k_scale", 4e-3), ("k_layer_average", 1e-2), ("kd_layer_average", 2e-3),
+                          ("v_scale", 4e-3), ("v_layer_average", 1e-2), ("vd_layer_average", 2e-3)):
+            g, w = getattr(gpu, name)[l], getattr(cpu, name)[l]
+            assert tuple(g.shape) == tuple(w.shape)
+            np.testing.assert_allclose(g.float().cpu().numpy(), w, rtol=tol, atol=tol)  # <= one ulp of bf16 / fp16
+        want_scale_dtype = torch.float16 if dtype == torch.float16 else torch.float32
+        assert gpu.k_scale[l].dtype == want_scale_dtype and gpu.kd_layer_average[l].dtype == torch.float16
+        assert gpu.k_layer_average[l].dtype == dtype
+    # decode steps
+    for s in range(steps):
+        for l in range(layers):
+            kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+            vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+            q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)), dtype)
+            kp, vp = gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), l)
+            kw, vw = cpu.update(kn, vn, l)
+            assert isinstance(kp, CacheParts)
+            _compare_parts(kp, kw, "k", dtype)
+            _compare_parts(vp, vw, "v", dtype)
+            assert gpu.curr_tokennum == cpu.curr_tokennum
+            assert gpu.get_seq_length(l) == cpu.get_seq_length(l) == prompt + s + 1
+            # attention on identical state: feed the oracle the GPU's statistics so that only the
+            # attention arithmetic is compared (the statistics were compared above)
+            cpu_stats = {n: getattr(cpu, n)[l] for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average")}
+            for n in cpu_stats:
+                getattr(cpu, n)[l] = getattr(gpu, n)[l].float().cpu().numpy()
+            want = cpu.attend(q, kw, vw, l, Hq, Hkv)
+            for n in cpu_stats:
+                getattr(cpu, n)[l] = cpu_stats[n]
+            got = gpu.decode_attention(H.to_gpu(q, dtype), l, Hq, Hkv)
+            err = np.abs(got.cpu().numpy() - want).max()
+            assert err <= 2e-2 and err <= 1e-3, err
+        assert gpu._seen_tokens == cpu._seen_tokens == prompt + s + 1
+
+
+def test_short_prompt_stays_in_window_and_matches_exact_attention():
+    from fourierattention_amd import DynamicCache, fourier_attention
+    B, Hq, Hkv, D = 2, 8, 2, 64
+    dtype = torch.bfloat16
+    masks = _masks(1, Hkv, D, [32, 32], [32, 32])
+    cfg = _cfg(masks)
+    gpu = DynamicCache(cfg)
+    cpu = OracleCache(cfg, masks=masks, model_dtype="bf16")
+    r = np.random.default_rng(12)
+    prompt = 30   # <= maxlen = 36
+    k0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype); v0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    q0 = H.to_dtype_np(r.standard_normal((B, Hq, prompt, D)), dtype)
+    out = fourier_attention(H.to_gpu(q0, dtype), H.to_gpu(k0, dtype), H.to_gpu(v0, dtype), gpu, 0, Hq, Hkv)
+    cpu.update(k0, v0, 0)
+    assert tuple(out.shape) == (B, prompt, Hq * D) and out.dtype == dtype
+    # last prompt position sees every key: compare with exact attention
+    kk = np.transpose(k0, (0, 2, 1, 3)).reshape(B, prompt, -1); vv = np.transpose(v0, (0, 2, 1, 3)).reshape(B, prompt, -1)
+    want = fo.softmax_attention(np.transpose(q0[:, :, -1:], (0, 2, 1, 3)).reshape(B, -1), kk, vv, Hq, Hkv).reshape(B, -1)
+    assert np.abs(out[:, -1].float().cpu().numpy() - want).max() <= 2e-2
+    for s in range(12):   # grows past maxlen without ever compressing (the reference's predicate)
+        kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype); vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+        q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)), dtype)
+        o = fourier_attention(H.to_gpu(q, dtype), H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), gpu, 0, Hq, Hkv)
+        kw, vw = cpu.update(kn, vn, 0)
+        assert kw["k_init"] is None
+        want = cpu.attend(q, kw, vw, 0, Hq, Hkv).reshape(B, 1, -1)
+        assert np.abs(o.float().cpu().numpy() - want).max() <= 2e-2
+        assert gpu.get_seq_length() == cpu.get_seq_length() == prompt + s + 1
+        kc = gpu.key_cache[0]
+        assert kc["k_init"].shape == (B, 0, Hkv * D) and kc["k_init"].device.type == "cpu" and kc["k_init"].dtype == torch.float32
+        assert tuple(kc["k_local"].shape) == (B, prompt + s + 1, Hkv * D)
+
+
+def test_append_branch_of_a_short_mid():
+    """Coefficient rows and batch size enter the decode predicate: with M < L < W - B the cache
+    keeps appending to the window and attention sees the window only (reference behaviour)."""
+    from fourierattention_amd import DynamicCache
+    B, Hq, Hkv, D = 1, 4, 2, 32
+    dtype = torch.bfloat16
+    masks = _masks(1, Hkv, D, [16, 16], [16, 16])
+    cfg = _cfg(masks, maxlocallen=64, maxmidstates=8, numinittokens=4, max_new_tokens=8)
+    gpu = DynamicCache(cfg); cpu = OracleCache(cfg, masks=masks, model_dtype="bf16")
+    r = np.random.default_rng(13)
+    prompt = 4 + 64 + 20    # L = 20: M(8) < L and 4 + 8 + 20 + 1 + 1 <= 76
+    k0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype); v0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    gpu.update(H.to_gpu(k0, dtype), H.to_gpu(v0, dtype), 0); cpu.update(k0, v0, 0)
+    for s in range(3):
+        kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype); vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+        q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)), dtype)
+        kp, vp = gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), 0)
+        kw, vw = cpu.update(kn, vn, 0)
+        assert kp["k_init"] is None and kw["k_init"] is None
+        np.testing.assert_array_equal(kp["k_local"].float().cpu().numpy(), kw["k_local"].astype(np.float32))
+        assert gpu.get_seq_length() == cpu.get_seq_length()
+        want = cpu.attend(q, kw, vw, 0, Hq, Hkv)
+        got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv)
+        assert np.abs(got.cpu().numpy() - want).max() <= 1e-3
+        _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype)
