@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the Fourier-cache decode hot path on one MI355X.
+
+One "step" = one decode-attention pass of one layer over a resident Fourier cache
+(BASELINE config 3: B=8, ctx 32768, Hq=32, Hkv=8, D=128, 4 sink + 1024 window rows full,
+64 of 128 dims per head stored as M=1024 coefficients, bf16).  Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+WORKLOADS = {
+    # name: B, ctx, Hq, Hkv, D, I, W, M, compressed dims per head, max_new_tokens
+    "config3_decode_attn_8b_32k": dict(B=8, ctx=32768, Hq=32, Hkv=8, D=128, I=4, W=1024, M=1024, cper=64, max_new=128),
+    "config1_cpu_geometry_3b_2k": dict(B=1, ctx=2048, Hq=24, Hkv=8, D=128, I=4, W=512, M=256, cper=64, max_new=64),
+}
+
+
+def algorithmic_bytes(w, coef_bytes=4, elem_bytes=2):
+    """Compulsory HBM bytes of one decode-attention pass (per layer, whole batch):
+    sink+window K,V (all dims) + stored dims of the mid rows (K,V) + coefficients (K,V) + q + out."""
+    L = w["ctx"] - w["I"] - w["W"]
+    hd = w["Hkv"] * w["D"]
+    ck = w["cper"] * w["Hkv"]
+    cn = hd - ck
+    per_b = 2 * (w["I"] + w["W"]) * hd * elem_bytes + 2 * L * cn * elem_bytes + 2 * w["M"] * ck * coef_bytes \
+        + 2 * w["Hq"] * w["D"] * elem_bytes
+    return per_b * w["B"]
+
+
+def build_cache(w, dtype, device, seed=0, layers=1):
+    """Random K/V of the workload's shape pushed through the cache's own prefill (split, spectral
+    compression, statistics), so the timed decode reads exactly what a real prompt leaves behind."""
+    from fourierattention_amd import DynamicCache, ExtraConfig, masks, synth
+    m = masks.synthetic_masks(layers, w["Hkv"], w["D"], w["cper"], seed=seed)
+    cfg = ExtraConfig(numinittokens=w["I"], maxlocallen=w["W"], maxmidstates=w["M"], non_critical_dims=m,
+                      non_critical_dims_path=None, max_position_embeddings=1 << 20, num_key_value_heads=w["Hkv"],
+                      max_new_tokens=w["max_new"], model_type="llama")
+    cache = DynamicCache(cfg, device=device)
+    g = torch.Generator(device=device).manual_seed(seed)
+    B, Hkv, S, D = w["B"], w["Hkv"], w["ctx"], w["D"]
+    cos, sin = synth.rope_tables(torch.arange(S), D)
+    cos, sin = cos.to(device), sin.to(device)
+    for layer in range(layers):
+        k = torch.randn((B, Hkv, S, D), generator=g, device=device, dtype=torch.float32)
+        k = synth.apply_rope(k, cos, sin).to(dtype)
+        v = torch.randn((B, Hkv, S, D), generator=g, device=device, dtype=torch.float32).to(dtype)
+        cache.update(k, v, layer)
+        del k, v
+    cq, sq = synth.rope_tables(torch.tensor([S]), D)
+    q = torch.randn((B, w["Hq"], 1, D), generator=g, device=device, dtype=torch.float32)
+    q = synth.apply_rope(q, cq.to(device), sq.to(device)).to(dtype)
+    kn = synth.apply_rope(torch.randn((B, Hkv, 1, D), generator=g, device=device), cq.to(device), sq.to(device)).to(dtype)
+    vn = torch.randn((B, Hkv, 1, D), generator=g, device=device).to(dtype)
+    return cache, q, kn, vn
+
+
+def parity_check(device):
+    """Small seeded case through the GPU cache and through the CPU oracle; returns max-abs error."""
+    from oracle.cache_oracle import OracleCache
+    from oracle import fourier_oracle as fo
+    from fourierattention_amd import DynamicCache, ExtraConfig, masks
+    B, Hq, Hkv, D, S = 2, 8, 2, 128, 700
+    m = masks.synthetic_masks(1, Hkv, D, 64, seed=3)
+    cfg = ExtraConfig(numinittokens=4, maxlocallen=64, maxmidstates=64, non_critical_dims=m, non_critical_dims_path=None,
+                      max_position_embeddings=1 << 20, num_key_value_heads=Hkv, max_new_tokens=16, model_type="llama")
+    r = np.random.default_rng(0)
+    rd = lambda a: fo.round_bf16(a).astype(np.float64)
+    k, v = rd(r.standard_normal((B, Hkv, S, D))), rd(r.standard_normal((B, Hkv, S, D)))
+    kn, vn, q = rd(r.standard_normal((B, Hkv, 1, D))), rd(r.standard_normal((B, Hkv, 1, D))), rd(r.standard_normal((B, Hq, 1, D)))
+    g = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16).to(device)
+    gpu = DynamicCache(cfg, device=device)
+    cpu = OracleCache(cfg, masks=m, model_dtype="bf16")
+    gpu.update(g(k), g(v), 0); cpu.update(k, v, 0)
+    gpu.update(g(kn), g(vn), 0); kw, vw = cpu.update(kn, vn, 0)
+    got = gpu.decode_attention(g(q), 0, Hq, Hkv).float().cpu().numpy()
+    want = cpu.attend(q, kw, vw, 0, Hq, Hkv)
+    return float(np.abs(got - want).max())
+
+
+def cpu_baseline():
+    """The CPU restatement of the reference path (numpy, float64) on BASELINE config 1:
+    one layer, one decode step = cache update (rank-1 coefficient update, eviction) + attention."""
+    from oracle.cache_oracle import OracleCache
+    from oracle import fourier_oracle as fo
+    from fourierattention_amd import ExtraConfig, masks
+    w = WORKLOADS["config1_cpu_geometry_3b_2k"]
+    m = masks.synthetic_masks(1, w["Hkv"], w["D"], w["cper"], seed=0)
+    cfg = ExtraConfig(numinittokens=w["I"], maxlocallen=w["W"], maxmidstates=w["M"], non_critical_dims=m,
+                      non_critical_dims_path=None, max_position_embeddings=131072, num_key_value_heads=w["Hkv"],
+                      max_new_tokens=w["max_new"], model_type="llama")
+    r = np.random.default_rng(0)
+    B, Hq, Hkv, D, S = w["B"], w["Hq"], w["Hkv"], w["D"], w["ctx"]
+    cos, sin = fo.rope_tables(np.arange(S), D)
+    k = fo.apply_rope(r.standard_normal((B, Hkv, S, D)), cos, sin).astype(np.float32).astype(np.float64)
+    v = r.standard_normal((B, Hkv, S, D)).astype(np.float32).astype(np.float64)
+    cache = OracleCache(cfg, masks=m, model_dtype="fp32")
+    cache.update(k, v, 0)
+    cq, sq = fo.rope_tables(np.array([S]), D)
+    times = []
+    for rep in range(13):
+        kn = fo.apply_rope(r.standard_normal((B, Hkv, 1, D)), cq, sq)
+        vn = r.standard_normal((B, Hkv, 1, D))
+        q = fo.apply_rope(r.standard_normal((B, Hq, 1, D)), cq, sq)
+        t0 = time.perf_counter()
+        kw, vw = cache.update(kn, vn, 0)
+        cache.attend(q, kw, vw, 0, Hq, Hkv)
+        times.append(time.perf_counter() - t0)
+    times = sorted(times[3:])
+    med = times[len(times) // 2]
+    nbytes = algorithmic_bytes(w, coef_bytes=4, elem_bytes=4)
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = 1
+    return {"value": round(nbytes / med / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "sample": f"config 1 (B=1, ctx 2048, Hq=24, Hkv=8, D=128, fp32 inputs, M=256, W=512): update + attention of one layer, "
+                      f"one decode step, median of 10 after 3 warm-ups = {med * 1e3:.2f} ms (min {times[0] * 1e3:.2f} ms), "
+                      f"{nbytes} algorithmic bytes; host has {os.cpu_count()} logical CPUs"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="config3_decode_attn_8b_32k", choices=list(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives exist on this path); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path exists only as HIP kernels", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    from fourierattention_amd import _lib
+    _lib.load()
+
+    w = WORKLOADS[args.workload]
+    dtype = torch.bfloat16
+    parity = parity_check(device)
+    if not parity <= 2e-2:
+        print(f"bench.py: parity check failed (max abs err {parity})", file=sys.stderr)
+        sys.exit(1)
+    cache, q, kn, vn = build_cache(w, dtype, device)
+    Hq, Hkv = w["Hq"], w["Hkv"]
+    for _ in range(args.warmup):
+        out = cache.decode_attention(q, 0, Hq, Hkv)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        out = cache.decode_attention(q, 0, Hq, Hkv)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = start.elapsed_time(stop) / args.steps
+    assert torch.isfinite(out).all()
+
+    nbytes = algorithmic_bytes(w)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    L = w["ctx"] - w["I"] - w["W"]
+    full = 2 * w["ctx"] * w["Hkv"] * w["D"] * 2
+    fourier = (2 * (w["I"] + w["W"]) * w["Hkv"] * w["D"] * 2 + 2 * L * (w["Hkv"] * w["D"] - w["cper"] * w["Hkv"]) * 2
+               + 2 * w["M"] * w["cper"] * w["Hkv"] * 4)
+    result = {
+        "metric": "Fourier decode attn HBM GB/s (% peak) + tok/s, Llama-3.1-8B geometry, 32k ctx",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "batch": w["B"], "context": w["ctx"], "q_heads": Hq, "kv_heads": Hkv,
+                   "head_dim": w["D"], "sink": w["I"], "window": w["W"], "coeff_rows": w["M"],
+                   "compressed_dims_per_head": w["cper"], "coeff_dtype": "f32"},
+        "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "attn_only_tok_s": round(w["B"] / (args.layers * ms * 1e-3), 1),
+        "kv_bytes_per_layer_per_seq": {"full_bf16": full, "fourier": fourier, "reduction": round(full / fourier, 3)},
+        "algorithmic_bytes_per_step": nbytes,
+        "parity_max_abs_err": parity,
+        "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "all kernels of one fa_decode_attn call"},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -112,7 +112,7 @@ def compress_prefill(x: np.ndarray, n_f: int, t_c: int, dtype=np.float64) -> np.
     t = np.arange(l_eff)
     ph = _phase_matrix(n, t, t_c)  # (n_f, l_eff)
     basis = np.concatenate([np.cos(ph), np.sin(ph)], axis=0).astype(dtype)  # (2 n_f, l_eff)
-    return np.einsum("nt,btc->bnc", basis, x[:, :l_eff, :], optimize=True)
+    return np.ascontiguousarray(np.einsum("nt,btc->bnc", basis, x[:, :l_eff, :], optimize=True))
 
 
 def coeff_update(coef: np.ndarray, evicted: np.ndarray, p: int, t_c: int, dtype=np.float64) -> np.ndarray:
@@ -156,7 +156,7 @@ def reconstruct(coef: np.ndarray, k: int, t_x: int, dtype=np.float64) -> np.ndar
     n_f = coef.shape[1] // 2
     ph = _phase_matrix(np.arange(k), np.arange(n_f), t_x)  # (k, n_f)
     basis = np.concatenate([np.cos(ph), np.sin(ph)], axis=1).astype(dtype)  # (k, 2 n_f)
-    return np.einsum("ln,bnc->blc", basis, coef, optimize=True) / n_f
+    return np.ascontiguousarray(np.einsum("ln,bnc->blc", basis, coef, optimize=True)) / n_f
 
 
 def stats_reconstructed(coef: np.ndarray, k: int, t_x: int) -> Tuple[np.ndarray, np.ndarray]:
