@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(PKG_DIR, "libfourier_attn_hip.so")
 
 FA_BF16, FA_FP16, FA_FP32 = 0, 1, 2
 FA_NO_ROUND = FA_FP32
+FA_MID_TOKEN_MAJOR, FA_MID_PAGED = 0, 1
+PAGE_TOKENS, K_DIM_PAD, V_DIM_PAD = 32, 32, 16
 
 STATUS_NAMES = {
     0: "FA_OK", -1: "FA_ERR_NULL_POINTER", -2: "FA_ERR_BAD_SHAPE", -3: "FA_ERR_BAD_DTYPE", -4: "FA_ERR_WORKSPACE",
@@ -37,6 +39,10 @@ class DecodeArgs(ctypes.Structure):
         ("k_mn", c_void_p), ("v_mn", c_void_p),
         ("k_mn_batch_stride", c_int64), ("k_mn_row_stride", c_int64),
         ("v_mn_batch_stride", c_int64), ("v_mn_row_stride", c_int64),
+        ("mid_layout", c_int32), ("mid_cap_pages", c_int32),
+        ("k_pad_h_list", c_void_p), ("v_pad_h_list", c_void_p),
+        ("mid_max_k_pad", c_int32), ("mid_max_v_pad", c_int32),
+        ("tables", c_void_p), ("force_generic", c_int32),
         ("avg_k_u", c_void_p), ("avg_k_d", c_void_p), ("scale_k", c_void_p),
         ("avg_v_u", c_void_p), ("avg_v_d", c_void_p), ("scale_v", c_void_p),
         ("kc_list", c_void_p), ("kc_h_list", c_void_p), ("kn_list", c_void_p), ("kn_h_list", c_void_p),
@@ -67,6 +73,14 @@ _SIGNATURES = {
                                 c_void_p]),
     "fa_decode_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "fa_decode_attn": (c_int, [POINTER(DecodeArgs), c_void_p]),
+    "fa_decode_tables_bytes": (c_size_t, [c_int]),
+    "fa_decode_tables_build": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),
+    "fa_mid_pack": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p,
+                            c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "fa_mid_append": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                              c_int, c_int, c_int, c_int, c_void_p]),
+    "fa_mid_unpack": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                              c_int, c_int, c_void_p]),
 }
 
 EXPORTED = tuple(_SIGNATURES)

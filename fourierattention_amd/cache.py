@@ -25,6 +25,7 @@ import torch
 
 from . import ops
 from .bookkeeping import Action, CacheBook
+from .midstore import MidStore
 
 _PART_NAMES = ("init", "compressed", "uncompressed", "local")
 
@@ -43,7 +44,7 @@ class _Tensor:
         self.init: Optional[torch.Tensor] = None        # (B, I, HD)
         self.ring: Optional[torch.Tensor] = None        # (B, W, HD) when compressed, else growing (B, cap, HD)
         self.coef: Optional[torch.Tensor] = None        # (B, 2N, C) fp32
-        self.mid: Optional[torch.Tensor] = None         # (B, cap, Cn)
+        self.mid: Optional[MidStore] = None             # paged store of the stored dims of the mid rows
         self.stats32: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None  # avg_u, avg_d, scale fp32
 
 
@@ -91,7 +92,7 @@ class CacheParts(Mapping):
         if part == "compressed":
             return t.coef
         if part == "uncompressed":
-            return t.mid[:, : layer.n_mid, :]
+            return t.mid.dense(layer.n_mid)
         return self.cache._window_in_order(layer, t)
 
 
@@ -151,6 +152,10 @@ class DynamicCache:
                 self.v_non_critical_dims[-1], self.v_non_critical_head_dims[-1],
                 self.v_critical_dims[-1], self.v_critical_head_dims[-1])))
         self._num_layers = len(masks)
+        self._head_lists = [([0] + list(masks[f"Layer_{i}"]["kn_h_list"]), [0] + list(masks[f"Layer_{i}"]["vn_h_list"]))
+                            for i in range(self._num_layers)]
+        self._tables: Optional[torch.Tensor] = None   # constant operands of the MFMA decode kernels
+        self.force_generic = False                     # testing: keep decode attention off the MFMA kernels
         self._book = CacheBook(self._num_layers, self.numinittokens, self.maxlocallen, self.maxmidstates,
                                self.maxnewtokens, self.maxtokens)
         self._layers: List[_Layer] = [_Layer() for _ in range(self._num_layers)]
@@ -216,17 +221,16 @@ class DynamicCache:
         """The window as up to two (k, v) views whose union is the window (order irrelevant to attention)."""
         return [(layer.k.ring[:, : layer.n_local, :], layer.v.ring[:, : layer.n_local, :])]
 
-    def _compress_tensor(self, t: _Tensor, states: torch.Tensor, c32: torch.Tensor, n64: torch.Tensor, L: int,
-                         fft_rows: int, n_f: int):
+    def _compress_tensor(self, t: _Tensor, states: torch.Tensor, c32: torch.Tensor, n32: torch.Tensor, nh32: torch.Tensor,
+                         nh_host, is_v: bool, L: int, fft_rows: int, n_f: int):
         I, W = self.numinittokens, self.maxlocallen
         B, S, HD = states.shape
         mid = states[:, I: S - W, :]
         t.init = states[:, :I, :].contiguous()
         t.ring = states[:, S - W:, :].contiguous()
         cap = max(self._book.t_x, L) + 1
-        t.mid = torch.empty((B, cap, n64.numel()), dtype=states.dtype, device=states.device)
-        if n64.numel():
-            t.mid[:, :L, :].copy_(mid[:, :, n64])
+        t.mid = MidStore(B, n32, nh32, nh_host, self.heads, self.head_dim, cap, states.dtype, states.device, is_v)
+        t.mid.pack(states, I, L)
         # spectral compression of the selected columns (gather fused into the kernel)
         t.coef = ops.mat_fourier(mid, n_f, self._book.t_c, 0, cols=c32, K=fft_rows)
         u_avg, u_std = ops.mat_avg_std(mid, cols=c32, round_dtype=states.dtype)
@@ -271,10 +275,13 @@ class DynamicCache:
             if step.action is Action.PREFILL_COMPRESS:
                 l32 = self._lists32[layer_idx]
                 n_f = self.maxmidstates // 2
-                ks, ku, kd = self._compress_tensor(layer.k, k, l32[0], self.k_critical_dims[layer_idx], step.mid_rows,
+                hl = self._head_lists[layer_idx]
+                ks, ku, kd = self._compress_tensor(layer.k, k, l32[0], l32[2], l32[3], hl[0], False, step.mid_rows,
                                                    step.fft_rows, n_f)
-                vs, vu, vd = self._compress_tensor(layer.v, v, l32[4], self.v_critical_dims[layer_idx], step.mid_rows,
+                vs, vu, vd = self._compress_tensor(layer.v, v, l32[4], l32[6], l32[7], hl[1], True, step.mid_rows,
                                                    step.fft_rows, n_f)
+                if self._tables is None and layer_idx == 0:
+                    self._tables = ops.decode_tables(n_f, self.period_reconstruct, self.device)
                 layer.compressed, layer.window_only, layer.growing, layer.ring_head = True, False, False, 0
                 layer.n_local, layer.n_mid = self.maxlocallen, step.mid_rows
                 self._store_stats(layer_idx, ks, ku, kd, vs, vu, vd)
@@ -333,16 +340,12 @@ class DynamicCache:
         p = step.phase
         l32 = self._lists32[layer_idx]
         h = layer.ring_head
-        for t, new, c32, n64 in ((layer.k, k, l32[0], self.k_critical_dims[layer_idx]),
-                                 (layer.v, v, l32[4], self.v_critical_dims[layer_idx])):
+        for t, new, c32 in ((layer.k, k, l32[0]), (layer.v, v, l32[4])):
             oldest = t.ring[:, h, :]
             ops.coeff_update_(t.coef, oldest, c32, p, self._book.t_c)
-            if layer.n_mid >= t.mid.shape[1]:
-                grown = torch.empty((bsz, 2 * t.mid.shape[1], t.mid.shape[2]), dtype=t.mid.dtype, device=t.mid.device)
-                grown[:, : layer.n_mid, :].copy_(t.mid[:, : layer.n_mid, :])
-                t.mid = grown
-            if n64.numel():
-                t.mid[:, layer.n_mid, :].copy_(oldest[:, n64])
+            if layer.n_mid >= t.mid.cap_tokens:
+                t.mid.grow(layer.n_mid, 2 * t.mid.cap_tokens)
+            t.mid.append(oldest, layer.n_mid)
             t.ring[:, h, :].copy_(new[:, 0, :])
         layer.n_mid += 1
         layer.ring_head = (h + 1) % self.maxlocallen
@@ -386,4 +389,4 @@ class DynamicCache:
         segs = [(layer.k.init, layer.v.init)] + self._window_segments(layer)
         return ops.decode_attn_raw(q, segs, layer.k.coef, layer.v.coef, layer.k.mid, layer.v.mid, layer.k.stats32,
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
-                                   sm_scale)
+                                   sm_scale, tables=self._tables, force_generic=self.force_generic)

@@ -1,4 +1,5 @@
-// Decode attention over [sink ; local window ; mid rows], any shape (generic path).
+// Decode attention over [sink ; local window ; mid rows]: the generic VALU kernels that accept any
+// shape, the vectorised sink/window kernel, and the dispatch to the MFMA path (fa_decode_mfma.h).
 //
 // The compressed dims of the mid rows are never rebuilt.  With s = scale,
 // a = avg_u - avg_d * s and F[l, n] = cos / sin(2 pi n l / T):
@@ -8,6 +9,7 @@
 // per-token reconstruction, and the token loop only touches the stored dims.
 // All exponentials are base 2 (scores carry log2(e)).
 #include "fa_common.h"
+#include "fa_decode_mfma.h"
 
 namespace {
 
@@ -192,10 +194,19 @@ __global__ __launch_bounds__(256) void decode_il_kernel(
 // ---------------------------------------------------------------------------
 // mid rows: split over tokens; per split partial (m, d, g[2N], o_n[vn_len])
 // ---------------------------------------------------------------------------
-template <typename E>
+// element offset of (token, stored dim j) inside one (batch, head) run of pages
+__device__ __forceinline__ int64_t paged_offset(bool is_v, int dp, int64_t token, int j) {
+  const int64_t page = token >> 5;
+  const int t = (int)(token & 31);
+  if (!is_v) return page * dp * 32 + (int64_t)((t >> 4) * (dp >> 5) + (j >> 5)) * 512 + (((j & 31) >> 3) * 16 + (t & 15)) * 8 + (j & 7);
+  return page * dp * 32 + (int64_t)(j >> 4) * 512 + ((t >> 3) * 16 + (j & 15)) * 8 + (t & 7);
+}
+
+template <typename E, bool PAGED>
 __global__ __launch_bounds__(256) void decode_mid_kernel(
     const E* __restrict__ q, const E* __restrict__ k_mn, int64_t k_bs, int64_t k_rs,
-    const E* __restrict__ v_mn, int64_t v_bs, int64_t v_rs, const float* __restrict__ W,
+    const E* __restrict__ v_mn, int64_t v_bs, int64_t v_rs, int cap_pages, const int32_t* __restrict__ kpad_h,
+    const int32_t* __restrict__ vpad_h, const float* __restrict__ W,
     const float* __restrict__ c0, const int32_t* __restrict__ kn_list, const int32_t* __restrict__ kn_h,
     const int32_t* __restrict__ vn_h, float* __restrict__ pm, float* __restrict__ pd,
     float* __restrict__ pg, float* __restrict__ pon, int Hq, int Hkv, int D, int N, int L_m, int T,
@@ -237,8 +248,18 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
 
   const int l_beg = split * tiles_per_split * kTile;
   const int l_end = min(L_m, l_beg + tiles_per_split * kTile);
-  const E* kb = k_mn + (int64_t)b * k_bs + kn0;
-  const E* vb = v_mn + (int64_t)b * v_bs + vn0;
+  int dpk = 0, dpv = 0;
+  const E* kb;
+  const E* vb;
+  if (PAGED) {
+    dpk = kpad_h[h + 1] - kpad_h[h];
+    dpv = vpad_h[h + 1] - vpad_h[h];
+    kb = k_mn + (int64_t)b * k_bs + (int64_t)kpad_h[h] * 32 * cap_pages;
+    vb = v_mn + (int64_t)b * v_bs + (int64_t)vpad_h[h] * 32 * cap_pages;
+  } else {
+    kb = k_mn + (int64_t)b * k_bs + kn0;
+    vb = v_mn + (int64_t)b * v_bs + vn0;
+  }
   const int dim = tid % 128, half = tid / 128;
 
   for (int l0 = l_beg; l0 < l_end; l0 += kTile) {
@@ -262,9 +283,8 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
         zr = nr;
         zi = ni;
       }
-      const E* krow = kb + (int64_t)l * k_rs;
       for (int j = 0; j < kn_len; ++j) {
-        float kv = fa_to_float(krow[j]);
+        float kv = fa_to_float(PAGED ? kb[paged_offset(false, dpk, l, j)] : kb[(int64_t)l * k_rs + j]);
 #pragma unroll
         for (int g = 0; g < kGMax; ++g)
           if (g < G) sc[g] = fmaf(kv, s_qn[g * D + j], sc[g]);
@@ -330,7 +350,7 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
     for (int g = 0; g < kGMax; ++g) on[g] *= alpha[g];
     if (dim < vn_len) {
       for (int tt = half; tt < t_len; tt += 2) {
-        float vv = fa_to_float(vb[(int64_t)(l0 + tt) * v_rs + dim]);
+        float vv = fa_to_float(PAGED ? vb[paged_offset(true, dpv, l0 + tt, dim)] : vb[(int64_t)(l0 + tt) * v_rs + dim]);
 #pragma unroll
         for (int g = 0; g < kGMax; ++g)
           if (g < G) on[g] = fmaf(s_p[g * kTile + tt], vv, on[g]);
@@ -442,45 +462,241 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// sink + local window, vectorised (16-bit storage, head_dim 64 or 128, 16-byte aligned rows):
+// LPT = D/8 lanes share one row, each holding 8 dims; a wave walks 64/LPT rows per step with an
+// online softmax of its own; the four waves of the block are merged through LDS.
+// ---------------------------------------------------------------------------
+template <typename E, int D>
+__global__ __launch_bounds__(256) void decode_il_fast_kernel(
+    const E* __restrict__ q, Seg s0, Seg s1, float* __restrict__ pm, float* __restrict__ pd,
+    float* __restrict__ po, int Hq, int Hkv, int n_split, float sm_log2e) {
+  constexpr int LPT = D / 8, TPW = 64 / LPT;
+  __shared__ float s_m[4][kGMax], s_d[4][kGMax];
+  __shared__ float s_o[4][kGMax][D];
+  const int G = Hq / Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int sub = lane % LPT, tl = lane / LPT;
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int n_il = s0.rows + s1.rows;
+  float qv[kGMax][8];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      qv[g][e] = g < G ? fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + sub * 8 + e]) * sm_log2e : 0.f;
+  float m[kGMax], d[kGMax], o[kGMax][8];
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g) {
+    m[g] = -INFINITY;
+    d[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
+  }
+  const int base = split * kTile + w * 64;
+  for (int it = 0; it < 64 / TPW; ++it) {
+    const int i = base + it * TPW + tl;
+    const bool ok = i < n_il;
+    if (__all(!ok)) break;
+    const int ii = ok ? i : 0;
+    const bool in0 = ii < s0.rows;
+    const int64_t off = in0 ? (int64_t)b * s0.bs + (int64_t)ii * s0.rs : (int64_t)b * s1.bs + (int64_t)(ii - s0.rows) * s1.rs;
+    const E* kp = (in0 ? (const E*)s0.k : (const E*)s1.k) + off + h * D + sub * 8;
+    const E* vp = (in0 ? (const E*)s0.v : (const E*)s1.v) + off + h * D + sub * 8;
+    uint4 kraw = *(const uint4*)kp, vraw = *(const uint4*)vp;
+    const E* ke = (const E*)&kraw;
+    const E* ve = (const E*)&vraw;
+    float kf[8], vf[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      kf[e] = fa_to_float(ke[e]);
+      vf[e] = fa_to_float(ve[e]);
+    }
+    float sc[kGMax], mx[kGMax];
+    bool changed = false;
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) {
+      if (g < G) {
+        float a = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a = fmaf(kf[e], qv[g][e], a);
+#pragma unroll
+        for (int o_ = 1; o_ < LPT; o_ <<= 1) a += __shfl_xor(a, o_, 64);
+        sc[g] = ok ? a : -INFINITY;
+        float t = sc[g];
+#pragma unroll
+        for (int o_ = LPT; o_ < 64; o_ <<= 1) t = fmaxf(t, __shfl_xor(t, o_, 64));
+        mx[g] = fmaxf(m[g], t);
+        changed |= mx[g] != m[g];
+      }
+    }
+    if (changed) {  // wave-uniform: every lane sees the same maxima
+#pragma unroll
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) {
+          const float al = exp2f(m[g] - mx[g]);
+          d[g] *= al;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[g][e] *= al;
+          m[g] = mx[g];
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) {
+        const float pv = exp2f(sc[g] - m[g]);
+        d[g] += pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pv, vf[e], o[g][e]);
+      }
+  }
+  // reduce over the rows a wave holds side by side, then over the four waves
+#pragma unroll
+  for (int g = 0; g < kGMax; ++g)
+    if (g < G) {
+#pragma unroll
+      for (int o_ = LPT; o_ < 64; o_ <<= 1) {
+        d[g] += __shfl_xor(d[g], o_, 64);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] += __shfl_xor(o[g][e], o_, 64);
+      }
+      if (tl == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_o[w][g][sub * 8 + e] = o[g][e];
+        if (sub == 0) {
+          s_m[w][g] = m[g];
+          s_d[w][g] = d[g];
+        }
+      }
+    }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int g = idx / D, dim = idx % D;
+    const float mm = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
+    float acc = 0.f, dd = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < 4; ++ww) {
+      const float wgt = s_m[ww][g] == -INFINITY ? 0.f : exp2f(s_m[ww][g] - mm);
+      acc = fmaf(wgt, s_o[ww][g][dim], acc);
+      dd = fmaf(wgt, s_d[ww][g], dd);
+    }
+    const int64_t r = ((int64_t)b * Hq + h * G + g) * n_split + split;
+    po[r * D + dim] = acc;
+    if (dim == 0) {
+      pm[r] = mm;
+      pd[r] = dd;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
+int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+// which implementation handles the mid rows
+enum class Path { Generic, Mfma };
+
 struct Plan {
-  int n_il_split, n_mid_split, tiles_per_split;
-  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, total;
+  Path path;
+  int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, total;
 };
 
-Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m) {
+bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
+  const int G = Hq / Hkv;
+  return layout == FA_MID_PAGED && (dtype == FA_BF16 || dtype == FA_FP16) && G <= 16 && D <= 128 &&
+         (N == 128 || N == 256 || N == 512);
+}
+
+Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma) {
   Plan p{};
+  p.path = mfma ? Path::Mfma : Path::Generic;
   p.n_il_split = fa_cdiv(n_il, kTile);
-  const int tiles = fa_cdiv(L_m, kTile);
-  int want = fa_cdiv(1024, (int64_t)B * Hkv);
-  if (want < 1) want = 1;
-  int ns = tiles < want ? tiles : want;
-  if (ns > 64) ns = 64;
-  p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
-  p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+  if (mfma) {
+    const int G = Hq / Hkv;
+    p.nbpg = 16 / G < 4 ? 16 / G : 4;       // one wave streams one batch element of the group
+    if (p.nbpg > B) p.nbpg = B;
+    p.n_groups = fa_cdiv(B, p.nbpg);
+    p.ks = N / 64;
+    const int tiles = fa_cdiv(L_m, 32);
+    int want = fa_cdiv(device_cu_count(), (int64_t)Hkv * p.n_groups);
+    if (want < 1) want = 1;
+    int ns = tiles < want ? tiles : want;
+    p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
+    p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+  } else {
+    const int tiles = fa_cdiv(L_m, kTile);
+    int want = fa_cdiv(1024, (int64_t)B * Hkv);
+    if (want < 1) want = 1;
+    int ns = tiles < want ? tiles : want;
+    if (ns > 64) ns = 64;
+    p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
+    p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+  }
   const size_t rows = (size_t)B * Hq;
   size_t o = 0;
-  auto take = [&](size_t n_float) {
+  auto take = [&](size_t bytes) {
     size_t at = o;
-    o += fa_align_up(n_float * sizeof(float), 256);
+    o += fa_align_up(bytes, 256);
     return at;
   };
-  p.off_W = take(rows * 2 * N);
-  p.off_c0 = take(rows);
-  p.off_ilm = take(rows * p.n_il_split);
-  p.off_ild = take(rows * p.n_il_split);
-  p.off_ilo = take(rows * p.n_il_split * D);
-  p.off_mm = take(rows * p.n_mid_split);
-  p.off_md = take(rows * p.n_mid_split);
-  p.off_mg = take(rows * p.n_mid_split * 2 * N);
-  p.off_mon = take(rows * p.n_mid_split * D);
+  p.off_W = take(rows * 2 * N * 4);
+  p.off_c0 = take(rows * 4);
+  p.off_ilm = take(rows * p.n_il_split * 4);
+  p.off_ild = take(rows * p.n_il_split * 4);
+  p.off_ilo = take(rows * p.n_il_split * D * 4);
+  p.off_mm = take(rows * p.n_mid_split * 4);
+  p.off_md = take(rows * p.n_mid_split * 4);
+  p.off_mg = take(rows * p.n_mid_split * 2 * N * 4);
+  p.off_mon = take(rows * p.n_mid_split * D * 4);
+  p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
   p.total = o;
   return p;
 }
 
 template <typename E>
-int launch_generic(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream_t st) {
+bool il_fast_ok(const fa_decode_args& a) {
+  if (sizeof(E) != 2 || (a.D != 64 && a.D != 128)) return false;
+  for (int i = 0; i < 2; ++i) {
+    if (a.il_rows[i] == 0) continue;
+    if (((uintptr_t)a.k_il[i] & 15) || ((uintptr_t)a.v_il[i] & 15)) return false;
+    if ((a.il_batch_stride[i] & 7) || (a.il_row_stride[i] & 7)) return false;
+  }
+  return true;
+}
+
+void launch_tables(void* tables, int N, int T, hipStream_t st) {
+  using namespace fa_mfma;
+  const int KS = N / 64;
+  half8* tabE = (half8*)tables;
+  half8* tabET = tabE + 4 * 2 * KS * 64;
+  float2v* rot = (float2v*)(tabET + 4 * 2 * KS * 64);
+  const int total = 2 * 4 * 2 * KS * 64 + N;
+  decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N);
+}
+
+template <typename E, int KS>
+void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
+  dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
+  if (wide)
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8><<<grid, 256, 0, st>>>(mp);
+  else
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4><<<grid, 256, 0, st>>>(mp);
+}
+
+template <typename E>
+int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream_t st) {
   char* ws = (char*)a.workspace;
   float* W = (float*)(ws + p.off_W);
   float* c0 = (float*)(ws + p.off_c0);
@@ -498,23 +714,67 @@ int launch_generic(const fa_decode_args& a, const Plan& p, float sm_scale, hipSt
     decode_prep_kernel<E><<<dim3(fa_cdiv(2 * a.N, rows_per_block), a.Hkv, a.B), 256, 0, st>>>(
         (const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0, a.Hq, a.Hkv, a.D,
         a.N, a.Ck, sm_log2e, rows_per_block);
-    size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
-    if (lds > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_mid_kernel<E>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
+    if (p.path == Path::Mfma) {
+      if constexpr (sizeof(E) == 2) {
+        using namespace fa_mfma;
+        void* tables = a.tables ? (void*)a.tables : (void*)(ws + p.off_tab);
+        if (!a.tables) launch_tables(tables, a.N, a.T, st);
+        const int KS = p.ks;
+        MidParams<E> mp{};
+        mp.q = (const E*)a.q; mp.W = W; mp.c0 = c0;
+        mp.k_mid = (const E*)a.k_mn; mp.v_mid = (const E*)a.v_mn;
+        mp.k_bs = a.k_mn_batch_stride; mp.v_bs = a.v_mn_batch_stride; mp.cap_pages = a.mid_cap_pages;
+        mp.kn_list = a.kn_list; mp.kn_h = a.kn_h_list; mp.kpad_h = a.k_pad_h_list;
+        mp.vn_h = a.vn_h_list; mp.vpad_h = a.v_pad_h_list;
+        mp.tabE = (const half8*)tables;
+        mp.tabET = mp.tabE + 4 * 2 * KS * 64;
+        mp.rot = (const float2v*)(mp.tabET + 4 * 2 * KS * 64);
+        mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
+        mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
+        mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
+        mp.sm_log2e = sm_log2e;
+        const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
+        switch (KS) {
+          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, st); break;
+          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, st); break;
+          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, st); break;
+        }
+      }
+    } else {
+      size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
+      const bool paged = a.mid_layout == FA_MID_PAGED;
+      const void* fn = paged ? reinterpret_cast<const void*>(&decode_mid_kernel<E, true>)
+                             : reinterpret_cast<const void*>(&decode_mid_kernel<E, false>);
+      if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
+      }
+      dim3 grid(p.n_mid_split, a.Hkv, a.B);
+      if (paged)
+        decode_mid_kernel<E, true><<<grid, 256, lds, st>>>(
+            (const E*)a.q, (const E*)a.k_mn, a.k_mn_batch_stride, 0, (const E*)a.v_mn, a.v_mn_batch_stride, 0,
+            a.mid_cap_pages, a.k_pad_h_list, a.v_pad_h_list, W, c0, a.kn_list, a.kn_h_list, a.vn_h_list, mm, md, mg,
+            mon, a.Hq, a.Hkv, a.D, a.N, a.L_m, a.T, p.n_mid_split, p.tiles_per_split, sm_log2e);
+      else
+        decode_mid_kernel<E, false><<<grid, 256, lds, st>>>(
+            (const E*)a.q, (const E*)a.k_mn, a.k_mn_batch_stride, a.k_mn_row_stride, (const E*)a.v_mn,
+            a.v_mn_batch_stride, a.v_mn_row_stride, 0, nullptr, nullptr, W, c0, a.kn_list, a.kn_h_list, a.vn_h_list,
+            mm, md, mg, mon, a.Hq, a.Hkv, a.D, a.N, a.L_m, a.T, p.n_mid_split, p.tiles_per_split, sm_log2e);
     }
-    decode_mid_kernel<E><<<dim3(p.n_mid_split, a.Hkv, a.B), 256, lds, st>>>(
-        (const E*)a.q, (const E*)a.k_mn, a.k_mn_batch_stride, a.k_mn_row_stride, (const E*)a.v_mn,
-        a.v_mn_batch_stride, a.v_mn_row_stride, W, c0, a.kn_list, a.kn_h_list, a.vn_h_list, mm, md, mg, mon, a.Hq,
-        a.Hkv, a.D, a.N, a.L_m, a.T, p.n_mid_split, p.tiles_per_split, sm_log2e);
   }
   if (p.n_il_split > 0) {
     Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
     Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
-    size_t lds = (2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
-    decode_il_kernel<E><<<dim3(p.n_il_split, a.Hkv, a.B), 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq,
-                                                                          a.Hkv, a.D, p.n_il_split, sm_log2e);
+    dim3 grid(p.n_il_split, a.Hkv, a.B);
+    if (il_fast_ok<E>(a)) {
+      if (a.D == 128)
+        decode_il_fast_kernel<E, 128><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+      else
+        decode_il_fast_kernel<E, 64><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+    } else {
+      size_t lds = (2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
+      decode_il_kernel<E><<<grid, 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, a.D, p.n_il_split, sm_log2e);
+    }
   }
   size_t lds = ((size_t)2 * a.N + a.D + 256 + p.n_il_split + p.n_mid_split) * sizeof(float);
   decode_merge_kernel<<<dim3(a.Hq, a.B), 256, lds, st>>>(ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split,
@@ -524,11 +784,35 @@ int launch_generic(const fa_decode_args& a, const Plan& p, float sm_scale, hipSt
   return fa_check_launch("fa_decode_attn");
 }
 
+bool use_mfma(const fa_decode_args& a) {
+  return a.L_m > 0 && !a.force_generic && mfma_shape_ok(a.Hq, a.Hkv, a.D, a.N, a.dtype, a.mid_layout) &&
+         a.Hq / a.Hkv <= kGMax && a.mid_max_k_pad <= 128 && a.mid_max_v_pad <= 128;
+}
+
 }  // namespace
 
 extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || N < 0 || il_rows_total < 0 || L_m < 0) return 0;
-  return make_plan(B, Hq, Hkv, D, N > 0 ? N : 1, il_rows_total, L_m).total;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || N < 0 || il_rows_total < 0 || L_m < 0 || Hq % Hkv) return 0;
+  const int n = N > 0 ? N : 1;
+  // large enough for either path
+  size_t a = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, false).total;
+  if (mfma_shape_ok(Hq, Hkv, D, n, FA_BF16, FA_MID_PAGED)) {
+    size_t b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, true).total;
+    if (b > a) a = b;
+  }
+  return a;
+}
+
+extern "C" size_t fa_decode_tables_bytes(int N) { return (N > 0 && N % 64 == 0) ? fa_mfma::tables_bytes(N) : 0; }
+
+extern "C" int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_stream_t stream) {
+  FA_REQUIRE(tables, FA_ERR_NULL_POINTER, "fa_decode_tables_build: null pointer");
+  FA_REQUIRE(N > 0 && N % 64 == 0 && T > 0, FA_ERR_BAD_SHAPE, "fa_decode_tables_build: N=%d T=%d", N, T);
+  FA_REQUIRE(tables_bytes >= fa_mfma::tables_bytes(N), FA_ERR_WORKSPACE, "fa_decode_tables_build: %zu < %zu bytes",
+             tables_bytes, fa_mfma::tables_bytes(N));
+  FA_REQUIRE(((uintptr_t)tables & 15) == 0, FA_ERR_MISALIGNED, "fa_decode_tables_build: tables not 16-byte aligned");
+  launch_tables(tables, N, T, fa_hip_stream(stream));
+  return fa_check_launch("fa_decode_tables_build");
 }
 
 extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
@@ -559,16 +843,28 @@ extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
                    (a->Cv == 0 || (a->v_mc && a->avg_v_u && a->avg_v_d && a->scale_v)),
                FA_ERR_NULL_POINTER, "fa_decode_attn: coefficient/statistics pointer null");
     FA_REQUIRE((a->Cnk == 0 || a->k_mn) && (a->Cnv == 0 || a->v_mn), FA_ERR_NULL_POINTER, "fa_decode_attn: k_mn/v_mn null");
+    FA_REQUIRE(a->mid_layout == FA_MID_TOKEN_MAJOR || a->mid_layout == FA_MID_PAGED, FA_ERR_BAD_SHAPE,
+               "fa_decode_attn: mid_layout %d", a->mid_layout);
+    if (a->mid_layout == FA_MID_PAGED) {
+      FA_REQUIRE(a->k_pad_h_list && a->v_pad_h_list, FA_ERR_NULL_POINTER, "fa_decode_attn: padded offset list null");
+      FA_REQUIRE((int64_t)a->mid_cap_pages * FA_PAGE_TOKENS >= a->L_m, FA_ERR_BAD_SHAPE,
+                 "fa_decode_attn: %d mid rows beyond %d pages", a->L_m, a->mid_cap_pages);
+      FA_REQUIRE(a->k_mn && a->v_mn, FA_ERR_NULL_POINTER, "fa_decode_attn: paged store null");
+      FA_REQUIRE((((uintptr_t)a->k_mn | (uintptr_t)a->v_mn) & 15) == 0 && (a->k_mn_batch_stride & 7) == 0 &&
+                     (a->v_mn_batch_stride & 7) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: paged store not 16-byte aligned");
+    }
   }
-  const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m);
+  const bool mfma = use_mfma(*a);
+  const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma);
   FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
              a->workspace_bytes, p.total);
   FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");
+  FA_REQUIRE(!a->tables || ((uintptr_t)a->tables & 15) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: tables not 16-byte aligned");
   const float sm = a->sm_scale > 0.f ? a->sm_scale : 1.0f / sqrtf((float)a->D);
   hipStream_t st = fa_hip_stream(stream);
   switch (a->dtype) {
-    case FA_BF16: return launch_generic<bf16_t>(*a, p, sm, st);
-    case FA_FP16: return launch_generic<f16_t>(*a, p, sm, st);
-    default: return launch_generic<float>(*a, p, sm, st);
+    case FA_BF16: return launch_all<bf16_t>(*a, p, sm, st);
+    case FA_FP16: return launch_all<f16_t>(*a, p, sm, st);
+    default: return launch_all<float>(*a, p, sm, st);
   }
 }

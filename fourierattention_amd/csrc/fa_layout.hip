@@ -1,0 +1,138 @@
+// Page layout of the stored mid dims: pack (prefill), append (eviction) and unpack.
+#include "fa_common.h"
+
+namespace {
+
+// element offset inside one (batch, head) run of pages
+__device__ __forceinline__ int64_t page_elem_offset(bool is_v, int dp, int64_t token, int j) {
+  const int64_t page = token >> 5;
+  const int t = (int)(token & 31);
+  int frag, lane, e;
+  if (!is_v) {
+    frag = (t >> 4) * (dp >> 5) + (j >> 5);
+    lane = ((j & 31) >> 3) * 16 + (t & 15);
+    e = j & 7;
+  } else {
+    frag = j >> 4;
+    lane = (t >> 3) * 16 + (j & 15);
+    e = t & 7;
+  }
+  return page * dp * 32 + (int64_t)frag * 512 + lane * 8 + e;
+}
+
+// one thread per (token, padded dim) of one (b, h): grid (ceil(L*dp/256), Hkv, B)
+template <typename E>
+__global__ __launch_bounds__(256) void mid_pack_kernel(
+    const E* __restrict__ src, int64_t src_bs, int64_t src_rs, int64_t row0, int L, E* __restrict__ store,
+    int64_t st_bs, int cap_pages, const int32_t* __restrict__ n_list, const int32_t* __restrict__ n_h,
+    const int32_t* __restrict__ pad_h, int is_v) {
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int n0 = n_h[h], n_len = n_h[h + 1] - n0;
+  const int p0 = pad_h[h], dp = pad_h[h + 1] - p0;
+  if (n_len == 0) return;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)L * n_len) return;
+  const int64_t token = idx / n_len;
+  const int j = (int)(idx % n_len);
+  const E v = src[(int64_t)b * src_bs + (row0 + token) * src_rs + n_list[n0 + j]];
+  store[(int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + page_elem_offset(is_v, dp, token, j)] = v;
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void mid_append_kernel(
+    const E* __restrict__ row, int64_t row_bs, int64_t pos, E* __restrict__ store, int64_t st_bs, int cap_pages,
+    const int32_t* __restrict__ n_list, const int32_t* __restrict__ n_h, const int32_t* __restrict__ pad_h, int Hkv,
+    int Cn, int is_v) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= Cn) return;
+  int h = 0;
+  while (h + 1 < Hkv && n_h[h + 1] <= c) ++h;
+  const int j = c - n_h[h];
+  const int p0 = pad_h[h], dp = pad_h[h + 1] - p0;
+  store[(int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + page_elem_offset(is_v, dp, pos, j)] =
+      row[(int64_t)b * row_bs + n_list[c]];
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void mid_unpack_kernel(
+    const E* __restrict__ store, int64_t st_bs, int cap_pages, int L, E* __restrict__ dst,
+    const int32_t* __restrict__ n_h, const int32_t* __restrict__ pad_h, int Cn, int is_v) {
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int n0 = n_h[h], n_len = n_h[h + 1] - n0;
+  const int p0 = pad_h[h], dp = pad_h[h + 1] - p0;
+  if (n_len == 0) return;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)L * n_len) return;
+  const int64_t token = idx / n_len;
+  const int j = (int)(idx % n_len);
+  dst[((int64_t)b * L + token) * Cn + n0 + j] =
+      store[(int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + page_elem_offset(is_v, dp, token, j)];
+}
+
+template <typename F>
+int dispatch16(int dtype, const char* what, F&& f) {
+  switch (dtype) {
+    case FA_BF16: f(bf16_t{}); return FA_OK;
+    case FA_FP16: f(f16_t{}); return FA_OK;
+    case FA_FP32: f(float{}); return FA_OK;
+    default: fa_set_error("%s: dtype %d", what, dtype); return FA_ERR_BAD_DTYPE;
+  }
+}
+
+}  // namespace
+
+extern "C" int fa_mid_pack(const void* src, int dtype, int64_t src_bs, int64_t src_rs, int64_t row0, int L,
+                           void* store, int64_t st_bs, int cap_pages, const int32_t* n_list, const int32_t* n_h,
+                           const int32_t* pad_h, int B, int Hkv, int D, int is_v, fa_stream_t stream) {
+  FA_REQUIRE(src && store && n_h && pad_h, FA_ERR_NULL_POINTER, "fa_mid_pack: null pointer");
+  FA_REQUIRE(B > 0 && Hkv > 0 && L >= 0 && cap_pages > 0 && row0 >= 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: bad shape");
+  FA_REQUIRE((int64_t)cap_pages * 32 >= L, FA_ERR_BAD_SHAPE, "fa_mid_pack: %d rows do not fit %d pages", L, cap_pages);
+  if (L == 0) return FA_OK;
+  hipStream_t st = fa_hip_stream(stream);
+  FA_REQUIRE(D > 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: head_dim %d", D);
+  dim3 grid(fa_cdiv((int64_t)L * D, 256), Hkv, B);  // a head stores at most D dims
+  int rc = dispatch16(dtype, "fa_mid_pack", [&](auto tag) {
+    using E = decltype(tag);
+    mid_pack_kernel<E><<<grid, 256, 0, st>>>((const E*)src, src_bs, src_rs, row0, L, (E*)store, st_bs, cap_pages, n_list,
+                                            n_h, pad_h, is_v);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_mid_pack");
+}
+
+extern "C" int fa_mid_append(const void* row, int dtype, int64_t row_bs, int64_t pos, void* store, int64_t st_bs,
+                             int cap_pages, const int32_t* n_list, const int32_t* n_h, const int32_t* pad_h, int B,
+                             int Hkv, int Cn, int is_v, fa_stream_t stream) {
+  FA_REQUIRE(row && store && n_h && pad_h, FA_ERR_NULL_POINTER, "fa_mid_append: null pointer");
+  FA_REQUIRE(B > 0 && Hkv > 0 && Cn >= 0 && pos >= 0 && cap_pages > 0, FA_ERR_BAD_SHAPE, "fa_mid_append: bad shape");
+  FA_REQUIRE(pos < (int64_t)cap_pages * 32, FA_ERR_BAD_SHAPE, "fa_mid_append: position %lld beyond %d pages",
+             (long long)pos, cap_pages);
+  if (Cn == 0) return FA_OK;
+  FA_REQUIRE(n_list, FA_ERR_NULL_POINTER, "fa_mid_append: index list null");
+  hipStream_t st = fa_hip_stream(stream);
+  dim3 grid(fa_cdiv(Cn, 256), B);
+  int rc = dispatch16(dtype, "fa_mid_append", [&](auto tag) {
+    using E = decltype(tag);
+    mid_append_kernel<E><<<grid, 256, 0, st>>>((const E*)row, row_bs, pos, (E*)store, st_bs, cap_pages, n_list, n_h, pad_h,
+                                              Hkv, Cn, is_v);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_mid_append");
+}
+
+extern "C" int fa_mid_unpack(const void* store, int dtype, int64_t st_bs, int cap_pages, int L, void* dst,
+                             const int32_t* n_h, const int32_t* pad_h, int B, int Hkv, int D, int Cn, int is_v,
+                             fa_stream_t stream) {
+  FA_REQUIRE(store && n_h && pad_h, FA_ERR_NULL_POINTER, "fa_mid_unpack: null pointer");
+  FA_REQUIRE(B > 0 && Hkv > 0 && L >= 0 && Cn >= 0 && cap_pages > 0, FA_ERR_BAD_SHAPE, "fa_mid_unpack: bad shape");
+  FA_REQUIRE((int64_t)cap_pages * 32 >= L, FA_ERR_BAD_SHAPE, "fa_mid_unpack: %d rows beyond %d pages", L, cap_pages);
+  if (L == 0 || Cn == 0) return FA_OK;
+  FA_REQUIRE(dst, FA_ERR_NULL_POINTER, "fa_mid_unpack: dst null");
+  FA_REQUIRE(D > 0, FA_ERR_BAD_SHAPE, "fa_mid_unpack: head_dim %d", D);
+  hipStream_t st = fa_hip_stream(stream);
+  dim3 grid(fa_cdiv((int64_t)L * D, 256), Hkv, B);
+  int rc = dispatch16(dtype, "fa_mid_unpack", [&](auto tag) {
+    using E = decltype(tag);
+    mid_unpack_kernel<E><<<grid, 256, 0, st>>>((const E*)store, st_bs, cap_pages, L, (E*)dst, n_h, pad_h, Cn, is_v);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_mid_unpack");
+}

@@ -198,13 +198,27 @@ class MultiDimHiPPO2(torch.nn.Module):
 
 
 # ------------------------------------------------------------------ decode attention
+def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
+    """Constant operand tables of the MFMA decode path for ``(N, T)``; ``None`` when that path
+    does not cover ``N`` (the call then takes the generic kernels)."""
+    lib = _lib.load()
+    nbytes = lib.fa_decode_tables_bytes(int(n_f))
+    if nbytes == 0 or n_f not in (128, 256, 512):
+        return None
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    check(lib.fa_decode_tables_build(buf.data_ptr(), nbytes, int(n_f), int(period), _stream(torch.device(device))))
+    return buf
+
+
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
-                    T, sm_scale=-1.0, out=None):
+                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False):
     """Thin call into ``fa_decode_attn``.
 
     ``il_segments``: up to two ``(k, v)`` pairs of ``(B, rows, Hkv*D)`` views (last dim contiguous).
+    ``k_mn`` / ``v_mn``: token-major ``(B, >=L_m, Cn)`` tensors or ``MidStore`` objects (paged).
     ``stats_*``: ``(avg_u, avg_d, scale)`` fp32 ``(B, C)``.  ``lists``: the eight int32 tensors
     ``kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h`` (``*_h`` with the leading 0)."""
+    from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
     D = feat // num_head_q
@@ -227,16 +241,28 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
         N = (k_mc.shape[1] if a.Ck else v_mc.shape[1]) // 2
         for t in (k_mc, v_mc):
             assert t.dtype == torch.float32 and t.is_contiguous()
-        for t in (k_mn, v_mn):
-            assert t.stride(2) == 1 and t.dtype == q.dtype
         a.k_mc, a.v_mc = _ptr(k_mc), _ptr(v_mc)
-        a.k_mn, a.v_mn = _ptr(k_mn), _ptr(v_mn)
-        a.k_mn_batch_stride, a.k_mn_row_stride = k_mn.stride(0), k_mn.stride(1)
-        a.v_mn_batch_stride, a.v_mn_row_stride = v_mn.stride(0), v_mn.stride(1)
+        if isinstance(k_mn, MidStore):
+            assert isinstance(v_mn, MidStore) and k_mn.dtype == q.dtype and k_mn.cap_pages == v_mn.cap_pages
+            a.mid_layout, a.mid_cap_pages = _lib.FA_MID_PAGED, k_mn.cap_pages
+            a.k_mn, a.v_mn = k_mn.data.data_ptr(), v_mn.data.data_ptr()
+            a.k_mn_batch_stride, a.v_mn_batch_stride = k_mn.batch_stride, v_mn.batch_stride
+            a.k_pad_h_list, a.v_pad_h_list = k_mn.pad_h32.data_ptr(), v_mn.pad_h32.data_ptr()
+            a.mid_max_k_pad, a.mid_max_v_pad = k_mn.max_pad, v_mn.max_pad
+        else:
+            for t in (k_mn, v_mn):
+                assert t.stride(2) == 1 and t.dtype == q.dtype
+            a.mid_layout = _lib.FA_MID_TOKEN_MAJOR
+            a.k_mn, a.v_mn = _ptr(k_mn), _ptr(v_mn)
+            a.k_mn_batch_stride, a.k_mn_row_stride = k_mn.stride(0), k_mn.stride(1)
+            a.v_mn_batch_stride, a.v_mn_row_stride = v_mn.stride(0), v_mn.stride(1)
         a.avg_k_u, a.avg_k_d, a.scale_k = (_ptr(t) for t in stats_k)
         a.avg_v_u, a.avg_v_d, a.scale_v = (_ptr(t) for t in stats_v)
         for t in (*stats_k, *stats_v):
             assert t.dtype == torch.float32 and t.is_contiguous()
+        if tables is not None:
+            a.tables = tables.data_ptr()
+    a.force_generic = int(bool(force_generic))
     a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()
     a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list = vc.data_ptr(), vc_h.data_ptr(), vn.data_ptr(), vn_h.data_ptr()
     if out is None:

@@ -117,12 +117,26 @@ typedef struct fa_decode_args {
   /* coefficients (B, 2N, Ck) / (B, 2N, Cv) fp32 contiguous (k_mc, v_mc) */
   const float* k_mc;
   const float* v_mc;
-  /* stored ("critical") dims of the mid rows, token-major (B, >=L_m, Cn):
-   * k_mn, v_mn with batch and row strides in elements */
+  /* stored ("critical") dims of the mid rows (k_mn, v_mn).
+   * mid_layout == FA_MID_TOKEN_MAJOR: (B, >=L_m, Cn) with batch and row strides
+   * in elements, as the reference holds k_uncompressed (CACHE:560, 735).
+   * mid_layout == FA_MID_PAGED: the library's own page layout written by
+   * fa_mid_pack / fa_mid_append (see there); row strides are ignored and
+   * mid_cap_pages, k_pad_h_list, v_pad_h_list describe the store. */
   const void* k_mn;
   const void* v_mn;
   int64_t k_mn_batch_stride, k_mn_row_stride;
   int64_t v_mn_batch_stride, v_mn_row_stride;
+  int32_t mid_layout;
+  int32_t mid_cap_pages;
+  const int32_t* k_pad_h_list;
+  const int32_t* v_pad_h_list;
+  int32_t mid_max_k_pad;   /* largest per-head padded dim count of K / V (host copies of */
+  int32_t mid_max_v_pad;   /* max_h(pad_h[h+1] - pad_h[h]); select the kernel instance)   */
+  /* optional constant operand tables built by fa_decode_tables_build for this (N, T);
+   * NULL lets the call build them in its workspace */
+  const void* tables;
+  int32_t force_generic;   /* != 0: never take the MFMA path (testing) */
   /* affine statistics, fp32 (B, Ck) / (B, Cv): avg_*_u, avg_*_d, scale_* */
   const float* avg_k_u; const float* avg_k_d; const float* scale_k;
   const float* avg_v_u; const float* avg_v_d; const float* scale_v;
@@ -152,6 +166,55 @@ typedef struct fa_decode_args {
 size_t fa_decode_args_size(void);
 
 size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m);
+
+/* ---------------------------------------------------------------------------
+ * Page layout of the stored mid dims (the cache's HBM layout; no counterpart in
+ * the reference, which keeps k_uncompressed token-major and grows it with
+ * torch.cat, CACHE:735, 741)
+ * ------------------------------------------------------------------------- */
+enum fa_mid_layout { FA_MID_TOKEN_MAJOR = 0, FA_MID_PAGED = 1 };
+#define FA_PAGE_TOKENS 32
+#define FA_K_DIM_PAD 32 /* per-head stored K dims are padded to a multiple of this */
+#define FA_V_DIM_PAD 16 /* per-head stored V dims are padded to a multiple of this */
+
+/* One tensor (K or V) of one layer is stored per (batch, KV head) as a run of
+ * pages of FA_PAGE_TOKENS tokens.  With pad_h_list the cumulative padded dim
+ * counts (Hkv + 1 int32, leading 0; head h owns dp = pad_h[h+1] - pad_h[h]
+ * padded dims), the page p of head h of batch b starts at element
+ *     b * batch_stride + pad_h[h] * 32 * cap_pages + p * dp * 32
+ * and holds dp * 32 elements in fragments of 512 elements (64 lanes x 8):
+ *   K: fragment (tb, s), tb in {0,1}, s < dp/32, at index tb * (dp/32) + s;
+ *      lane l, element e = token p*32 + tb*16 + l%16, stored dim s*32 + 8*(l/16) + e
+ *   V: fragment dg < dp/16;
+ *      lane l, element e = stored dim dg*16 + l%16, token p*32 + 8*(l/16) + e
+ * i.e. exactly the register image of a 16x16x32 MFMA A operand, so a wave
+ * loads a fragment with one 16-byte load per lane.  Padded dims and unused
+ * token slots must be zero: allocate the store zero-filled.
+ * batch_stride >= pad_h[Hkv] * 32 * cap_pages. */
+
+/* Scatter rows [row0, row0 + L) of src (B, S, Hkv*D), taking for each head the
+ * columns n_list[n_h[h] .. n_h[h+1]) (the gather x[:, :, kn] of CACHE:560, 578),
+ * into pages starting at token 0.  is_v selects the V fragment order. */
+int fa_mid_pack(const void* src, int dtype, int64_t src_batch_stride, int64_t src_row_stride, int64_t row0,
+                int L, void* store, int64_t store_batch_stride, int cap_pages, const int32_t* n_list,
+                const int32_t* n_h_list, const int32_t* pad_h_list, int B, int Hkv, int D, int is_v,
+                fa_stream_t stream);
+
+/* Write one row (the evicted window row, CACHE:735, 741) at token position pos. */
+int fa_mid_append(const void* row, int dtype, int64_t row_batch_stride, int64_t pos, void* store,
+                  int64_t store_batch_stride, int cap_pages, const int32_t* n_list, const int32_t* n_h_list,
+                  const int32_t* pad_h_list, int B, int Hkv, int Cn, int is_v, fa_stream_t stream);
+
+/* Inverse of fa_mid_pack: dst (B, L, Cn) token-major contiguous, the reference's
+ * k_uncompressed / v_uncompressed. */
+int fa_mid_unpack(const void* store, int dtype, int64_t store_batch_stride, int cap_pages, int L, void* dst,
+                  const int32_t* n_h_list, const int32_t* pad_h_list, int B, int Hkv, int D, int Cn, int is_v,
+                  fa_stream_t stream);
+
+/* Constant MFMA operand tables of decode attention (cos/sin of in-page token offsets and
+ * the per-page rotation); they depend on N and T only, so a cache builds them once. */
+size_t fa_decode_tables_bytes(int N);
+int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_stream_t stream);
 
 /* One decode step of Fourier attention over
  * [sink ; local window ; mid rows (stored dims + dims rebuilt from coefficients)]. */
