@@ -8,6 +8,8 @@
 // so one pass over the coefficients before (prep) and one after (merge) replace the
 // per-token reconstruction, and the token loop only touches the stored dims.
 // All exponentials are base 2 (scores carry log2(e)).
+#include <stdlib.h>
+
 #include "fa_common.h"
 #include "fa_decode_mfma.h"
 
@@ -387,9 +389,11 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// merge: one block per (b, hq)
+// merge: one block of 1024 threads per (b, KV head) combines, for the G query heads of that head,
+// the partials of every split and applies the V coefficients once:
+//   out_c = s_v * ((1/N) V_coef^T g - avg_d_v * P) + avg_u_v * P
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void decode_merge_kernel(
+__global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
     const float* __restrict__ md_m, const float* __restrict__ md_d, const float* __restrict__ md_g,
     const float* __restrict__ md_on, int n_mid_split, const float* __restrict__ v_mc,
@@ -397,67 +401,103 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(
     const int32_t* __restrict__ vc_list, const int32_t* __restrict__ vc_h, const int32_t* __restrict__ vn_list,
     const int32_t* __restrict__ vn_h, float* __restrict__ out, int Hq, int Hkv, int D, int N, int Cv) {
   extern __shared__ float smem[];
-  float* s_g = smem;              // [2N]
-  float* s_o = s_g + 2 * N;       // [D]
-  float* s_part = s_o + D;        // [2][128]
-  float* s_w = s_part + 256;      // [n_il_split + n_mid_split]
-  const int tid = threadIdx.x;
-  const int hq = blockIdx.x, b = blockIdx.y;
-  const int G = Hq / Hkv, h = hq / G;
-  const int64_t r = (int64_t)b * Hq + hq;
+  const int G = Hq / Hkv;
   const int n_all = n_il_split + n_mid_split;
+  float* s_g = smem;                     // [G][2N]
+  float* s_o = s_g + G * 2 * N;          // [G][D]
+  float* s_w = s_o + G * D;              // [G][n_all]
+  float* s_sc = s_w + G * n_all;         // [3][kGMax]: m*, sum of d, sum of d over the mid rows
+  float* s_part = s_sc + 3 * kGMax;      // [8][G][128]
+  const int tid = threadIdx.x;
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int64_t r0 = (int64_t)b * Hq + h * G;
 
-  float mstar = -INFINITY;
-  for (int s = 0; s < n_il_split; ++s) mstar = fmaxf(mstar, il_m[r * n_il_split + s]);
-  for (int s = 0; s < n_mid_split; ++s) mstar = fmaxf(mstar, md_m[r * n_mid_split + s]);
-  for (int s = tid; s < n_all; s += 256) {
-    float m = s < n_il_split ? il_m[r * n_il_split + s] : md_m[r * n_mid_split + (s - n_il_split)];
-    s_w[s] = (m == -INFINITY) ? 0.f : exp2f(m - mstar);
+  if (tid < G) {
+    const int64_t r = r0 + tid;
+    float mstar = -INFINITY;
+    for (int s = 0; s < n_il_split; ++s) mstar = fmaxf(mstar, il_m[r * n_il_split + s]);
+    for (int s = 0; s < n_mid_split; ++s) mstar = fmaxf(mstar, md_m[r * n_mid_split + s]);
+    float dsum = 0.f, pmid = 0.f;
+    for (int s = 0; s < n_il_split; ++s) {
+      const float m = il_m[r * n_il_split + s];
+      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+      s_w[tid * n_all + s] = wgt;
+      dsum += wgt * il_d[r * n_il_split + s];
+    }
+    for (int s = 0; s < n_mid_split; ++s) {
+      const float m = md_m[r * n_mid_split + s];
+      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+      s_w[tid * n_all + n_il_split + s] = wgt;
+      pmid += wgt * md_d[r * n_mid_split + s];
+    }
+    s_sc[tid] = mstar;
+    s_sc[kGMax + tid] = dsum + pmid;
+    s_sc[2 * kGMax + tid] = pmid;
   }
-  for (int d = tid; d < D; d += 256) s_o[d] = 0.f;
+  for (int idx = tid; idx < G * D; idx += 1024) s_o[idx] = 0.f;
   __syncthreads();
-  float dsum = 0.f, pmid = 0.f;
-  for (int s = 0; s < n_il_split; ++s) dsum += s_w[s] * il_d[r * n_il_split + s];
-  for (int s = 0; s < n_mid_split; ++s) pmid += s_w[n_il_split + s] * md_d[r * n_mid_split + s];
-  dsum += pmid;
 
-  for (int n = tid; n < 2 * N; n += 256) {
+  // g summed over the splits
+  for (int idx = tid; idx < G * 2 * N; idx += 1024) {
+    const int g = idx / (2 * N), n = idx - g * 2 * N;
+    const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + n;
     float a = 0.f;
-    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[n_il_split + s], md_g[(r * n_mid_split + s) * 2 * N + n], a);
-    s_g[n] = a;
+    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[g * n_all + n_il_split + s], gp[(int64_t)s * 2 * N], a);
+    s_g[idx] = a;
   }
   __syncthreads();
 
-  // stored dims of V
-  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
-  for (int j = tid; j < vn_len; j += 256) {
-    float a = 0.f;
-    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[n_il_split + s], md_on[(r * n_mid_split + s) * D + j], a);
-    s_o[vn_list[vn0 + j] - h * D] = a;
-  }
-  // compressed dims of V: g . V_coef
+  // compressed dims: g . V_coef, thread = (dim j, one of 8 row classes)
   const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
+  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
   {
-    const int j = tid % 128, part = tid / 128;
-    float a = 0.f;
+    const int j = tid & 127, part = tid >> 7;
+    float acc[kGMax];
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
     if (j < vc_len && n_mid_split > 0) {
       const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + j;
-      for (int n = part; n < 2 * N; n += 2) a = fmaf(s_g[n], vp[(int64_t)n * Cv], a);
+      for (int n = part; n < 2 * N; n += 32) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = (n + 8 * u < 2 * N) ? vp[(int64_t)(n + 8 * u) * Cv] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int g = 0; g < kGMax; ++g)
+            if (g < G && n + 8 * u < 2 * N) acc[g] = fmaf(s_g[g * 2 * N + n + 8 * u], v[u], acc[g]);
+      }
     }
-    s_part[part * 128 + j] = a;
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) s_part[(part * G + g) * 128 + j] = acc[g];
   }
   __syncthreads();
-  for (int j = tid; j < vc_len; j += 256) {
-    float a = (s_part[j] + s_part[128 + j]) / (float)N;
-    int64_t o = (int64_t)b * Cv + vc0 + j;
-    float v = n_mid_split > 0 ? scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid : 0.f;
-    s_o[vc_list[vc0 + j] - h * D] = v;
+  for (int idx = tid; idx < G * vc_len; idx += 1024) {
+    const int g = idx / vc_len, j = idx - g * vc_len;
+    float a = 0.f;
+#pragma unroll
+    for (int part = 0; part < 8; ++part) a += s_part[(part * G + g) * 128 + j];
+    a /= (float)N;
+    const int64_t o = (int64_t)b * Cv + vc0 + j;
+    const float pmid = s_sc[2 * kGMax + g];
+    s_o[g * D + (vc_list[vc0 + j] - h * D)] = n_mid_split > 0 ? scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid : 0.f;
+  }
+  // stored dims
+  for (int idx = tid; idx < G * vn_len; idx += 1024) {
+    const int g = idx / vn_len, j = idx - g * vn_len;
+    const float* op = md_on + (r0 + g) * n_mid_split * D + j;
+    float a = 0.f;
+    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[g * n_all + n_il_split + s], op[(int64_t)s * D], a);
+    s_o[g * D + (vn_list[vn0 + j] - h * D)] = a;
   }
   __syncthreads();
-  for (int d = tid; d < D; d += 256) {
-    float a = s_o[d];
-    for (int s = 0; s < n_il_split; ++s) a = fmaf(s_w[s], il_o[(r * n_il_split + s) * D + d], a);
-    out[r * D + d] = a / dsum;
+  for (int idx = tid; idx < G * D; idx += 1024) {
+    const int g = idx / D, d = idx - g * D;
+    const float* op = il_o + (r0 + g) * n_il_split * D + d;
+    float a = s_o[idx];
+    for (int s = 0; s < n_il_split; ++s) a = fmaf(s_w[g * n_all + s], op[(int64_t)s * D], a);
+    out[(r0 + g) * D + d] = a / s_sc[kGMax + g];
   }
 }
 
@@ -680,9 +720,9 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
   using namespace fa_mfma;
   const int KS = N / 64;
   half8* tabE = (half8*)tables;
-  half8* tabET = tabE + 4 * 2 * KS * 64;
-  float2v* rot = (float2v*)(tabET + 4 * 2 * KS * 64);
-  const int total = 2 * 4 * 2 * KS * 64 + N;
+  half8* tabET = tabE + kFreqWaves * 2 * KS * 64;
+  float2v* rot = (float2v*)(tabET + kFreqWaves * 2 * KS * 64);
+  const int total = 2 * kFreqWaves * 2 * KS * 64 + N;
   decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N);
 }
 
@@ -690,9 +730,9 @@ template <typename E, int KS>
 void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
   dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
   if (wide)
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8><<<grid, 256, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8><<<grid, 512, 0, st>>>(mp);
   else
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4><<<grid, 256, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4><<<grid, 512, 0, st>>>(mp);
 }
 
 template <typename E>
@@ -727,12 +767,16 @@ int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream
         mp.kn_list = a.kn_list; mp.kn_h = a.kn_h_list; mp.kpad_h = a.k_pad_h_list;
         mp.vn_h = a.vn_h_list; mp.vpad_h = a.v_pad_h_list;
         mp.tabE = (const half8*)tables;
-        mp.tabET = mp.tabE + 4 * 2 * KS * 64;
-        mp.rot = (const float2v*)(mp.tabET + 4 * 2 * KS * 64);
+        mp.tabET = mp.tabE + kFreqWaves * 2 * KS * 64;
+        mp.rot = (const float2v*)(mp.tabET + kFreqWaves * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
         mp.sm_log2e = sm_log2e;
+        {
+          static const int dbg = getenv("FA_DEBUG_FLAGS") ? atoi(getenv("FA_DEBUG_FLAGS")) : 0;
+          mp.dbg = dbg;
+        }
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
         switch (KS) {
           case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, st); break;
@@ -776,11 +820,19 @@ int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream
       decode_il_kernel<E><<<grid, 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, a.D, p.n_il_split, sm_log2e);
     }
   }
-  size_t lds = ((size_t)2 * a.N + a.D + 256 + p.n_il_split + p.n_mid_split) * sizeof(float);
-  decode_merge_kernel<<<dim3(a.Hq, a.B), 256, lds, st>>>(ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split,
-                                                         a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v, a.vc_list,
-                                                         a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D,
-                                                         a.N, a.Cv);
+  {
+    size_t lds = ((size_t)G * 2 * a.N + (size_t)G * a.D + (size_t)G * (p.n_il_split + p.n_mid_split) + 3 * kGMax +
+                  8 * (size_t)G * 128) * sizeof(float);
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_merge_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
+    }
+    decode_merge_kernel<<<dim3(a.Hkv, a.B), 1024, lds, st>>>(ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split,
+                                                             a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v, a.vc_list,
+                                                             a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv,
+                                                             a.D, a.N, a.Cv);
+  }
   return fa_check_launch("fa_decode_attn");
 }
 
