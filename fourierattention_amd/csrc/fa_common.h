@@ -74,3 +74,60 @@ __device__ __forceinline__ float fa_wave_min(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, FA_WAVE));
   return v;
 }
+
+// ---- cross-lane helpers without LDS traffic -----------------------------------
+template <int CTRL>
+__device__ __forceinline__ float fa_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// butterfly partners inside a 16-lane row: xor 1, xor 2, (7 - i within 8 lanes), (15 - i), rotate by 8
+#define FA_DPP_XOR1 0xB1
+#define FA_DPP_XOR2 0x4E
+#define FA_DPP_HALF_MIRROR 0x141
+#define FA_DPP_MIRROR 0x140
+#define FA_DPP_ROR8 0x128
+
+// sum over the LANES consecutive lanes (4, 8 or 16, aligned) that contain this lane; every lane gets it
+template <int LANES>
+__device__ __forceinline__ float fa_group_sum(float v) {
+  v += fa_dpp<FA_DPP_XOR1>(v);
+  v += fa_dpp<FA_DPP_XOR2>(v);
+  if (LANES >= 8) v += fa_dpp<FA_DPP_HALF_MIRROR>(v);
+  if (LANES >= 16) v += fa_dpp<FA_DPP_MIRROR>(v);
+  return v;
+}
+
+// partner values across the four 16-lane rows of a wave (lane i, i+16, i+32, i+48):
+// one v_permlane16_swap / v_permlane32_swap each (gfx950); the two operands must sit in
+// different registers, which the empty asm enforces
+__device__ __forceinline__ void fa_swap16(float x, float* lo, float* hi) {
+  unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+  asm volatile("" : "+v"(b));
+  auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+  const unsigned r0 = r[0], r1 = r[1];  // scalars first: bit_cast of a vector element reads element 0
+  *lo = __builtin_bit_cast(float, r0);
+  *hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ void fa_swap32(float x, float* lo, float* hi) {
+  unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+  asm volatile("" : "+v"(b));
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  const unsigned r0 = r[0], r1 = r[1];  // scalars first: bit_cast of a vector element reads element 0
+  *lo = __builtin_bit_cast(float, r0);
+  *hi = __builtin_bit_cast(float, r1);
+}
+// max / sum over the four lanes that share (lane % 16); every lane gets the result
+__device__ __forceinline__ float fa_rows_max(float x) {
+  float a, b;
+  fa_swap16(x, &a, &b);
+  x = fmaxf(a, b);
+  fa_swap32(x, &a, &b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float fa_rows_sum(float x) {
+  float a, b;
+  fa_swap16(x, &a, &b);
+  x = a + b;
+  fa_swap32(x, &a, &b);
+  return a + b;
+}

@@ -30,57 +30,64 @@ struct Seg {
 // ---------------------------------------------------------------------------
 // prep: W[b, hq, n] = (sm*log2e/N) sum_j coef[b, n, kc0 + j] q[b, hq, d_j] s[b, kc0 + j]
 //       c0[b, hq]   = sm*log2e * sum_j q[b, hq, d_j] (avg_u - avg_d s)[b, kc0 + j]
+// block = 64 coefficient rows of one (b, KV head); thread = (row, one of 4 column classes):
+// a thread reads every 4th compressed dim of its row (up to 32 independent loads in flight),
+// four neighbouring lanes finish the dot product.  Block x == 0 also clears the merge tickets.
 // ---------------------------------------------------------------------------
+constexpr int kPrepRows = 64;
+
 template <typename E>
 __global__ __launch_bounds__(256) void decode_prep_kernel(
     const E* __restrict__ q, const float* __restrict__ k_mc, const float* __restrict__ avg_u,
     const float* __restrict__ avg_d, const float* __restrict__ scale, const int32_t* __restrict__ kc_list,
-    const int32_t* __restrict__ kc_h, float* __restrict__ W, float* __restrict__ c0, int Hq, int Hkv, int D,
-    int N, int Ck, float sm_log2e, int rows_per_block) {
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int32_t* __restrict__ kc_h, float* __restrict__ W, float* __restrict__ c0, unsigned* __restrict__ tickets,
+    int Hq, int Hkv, int D, int N, int Ck, float sm_log2e) {
+  __shared__ float s_qs[kGMax][128];
+  __shared__ float s_qa[kGMax][128];
+  const int tid = threadIdx.x;
   const int h = blockIdx.y, b = blockIdx.z;
   const int G = Hq / Hkv;
   const int kc0 = kc_h[h], kc_len = kc_h[h + 1] - kc0;
-  float qs[kGMax][2], qa[kGMax][2];
-#pragma unroll
-  for (int g = 0; g < kGMax; ++g) qs[g][0] = qs[g][1] = qa[g][0] = qa[g][1] = 0.f;
-#pragma unroll
-  for (int jj = 0; jj < 2; ++jj) {
-    int j = lane + 64 * jj;
-    if (j < kc_len) {
-      int d = kc_list[kc0 + j] - h * D;
-      float s = scale[(int64_t)b * Ck + kc0 + j];
-      float a = avg_u[(int64_t)b * Ck + kc0 + j] - avg_d[(int64_t)b * Ck + kc0 + j] * s;
-#pragma unroll
-      for (int g = 0; g < kGMax; ++g)
-        if (g < G) {
-          float qv = fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + d]);
-          qs[g][jj] = qv * s;
-          qa[g][jj] = qv * a;
-        }
+  if (blockIdx.x == 0 && tid == 0) tickets[b * Hkv + h] = 0u;
+  for (int e = tid; e < kGMax * 128; e += 256) {
+    const int g = e >> 7, j = e & 127;
+    float qs = 0.f, qa = 0.f;
+    if (g < G && j < kc_len) {
+      const int d = kc_list[kc0 + j] - h * D;
+      const float sc = scale[(int64_t)b * Ck + kc0 + j];
+      const float a = avg_u[(int64_t)b * Ck + kc0 + j] - avg_d[(int64_t)b * Ck + kc0 + j] * sc;
+      const float qv = fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + d]);
+      qs = qv * sc;
+      qa = qv * a;
+    }
+    s_qs[g][j] = qs;
+    s_qa[g][j] = qa;
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && tid < 64) {
+    for (int g = 0; g < G; ++g) {
+      float v = fa_wave_sum(s_qa[g][tid] + s_qa[g][tid + 64]);
+      if (tid == 0) c0[(int64_t)b * Hq + h * G + g] = v * sm_log2e;
     }
   }
-  if (blockIdx.x == 0 && w == 0) {
+  const int n = blockIdx.x * kPrepRows + (tid >> 2), jq = tid & 3;
+  if (n >= 2 * N) return;
+  const float* row = k_mc + ((int64_t)b * 2 * N + n) * Ck + kc0;
+  float v[32];
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g)
-      if (g < G) {
-        float v = fa_wave_sum(qa[g][0] + qa[g][1]);
-        if (lane == 0) c0[(int64_t)b * Hq + h * G + g] = v * sm_log2e;
-      }
+  for (int i = 0; i < 32; ++i) {
+    const int j = jq + 4 * i;
+    v[i] = j < kc_len ? row[j] : 0.f;
   }
   const float mul = sm_log2e / (float)N;
-  const int n_beg = blockIdx.x * rows_per_block;
-  const int n_end = min(2 * N, n_beg + rows_per_block);
-  for (int n = n_beg + w; n < n_end; n += 4) {
-    const float* row = k_mc + ((int64_t)b * 2 * N + n) * Ck + kc0;
-    float v0 = lane < kc_len ? row[lane] : 0.f;
-    float v1 = lane + 64 < kc_len ? row[lane + 64] : 0.f;
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g)
-      if (g < G) {
-        float v = fa_wave_sum(v0 * qs[g][0] + v1 * qs[g][1]);
-        if (lane == 0) W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = v * mul;
-      }
+  for (int g = 0; g < kGMax; ++g) {
+    if (g >= G) break;
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) a = fmaf(v[i], s_qs[g][jq + 4 * i], a);
+    a = fa_group_sum<4>(a);
+    if (jq == 0) W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = a * mul;
   }
 }
 
@@ -392,7 +399,22 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
 // merge: one block of 1024 threads per (b, KV head) combines, for the G query heads of that head,
 // the partials of every split and applies the V coefficients once:
 //   out_c = s_v * ((1/N) V_coef^T g - avg_d_v * P) + avg_u_v * P
+// Every phase issues its global loads in batches of 16 per thread before using them.
 // ---------------------------------------------------------------------------
+// sum_s w[s] * ptr[s * stride] with the loads issued sixteen at a time
+__device__ __forceinline__ float weighted_sum(const float* __restrict__ ptr, int64_t stride, const float* w, int n) {
+  float a = 0.f;
+  for (int s0 = 0; s0 < n; s0 += 16) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = (s0 + u < n) ? ptr[(int64_t)(s0 + u) * stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (s0 + u < n) a = fmaf(w[s0 + u], v[u], a);
+  }
+  return a;
+}
+
 __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
     const float* __restrict__ md_m, const float* __restrict__ md_d, const float* __restrict__ md_g,
@@ -404,113 +426,114 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   const int G = Hq / Hkv;
   const int n_all = n_il_split + n_mid_split;
   float* s_g = smem;                     // [G][2N]
-  float* s_o = s_g + G * 2 * N;          // [G][D]
-  float* s_w = s_o + G * D;              // [G][n_all]
-  float* s_sc = s_w + G * n_all;         // [3][kGMax]: m*, sum of d, sum of d over the mid rows
-  float* s_part = s_sc + 3 * kGMax;      // [8][G][128]
+  float* s_w = s_g + G * 2 * N;          // [G][n_all]
+  float* s_d = s_w + G * n_all;          // [G][n_all]
+  float* s_sc = s_d + G * n_all;         // [2][kGMax]: sum of d, sum of d over the mid rows
+  float* s_part = s_sc + 2 * kGMax;      // [16][G][128]
+  float* s_o = s_part + 16 * G * 128;    // [G][D]
   const int tid = threadIdx.x;
   const int h = blockIdx.x, b = blockIdx.y;
   const int64_t r0 = (int64_t)b * Hq + h * G;
+  const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
+  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
 
-  if (tid < G) {
-    const int64_t r = r0 + tid;
-    float mstar = -INFINITY;
-    for (int s = 0; s < n_il_split; ++s) mstar = fmaxf(mstar, il_m[r * n_il_split + s]);
-    for (int s = 0; s < n_mid_split; ++s) mstar = fmaxf(mstar, md_m[r * n_mid_split + s]);
-    float dsum = 0.f, pmid = 0.f;
-    for (int s = 0; s < n_il_split; ++s) {
-      const float m = il_m[r * n_il_split + s];
-      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
-      s_w[tid * n_all + s] = wgt;
-      dsum += wgt * il_d[r * n_il_split + s];
-    }
-    for (int s = 0; s < n_mid_split; ++s) {
-      const float m = md_m[r * n_mid_split + s];
-      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
-      s_w[tid * n_all + n_il_split + s] = wgt;
-      pmid += wgt * md_d[r * n_mid_split + s];
-    }
-    s_sc[tid] = mstar;
-    s_sc[kGMax + tid] = dsum + pmid;
-    s_sc[2 * kGMax + tid] = pmid;
+  for (int idx = tid; idx < G * n_all; idx += 1024) {
+    const int g = idx / n_all, s_ = idx - g * n_all;
+    const int64_t r = r0 + g;
+    const bool il = s_ < n_il_split;
+    s_w[idx] = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
+    s_d[idx] = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
   }
   for (int idx = tid; idx < G * D; idx += 1024) s_o[idx] = 0.f;
   __syncthreads();
-
-  // g summed over the splits
-  for (int idx = tid; idx < G * 2 * N; idx += 1024) {
-    const int g = idx / (2 * N), n = idx - g * 2 * N;
-    const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + n;
-    float a = 0.f;
-    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[g * n_all + n_il_split + s], gp[(int64_t)s * 2 * N], a);
-    s_g[idx] = a;
+  if (tid < G) {
+    float mstar = -INFINITY;
+    for (int s_ = 0; s_ < n_all; ++s_) mstar = fmaxf(mstar, s_w[tid * n_all + s_]);
+    float dsum = 0.f, pmid = 0.f;
+    for (int s_ = 0; s_ < n_all; ++s_) {
+      const float m = s_w[tid * n_all + s_];
+      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+      s_w[tid * n_all + s_] = wgt;
+      if (s_ < n_il_split) dsum += wgt * s_d[tid * n_all + s_]; else pmid += wgt * s_d[tid * n_all + s_];
+    }
+    s_sc[tid] = dsum + pmid;
+    s_sc[kGMax + tid] = pmid;
   }
   __syncthreads();
 
-  // compressed dims: g . V_coef, thread = (dim j, one of 8 row classes)
-  const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
-  const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
-  {
-    const int j = tid & 127, part = tid >> 7;
-    float acc[kGMax];
+  if (n_mid_split > 0) {
+    if (vc_len > 0) {
+      // g summed over the splits
+      for (int idx = tid; idx < G * 2 * N; idx += 1024) {
+        const int g = idx / (2 * N), n = idx - g * 2 * N;
+        s_g[idx] = weighted_sum(md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N, s_w + g * n_all + n_il_split, n_mid_split);
+      }
+      __syncthreads();
+      // g . V_coef: thread = (dim j, row class)
+      const int jw = vc_len > 64 ? 128 : 64, parts = 1024 / jw;
+      const int j = tid % jw, part = tid / jw;
+      float acc[kGMax];
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
-    if (j < vc_len && n_mid_split > 0) {
-      const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + j;
-      for (int n = part; n < 2 * N; n += 32) {
-        float v[4];
+      for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
+      if (j < vc_len) {
+        const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + j;
+        for (int n0 = part; n0 < 2 * N; n0 += 16 * parts) {
+          float v[16];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = (n + 8 * u < 2 * N) ? vp[(int64_t)(n + 8 * u) * Cv] : 0.f;
+          for (int u = 0; u < 16; ++u) v[u] = (n0 + u * parts < 2 * N) ? vp[(int64_t)(n0 + u * parts) * Cv] : 0.f;
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+          for (int u = 0; u < 16; ++u)
+            if (n0 + u * parts < 2 * N) {
 #pragma unroll
-          for (int g = 0; g < kGMax; ++g)
-            if (g < G && n + 8 * u < 2 * N) acc[g] = fmaf(s_g[g * 2 * N + n + 8 * u], v[u], acc[g]);
+              for (int g = 0; g < kGMax; ++g)
+                if (g < G) acc[g] = fmaf(s_g[g * 2 * N + n0 + u * parts], v[u], acc[g]);
+            }
+        }
+      }
+      // fold the row classes pairwise down to 16 per dim, then finish below
+      if (part < 16 && j < 128) {
+#pragma unroll
+        for (int g = 0; g < kGMax; ++g)
+          if (g < G) s_part[(part * G + g) * 128 + j] = acc[g];
+      }
+      __syncthreads();
+      for (int idx = tid; idx < G * vc_len; idx += 1024) {
+        const int g = idx / vc_len, jj = idx - g * vc_len;
+        float a = 0.f;
+        for (int pp = 0; pp < parts; ++pp) a += s_part[(pp * G + g) * 128 + jj];
+        a /= (float)N;
+        const int64_t o = (int64_t)b * Cv + vc0 + jj;
+        const float pmid = s_sc[kGMax + g];
+        s_o[g * D + (vc_list[vc0 + jj] - h * D)] = scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid;
       }
     }
-#pragma unroll
-    for (int g = 0; g < kGMax; ++g)
-      if (g < G) s_part[(part * G + g) * 128 + j] = acc[g];
-  }
-  __syncthreads();
-  for (int idx = tid; idx < G * vc_len; idx += 1024) {
-    const int g = idx / vc_len, j = idx - g * vc_len;
-    float a = 0.f;
-#pragma unroll
-    for (int part = 0; part < 8; ++part) a += s_part[(part * G + g) * 128 + j];
-    a /= (float)N;
-    const int64_t o = (int64_t)b * Cv + vc0 + j;
-    const float pmid = s_sc[2 * kGMax + g];
-    s_o[g * D + (vc_list[vc0 + j] - h * D)] = n_mid_split > 0 ? scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid : 0.f;
-  }
-  // stored dims
-  for (int idx = tid; idx < G * vn_len; idx += 1024) {
-    const int g = idx / vn_len, j = idx - g * vn_len;
-    const float* op = md_on + (r0 + g) * n_mid_split * D + j;
-    float a = 0.f;
-    for (int s = 0; s < n_mid_split; ++s) a = fmaf(s_w[g * n_all + n_il_split + s], op[(int64_t)s * D], a);
-    s_o[g * D + (vn_list[vn0 + j] - h * D)] = a;
+    for (int idx = tid; idx < G * vn_len; idx += 1024) {
+      const int g = idx / vn_len, jj = idx - g * vn_len;
+      s_o[g * D + (vn_list[vn0 + jj] - h * D)] =
+          weighted_sum(md_on + (r0 + g) * n_mid_split * D + jj, D, s_w + g * n_all + n_il_split, n_mid_split);
+    }
   }
   __syncthreads();
   for (int idx = tid; idx < G * D; idx += 1024) {
     const int g = idx / D, d = idx - g * D;
-    const float* op = il_o + (r0 + g) * n_il_split * D + d;
-    float a = s_o[idx];
-    for (int s = 0; s < n_il_split; ++s) a = fmaf(s_w[g * n_all + s], op[(int64_t)s * D], a);
-    out[(r0 + g) * D + d] = a / s_sc[kGMax + g];
+    const float a = s_o[idx] + weighted_sum(il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
+    out[(r0 + g) * D + d] = a / s_sc[g];
   }
 }
 
 // ---------------------------------------------------------------------------
 // sink + local window, vectorised (16-bit storage, head_dim 64 or 128, 16-byte aligned rows):
-// LPT = D/8 lanes share one row, each holding 8 dims; a wave walks 64/LPT rows per step with an
-// online softmax of its own; the four waves of the block are merged through LDS.
+// a block takes kIlFastTile rows; LPT = D/8 lanes share one row, each holding 8 dims; every wave
+// issues all of its loads first, then runs an online softmax of its own; the four waves of the
+// block are merged through LDS.
 // ---------------------------------------------------------------------------
+constexpr int kIlFastTile = 64;
+
 template <typename E, int D>
 __global__ __launch_bounds__(256) void decode_il_fast_kernel(
     const E* __restrict__ q, Seg s0, Seg s1, float* __restrict__ pm, float* __restrict__ pd,
     float* __restrict__ po, int Hq, int Hkv, int n_split, float sm_log2e) {
-  constexpr int LPT = D / 8, TPW = 64 / LPT;
+  constexpr int LPT = D / 8, TPW = 64 / LPT, ITERS = kIlFastTile / 4 / TPW;
   __shared__ float s_m[4][kGMax], s_d[4][kGMax];
   __shared__ float s_o[4][kGMax][D];
   const int G = Hq / Hkv;
@@ -518,6 +541,17 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
   const int sub = lane % LPT, tl = lane / LPT;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int n_il = s0.rows + s1.rows;
+  const int base = split * kIlFastTile + w * (kIlFastTile / 4);
+  uint4 kraw[ITERS], vraw[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int i = base + it * TPW + tl;
+    const int ii = i < n_il ? i : 0;
+    const bool in0 = ii < s0.rows;
+    const int64_t off = in0 ? (int64_t)b * s0.bs + (int64_t)ii * s0.rs : (int64_t)b * s1.bs + (int64_t)(ii - s0.rows) * s1.rs;
+    kraw[it] = *(const uint4*)((in0 ? (const E*)s0.k : (const E*)s1.k) + off + h * D + sub * 8);
+    vraw[it] = *(const uint4*)((in0 ? (const E*)s0.v : (const E*)s1.v) + off + h * D + sub * 8);
+  }
   float qv[kGMax][8];
 #pragma unroll
   for (int g = 0; g < kGMax; ++g)
@@ -532,19 +566,11 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
   }
-  const int base = split * kTile + w * 64;
-  for (int it = 0; it < 64 / TPW; ++it) {
-    const int i = base + it * TPW + tl;
-    const bool ok = i < n_il;
-    if (__all(!ok)) break;
-    const int ii = ok ? i : 0;
-    const bool in0 = ii < s0.rows;
-    const int64_t off = in0 ? (int64_t)b * s0.bs + (int64_t)ii * s0.rs : (int64_t)b * s1.bs + (int64_t)(ii - s0.rows) * s1.rs;
-    const E* kp = (in0 ? (const E*)s0.k : (const E*)s1.k) + off + h * D + sub * 8;
-    const E* vp = (in0 ? (const E*)s0.v : (const E*)s1.v) + off + h * D + sub * 8;
-    uint4 kraw = *(const uint4*)kp, vraw = *(const uint4*)vp;
-    const E* ke = (const E*)&kraw;
-    const E* ve = (const E*)&vraw;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const bool ok = base + it * TPW + tl < n_il;
+    const E* ke = (const E*)&kraw[it];
+    const E* ve = (const E*)&vraw[it];
     float kf[8], vf[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -559,12 +585,11 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
         float a = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) a = fmaf(kf[e], qv[g][e], a);
-#pragma unroll
-        for (int o_ = 1; o_ < LPT; o_ <<= 1) a += __shfl_xor(a, o_, 64);
+        a = fa_group_sum<LPT>(a);
         sc[g] = ok ? a : -INFINITY;
         float t = sc[g];
-#pragma unroll
-        for (int o_ = LPT; o_ < 64; o_ <<= 1) t = fmaxf(t, __shfl_xor(t, o_, 64));
+        if (LPT == 8) t = fmaxf(t, fa_dpp<FA_DPP_ROR8>(t));
+        t = fa_rows_max(t);
         mx[g] = fmaxf(m[g], t);
         changed |= mx[g] != m[g];
       }
@@ -573,7 +598,7 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
 #pragma unroll
       for (int g = 0; g < kGMax; ++g)
         if (g < G) {
-          const float al = exp2f(m[g] - mx[g]);
+          const float al = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx[g]);
           d[g] *= al;
 #pragma unroll
           for (int e = 0; e < 8; ++e) o[g][e] *= al;
@@ -583,7 +608,7 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
 #pragma unroll
     for (int g = 0; g < kGMax; ++g)
       if (g < G) {
-        const float pv = exp2f(sc[g] - m[g]);
+        const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[g] - m[g]);
         d[g] += pv;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pv, vf[e], o[g][e]);
@@ -593,12 +618,14 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
 #pragma unroll
   for (int g = 0; g < kGMax; ++g)
     if (g < G) {
+      if (LPT == 8) {
+        d[g] += fa_dpp<FA_DPP_ROR8>(d[g]);
 #pragma unroll
-      for (int o_ = LPT; o_ < 64; o_ <<= 1) {
-        d[g] += __shfl_xor(d[g], o_, 64);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[g][e] += __shfl_xor(o[g][e], o_, 64);
+        for (int e = 0; e < 8; ++e) o[g][e] += fa_dpp<FA_DPP_ROR8>(o[g][e]);
       }
+      d[g] = fa_rows_sum(d[g]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[g][e] = fa_rows_sum(o[g][e]);
       if (tl == 0) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) s_o[w][g][sub * 8 + e] = o[g][e];
@@ -650,7 +677,8 @@ enum class Path { Generic, Mfma };
 struct Plan {
   Path path;
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
-  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, total;
+  int n_merge_chunks;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, off_tick, total;
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
@@ -659,10 +687,10 @@ bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
          (N == 128 || N == 256 || N == 512);
 }
 
-Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma) {
+Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma, bool il_fast) {
   Plan p{};
   p.path = mfma ? Path::Mfma : Path::Generic;
-  p.n_il_split = fa_cdiv(n_il, kTile);
+  p.n_il_split = fa_cdiv(n_il, il_fast ? kIlFastTile : kTile);
   if (mfma) {
     const int G = Hq / Hkv;
     p.nbpg = 16 / G < 4 ? 16 / G : 4;       // one wave streams one batch element of the group
@@ -701,13 +729,15 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_mg = take(rows * p.n_mid_split * 2 * N * 4);
   p.off_mon = take(rows * p.n_mid_split * D * 4);
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
+  p.n_merge_chunks = 1;
+  p.off_cpart = take(256);
+  p.off_tick = take((size_t)B * Hkv * 4);
   p.total = o;
   return p;
 }
 
-template <typename E>
 bool il_fast_ok(const fa_decode_args& a) {
-  if (sizeof(E) != 2 || (a.D != 64 && a.D != 128)) return false;
+  if (a.dtype == FA_FP32 || (a.D != 64 && a.D != 128)) return false;
   for (int i = 0; i < 2; ++i) {
     if (a.il_rows[i] == 0) continue;
     if (((uintptr_t)a.k_il[i] & 15) || ((uintptr_t)a.v_il[i] & 15)) return false;
@@ -736,7 +766,7 @@ void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wid
 }
 
 template <typename E>
-int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream_t st) {
+int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_scale, hipStream_t st) {
   char* ws = (char*)a.workspace;
   float* W = (float*)(ws + p.off_W);
   float* c0 = (float*)(ws + p.off_c0);
@@ -747,13 +777,14 @@ int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream
   float* md = (float*)(ws + p.off_md);
   float* mg = (float*)(ws + p.off_mg);
   float* mon = (float*)(ws + p.off_mon);
+  float* cpart = (float*)(ws + p.off_cpart);
+  unsigned* tickets = (unsigned*)(ws + p.off_tick);
   const int G = a.Hq / a.Hkv;
   const float sm_log2e = sm_scale * kLog2e;
   if (p.n_mid_split > 0) {
-    const int rows_per_block = 64;
-    decode_prep_kernel<E><<<dim3(fa_cdiv(2 * a.N, rows_per_block), a.Hkv, a.B), 256, 0, st>>>(
-        (const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0, a.Hq, a.Hkv, a.D,
-        a.N, a.Ck, sm_log2e, rows_per_block);
+    decode_prep_kernel<E><<<dim3(fa_cdiv(2 * a.N, kPrepRows), a.Hkv, a.B), 256, 0, st>>>(
+        (const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0, tickets, a.Hq, a.Hkv,
+        a.D, a.N, a.Ck, sm_log2e);
     if (p.path == Path::Mfma) {
       if constexpr (sizeof(E) == 2) {
         using namespace fa_mfma;
@@ -810,28 +841,32 @@ int launch_all(const fa_decode_args& a, const Plan& p, float sm_scale, hipStream
     Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
     Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
     dim3 grid(p.n_il_split, a.Hkv, a.B);
-    if (il_fast_ok<E>(a)) {
-      if (a.D == 128)
+    bool launched = false;
+    if constexpr (sizeof(E) == 2) {
+      if (p_il_fast) {
+        launched = true;
+        if (a.D == 128)
         decode_il_fast_kernel<E, 128><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
       else
         decode_il_fast_kernel<E, 64><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
-    } else {
+      }
+    }
+    if (!launched) {
       size_t lds = (2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);
       decode_il_kernel<E><<<grid, 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, a.D, p.n_il_split, sm_log2e);
     }
   }
   {
-    size_t lds = ((size_t)G * 2 * a.N + (size_t)G * a.D + (size_t)G * (p.n_il_split + p.n_mid_split) + 3 * kGMax +
-                  8 * (size_t)G * 128) * sizeof(float);
+    const int n_all = p.n_il_split + p.n_mid_split;
+    size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 16 * (size_t)G * 128 + (size_t)G * a.D) * sizeof(float);
     if (lds > 64 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_merge_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
     }
-    decode_merge_kernel<<<dim3(a.Hkv, a.B), 1024, lds, st>>>(ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split,
-                                                             a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v, a.vc_list,
-                                                             a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv,
-                                                             a.D, a.N, a.Cv);
+    decode_merge_kernel<<<dim3(a.Hkv, a.B), 1024, lds, st>>>(
+        ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
+        a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv);
   }
   return fa_check_launch("fa_decode_attn");
 }
@@ -847,10 +882,14 @@ extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, 
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || N < 0 || il_rows_total < 0 || L_m < 0 || Hq % Hkv) return 0;
   const int n = N > 0 ? N : 1;
   // large enough for either path
-  size_t a = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, false).total;
-  if (mfma_shape_ok(Hq, Hkv, D, n, FA_BF16, FA_MID_PAGED)) {
-    size_t b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, true).total;
+  size_t a = 0;
+  for (int il_fast = 0; il_fast < 2; ++il_fast) {
+    size_t b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, false, il_fast != 0).total;
     if (b > a) a = b;
+    if (mfma_shape_ok(Hq, Hkv, D, n, FA_BF16, FA_MID_PAGED)) {
+      b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, true, il_fast != 0).total;
+      if (b > a) a = b;
+    }
   }
   return a;
 }
@@ -907,7 +946,9 @@ extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
     }
   }
   const bool mfma = use_mfma(*a);
-  const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma);
+  const bool il_fast = il_fast_ok(*a);
+  const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma,
+                           il_fast);
   FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
              a->workspace_bytes, p.total);
   FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");
@@ -915,8 +956,8 @@ extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
   const float sm = a->sm_scale > 0.f ? a->sm_scale : 1.0f / sqrtf((float)a->D);
   hipStream_t st = fa_hip_stream(stream);
   switch (a->dtype) {
-    case FA_BF16: return launch_all<bf16_t>(*a, p, sm, st);
-    case FA_FP16: return launch_all<f16_t>(*a, p, sm, st);
-    default: return launch_all<float>(*a, p, sm, st);
+    case FA_BF16: return launch_all<bf16_t>(*a, p, il_fast, sm, st);
+    case FA_FP16: return launch_all<f16_t>(*a, p, il_fast, sm, st);
+    default: return launch_all<float>(*a, p, il_fast, sm, st);
   }
 }

@@ -208,8 +208,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         wmax = fmaxf(wmax, fmaxf(fmaxf(fabsf(c2[0]), fabsf(c2[1])), fmaxf(fabsf(s2[0]), fabsf(s2[1]))));
       }
     }
-    wmax = fmaxf(wmax, __shfl_xor(wmax, 16, 64));
-    wmax = fmaxf(wmax, __shfl_xor(wmax, 32, 64));
+    wmax = fa_rows_max(wmax);
     if (lg == 0) s_max[sl][lc] = wmax;
     __syncthreads();
     wmax = fmaxf(fmaxf(s_max[0][lc], s_max[1][lc]), fmaxf(s_max[2][lc], s_max[3][lc]));
@@ -356,8 +355,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (tok0 + e >= p.L_m) sc[e] = -INFINITY;
         }
         float tmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        tmax = fa_rows_max(tmax);
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first page (m_run = -inf)
         float psum = 0.f;
@@ -410,8 +408,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- partials of this split ------------------------------------------------------
-    float dsum = d_run + __shfl_xor(d_run, 16, 64);
-    dsum += __shfl_xor(dsum, 32, 64);
+    const float dsum = fa_rows_sum(d_run);
     if (valid_r) {
       const int64_t base = qrow * p.n_split + split;
       if (sl == 0 && lg == 0) {
