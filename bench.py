@@ -141,6 +141,8 @@ def main():
     ap.add_argument("--workload", default="config3_decode_attn_8b_32k", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run ten 1 GiB device-to-device copies (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives exist on this path); use --gpus 1",
@@ -153,6 +155,14 @@ def main():
     torch.cuda.set_device(device)
     from fourierattention_amd import _lib
     _lib.load()
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_per_copy": 1 << 30, "copies": 10}))
+        return
 
     w = WORKLOADS[args.workload]
     dtype = torch.bfloat16
@@ -179,9 +189,32 @@ def main():
     nbytes = algorithmic_bytes(w)
     gbs = nbytes / (ms * 1e-3) / 1e9
     L = w["ctx"] - w["I"] - w["W"]
-    full = 2 * w["ctx"] * w["Hkv"] * w["D"] * 2
-    fourier = (2 * (w["I"] + w["W"]) * w["Hkv"] * w["D"] * 2 + 2 * L * (w["Hkv"] * w["D"] - w["cper"] * w["Hkv"]) * 2
-               + 2 * w["M"] * w["cper"] * w["Hkv"] * 4)
+    hd = w["Hkv"] * w["D"]
+    ck = w["cper"] * w["Hkv"]
+    # per-kernel durations, HIP events recorded inside the library on the launch stream
+    reps = max(10, min(50, args.steps))
+    per = np.zeros(4)
+    for _ in range(reps):
+        tm = []
+        cache.decode_attention(q, 0, Hq, Hkv, timings=tm)
+        per += np.array(tm)
+    per /= reps
+    kernel_ms = {"coeff_query": per[0], "mid_rows": per[1], "sink_window": per[2], "merge": per[3]}
+    # algorithmic bytes of each kernel's own launch
+    kbytes = {
+        "coeff_query": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4,
+        "mid_rows": w["B"] * 2 * L * (hd - ck) * 2,
+        "sink_window": w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,
+        "merge": w["B"] * w["M"] * ck * 4,
+    }
+    dom = max(kernel_ms, key=kernel_ms.get)
+    dom_gbs = kbytes[dom] / (kernel_ms[dom] * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_mid_rows_traffic.json")
+    if dom == "mid_rows" and args.workload.startswith("config3") and os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+    full = 2 * w["ctx"] * hd * 2
+    fourier = 2 * (w["I"] + w["W"]) * hd * 2 + 2 * L * (hd - ck) * 2 + 2 * w["M"] * ck * 4
     result = {
         "metric": "Fourier decode attn HBM GB/s (% peak) + tok/s, Llama-3.1-8B geometry, 32k ctx",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -196,9 +229,11 @@ def main():
         "algorithmic_bytes_per_step": nbytes,
         "parity_max_abs_err": parity,
         "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "all kernels of one fa_decode_attn call"},
+        "kernel_ms": {k: round(float(v), 5) for k, v in kernel_ms.items()},
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom,
+                     "algorithmic_bytes_per_launch": kbytes[dom], "kernel_ms": round(float(kernel_ms[dom]), 5),
+                     "whole_step_frac": round(gbs / HBM_PEAK_GBS, 4)},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()

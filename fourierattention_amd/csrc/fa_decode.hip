@@ -529,13 +529,13 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kIlFastTile = 64;
 
-template <typename E, int D>
+template <typename E, int D, int GM>
 __global__ __launch_bounds__(256) void decode_il_fast_kernel(
     const E* __restrict__ q, Seg s0, Seg s1, float* __restrict__ pm, float* __restrict__ pd,
     float* __restrict__ po, int Hq, int Hkv, int n_split, float sm_log2e) {
   constexpr int LPT = D / 8, TPW = 64 / LPT, ITERS = kIlFastTile / 4 / TPW;
-  __shared__ float s_m[4][kGMax], s_d[4][kGMax];
-  __shared__ float s_o[4][kGMax][D];
+  __shared__ float s_m[4][GM], s_d[4][GM];
+  __shared__ float s_o[4][GM][D];
   const int G = Hq / Hkv;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int sub = lane % LPT, tl = lane / LPT;
@@ -552,15 +552,15 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
     kraw[it] = *(const uint4*)((in0 ? (const E*)s0.k : (const E*)s1.k) + off + h * D + sub * 8);
     vraw[it] = *(const uint4*)((in0 ? (const E*)s0.v : (const E*)s1.v) + off + h * D + sub * 8);
   }
-  float qv[kGMax][8];
+  float qv[GM][8];
 #pragma unroll
-  for (int g = 0; g < kGMax; ++g)
+  for (int g = 0; g < GM; ++g)
 #pragma unroll
     for (int e = 0; e < 8; ++e)
       qv[g][e] = g < G ? fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + sub * 8 + e]) * sm_log2e : 0.f;
-  float m[kGMax], d[kGMax], o[kGMax][8];
+  float m[GM], d[GM], o[GM][8];
 #pragma unroll
-  for (int g = 0; g < kGMax; ++g) {
+  for (int g = 0; g < GM; ++g) {
     m[g] = -INFINITY;
     d[g] = 0.f;
 #pragma unroll
@@ -577,10 +577,10 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
       kf[e] = fa_to_float(ke[e]);
       vf[e] = fa_to_float(ve[e]);
     }
-    float sc[kGMax], mx[kGMax];
+    float sc[GM], mx[GM];
     bool changed = false;
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g) {
+    for (int g = 0; g < GM; ++g) {
       if (g < G) {
         float a = 0.f;
 #pragma unroll
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
     }
     if (changed) {  // wave-uniform: every lane sees the same maxima
 #pragma unroll
-      for (int g = 0; g < kGMax; ++g)
+      for (int g = 0; g < GM; ++g)
         if (g < G) {
           const float al = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx[g]);
           d[g] *= al;
@@ -606,7 +606,7 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
         }
     }
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g)
+    for (int g = 0; g < GM; ++g)
       if (g < G) {
         const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[g] - m[g]);
         d[g] += pv;
@@ -616,7 +616,7 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
   }
   // reduce over the rows a wave holds side by side, then over the four waves
 #pragma unroll
-  for (int g = 0; g < kGMax; ++g)
+  for (int g = 0; g < GM; ++g)
     if (g < G) {
       if (LPT == 8) {
         d[g] += fa_dpp<FA_DPP_ROR8>(d[g]);
@@ -765,8 +765,11 @@ void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wid
     fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4><<<grid, 512, 0, st>>>(mp);
 }
 
+// ev (optional): five events recorded before the first kernel and after each of prep (+ tables),
+// mid, sink/window and merge
 template <typename E>
-int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_scale, hipStream_t st) {
+int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_scale, hipStream_t st, hipEvent_t* ev) {
+  if (ev) hipEventRecord(ev[0], st);
   char* ws = (char*)a.workspace;
   float* W = (float*)(ws + p.off_W);
   float* c0 = (float*)(ws + p.off_c0);
@@ -804,6 +807,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
         mp.sm_log2e = sm_log2e;
+        if (ev) hipEventRecord(ev[1], st);
         {
           static const int dbg = getenv("FA_DEBUG_FLAGS") ? atoi(getenv("FA_DEBUG_FLAGS")) : 0;
           mp.dbg = dbg;
@@ -837,6 +841,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
             mm, md, mg, mon, a.Hq, a.Hkv, a.D, a.N, a.L_m, a.T, p.n_mid_split, p.tiles_per_split, sm_log2e);
     }
   }
+  if (ev && (p.n_mid_split == 0 || p.path != Path::Mfma)) hipEventRecord(ev[1], st);
+  if (ev) hipEventRecord(ev[2], st);
   if (p.n_il_split > 0) {
     Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
     Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
@@ -845,10 +851,14 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     if constexpr (sizeof(E) == 2) {
       if (p_il_fast) {
         launched = true;
-        if (a.D == 128)
-        decode_il_fast_kernel<E, 128><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
-      else
-        decode_il_fast_kernel<E, 64><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+        if (a.D == 128 && G <= 4)
+          decode_il_fast_kernel<E, 128, 4><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+        else if (a.D == 128)
+          decode_il_fast_kernel<E, 128, kGMax><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+        else if (G <= 4)
+          decode_il_fast_kernel<E, 64, 4><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+        else
+          decode_il_fast_kernel<E, 64, kGMax><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
       }
     }
     if (!launched) {
@@ -856,6 +866,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
       decode_il_kernel<E><<<grid, 256, lds, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, a.D, p.n_il_split, sm_log2e);
     }
   }
+  if (ev) hipEventRecord(ev[3], st);
   {
     const int n_all = p.n_il_split + p.n_mid_split;
     size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 16 * (size_t)G * 128 + (size_t)G * a.D) * sizeof(float);
@@ -868,6 +879,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
         a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv);
   }
+  if (ev) hipEventRecord(ev[4], st);
   return fa_check_launch("fa_decode_attn");
 }
 
@@ -906,7 +918,7 @@ extern "C" int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, 
   return fa_check_launch("fa_decode_tables_build");
 }
 
-extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
+static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEvent_t* ev) {
   FA_REQUIRE(a, FA_ERR_NULL_POINTER, "fa_decode_attn: null argument block");
   FA_REQUIRE(a->q_len == 1, FA_ERR_BAD_SHAPE, "fa_decode_attn: q_len = %d, decode needs exactly one query row", a->q_len);
   FA_REQUIRE(a->B > 0 && a->Hq > 0 && a->Hkv > 0 && a->D > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: bad B/Hq/Hkv/D");
@@ -956,8 +968,29 @@ extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) {
   const float sm = a->sm_scale > 0.f ? a->sm_scale : 1.0f / sqrtf((float)a->D);
   hipStream_t st = fa_hip_stream(stream);
   switch (a->dtype) {
-    case FA_BF16: return launch_all<bf16_t>(*a, p, il_fast, sm, st);
-    case FA_FP16: return launch_all<f16_t>(*a, p, il_fast, sm, st);
-    default: return launch_all<float>(*a, p, il_fast, sm, st);
+    case FA_BF16: return launch_all<bf16_t>(*a, p, il_fast, sm, st, ev);
+    case FA_FP16: return launch_all<f16_t>(*a, p, il_fast, sm, st, ev);
+    default: return launch_all<float>(*a, p, il_fast, sm, st, ev);
   }
+}
+
+extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) { return decode_attn_impl(a, stream, nullptr); }
+
+extern "C" int fa_decode_attn_timed(const fa_decode_args* a, fa_stream_t stream, float* ms_out) {
+  FA_REQUIRE(ms_out, FA_ERR_NULL_POINTER, "fa_decode_attn_timed: ms_out null");
+  hipEvent_t ev[5];
+  for (int i = 0; i < 5; ++i)
+    if (hipEventCreate(&ev[i]) != hipSuccess) {
+      fa_set_error("fa_decode_attn_timed: hipEventCreate failed");
+      return FA_ERR_LAUNCH;
+    }
+  int rc = decode_attn_impl(a, stream, ev);
+  if (rc == FA_OK && hipEventSynchronize(ev[4]) != hipSuccess) {
+    fa_set_error("fa_decode_attn_timed: hipEventSynchronize failed");
+    rc = FA_ERR_LAUNCH;
+  }
+  if (rc == FA_OK)
+    for (int i = 0; i < 4; ++i) hipEventElapsedTime(&ms_out[i], ev[i], ev[i + 1]);
+  for (int i = 0; i < 5; ++i) hipEventDestroy(ev[i]);
+  return rc;
 }

@@ -211,7 +211,7 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
-                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False):
+                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None):
     """Thin call into ``fa_decode_attn``.
 
     ``il_segments``: up to two ``(k, v)`` pairs of ``(B, rows, Hkv*D)`` views (last dim contiguous).
@@ -276,7 +276,12 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     nbytes = lib.fa_decode_attn_workspace_bytes(B, num_head_q, num_head_kv, D, N, total_il, int(seq_len_m))
     ws = workspace(q.device, nbytes, "decode")
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-    check(lib.fa_decode_attn(ctypes.byref(a), _stream(q.device)))
+    if timings is not None:   # list to receive [prep, mid, sink/window, merge] milliseconds
+        ms = (ctypes.c_float * 4)()
+        check(lib.fa_decode_attn_timed(ctypes.byref(a), _stream(q.device), ms))
+        timings[:] = list(ms)
+    else:
+        check(lib.fa_decode_attn(ctypes.byref(a), _stream(q.device)))
     return out
 
 

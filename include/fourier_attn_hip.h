@@ -220,6 +220,12 @@ int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_s
  * [sink ; local window ; mid rows (stored dims + dims rebuilt from coefficients)]. */
 int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
 
+/* Same call, bracketed by HIP events on `stream`; synchronises and returns in ms_out[0..3] the
+ * milliseconds spent in (0) the coefficient-domain query kernel (plus the operand tables when
+ * they are built in the workspace), (1) the mid-row kernel, (2) the sink/window kernel and
+ * (3) the merge kernel.  A measurement aid for benchmarks (the reference has no timers). */
+int fa_decode_attn_timed(const fa_decode_args* args, fa_stream_t stream, float* ms_out);
+
 #ifdef __cplusplus
 }
 #endif
