@@ -52,8 +52,15 @@ __device__ __forceinline__ float fa_round_through(float v, int dtype) {
 // ---- exact Fourier phases ---------------------------------------------------
 // cos/sin of 2*pi*((a*b) mod T)/T; the product is reduced in integers so the
 // angle handed to the float unit is always inside one period.
+// (a*b) mod T for non-negative a, b: the 64-bit division is a long software routine, so products that fit
+// 32 bits (all but very long contexts) take the short one
+__device__ __forceinline__ uint32_t fa_phase_mod(int64_t a, int64_t b, int T) {
+  const uint64_t prod = (uint64_t)a * (uint64_t)b;
+  if ((prod >> 32) == 0) return (uint32_t)prod % (uint32_t)T;
+  return (uint32_t)(prod % (uint64_t)T);
+}
 __device__ __forceinline__ void fa_sincos_phase(int64_t a, int64_t b, int T, float* s, float* c) {
-  int64_t r = (a * b) % (int64_t)T;
+  const uint32_t r = fa_phase_mod(a, b, T);
   float x = 2.0f * (float)r / (float)T;  // in [0, 2)
   sincospif(x, s, c);
 }

@@ -760,9 +760,9 @@ template <typename E, int KS>
 void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
   dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
   if (wide)
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2><<<grid, 512, 0, st>>>(mp);
   else
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2><<<grid, 512, 0, st>>>(mp);
 }
 
 // ev (optional): five events recorded before the first kernel and after each of prep (+ tables),
@@ -808,10 +808,6 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
         mp.sm_log2e = sm_log2e;
         if (ev) hipEventRecord(ev[1], st);
-        {
-          static const int dbg = getenv("FA_DEBUG_FLAGS") ? atoi(getenv("FA_DEBUG_FLAGS")) : 0;
-          mp.dbg = dbg;
-        }
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
         switch (KS) {
           case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, st); break;

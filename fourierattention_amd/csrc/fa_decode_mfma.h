@@ -105,6 +105,87 @@ static inline size_t tables_bytes(int N) {
   return (size_t)(2 * kFreqWaves * 2 * KS * 64) * 16 + (size_t)N * 8;
 }
 
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt 15 << 8 | vmcnt[5:4] << 14)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+// one fragment (64 lanes x 16 bytes) from global memory straight into LDS at lds_frag + lane * 16
+template <typename E>
+__device__ __forceinline__ void load_frag_to_lds(const E* g_lane_ptr, void* lds_frag) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g_lane_ptr,
+                                   (__attribute__((address_space(3))) void*)lds_frag, 16, 0, 0);
+}
+
+// LDS accesses that the compiler must not tie to the asynchronous page loads (it would otherwise wait
+// for every outstanding global_load_lds before each read and before each barrier)
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4v lds_read_b128_async(const void* lds_ptr) {
+  uint4v r;
+  const unsigned addr = (unsigned)(size_t)(const __attribute__((address_space(3))) void*)lds_ptr;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+// the read above completes asynchronously: tie the wait to the value so no use can be scheduled before it
+__device__ __forceinline__ void lds_wait_for(uint4v& r) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r)::"memory"); }
+// same for a batch of four reads, leaving the AFTER LDS operations issued after the batch in flight (LDS
+// operations complete in issue order, so a count is enough; later LDS traffic only makes the wait longer)
+template <int AFTER>
+__device__ __forceinline__ void lds_wait_for4(uint4v (&r)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(AFTER) : "memory");
+}
+// workgroup barrier that orders LDS traffic only (global loads stay in flight)
+__device__ __forceinline__ void barrier_lds_only() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// ---- page-step rotation of coefficient-domain state ---------------------------------------------------
+// Both wave roles turn 2*KS row tiles of (cos, sin) pairs by the per-frequency angle of one page.  The
+// constants sit in LDS as float4 {c, s, c', s'} per (row tile, lane group), 64 bytes between row tiles.
+// They are fetched in batches of four tiles, two batches in flight, so that the LDS latency hides behind
+// the arithmetic of the previous batch instead of being paid once per tile.
+__device__ __forceinline__ void rot_issue(const void* lane_base, int batch, uint4v (&buf)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) buf[j] = lds_read_b128_async((const char*)lane_base + (batch * 4 + j) * 64);
+}
+// the same, issued only once `after` has been computed: keeps a refill of a constant buffer behind the
+// arithmetic that consumed its previous contents (otherwise all batches are hoisted and held at once)
+__device__ __forceinline__ void rot_issue_after(const void* lane_base, int batch, uint4v (&buf)[4], float after) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned addr =
+        (unsigned)(size_t)(const __attribute__((address_space(3))) void*)((const char*)lane_base + (batch * 4 + j) * 64);
+    asm volatile("ds_read_b128 %0, %1 ; after %2" : "=v"(buf[j]) : "v"(addr), "v"(after));
+  }
+}
+__device__ __forceinline__ void rot_pair(float c, float s, float& x, float& y) {
+  const float sy = s * y, sx = s * x;
+  x = __builtin_fmaf(c, x, sy);
+  y = __builtin_fmaf(c, y, -sx);
+}
+// pair(rt, f2, c, s) applies one rotation and returns one of its results; pin(b) passes the results of
+// batch b (row tiles 4b .. 4b+3) through an empty asm volatile, which keeps their arithmetic above the
+// next wait (it is otherwise sunk to its uses, and every batch of constants is then held at once);
+// batches 0 and 1 must already be in flight in rc[0], rc[1]
+template <int NT, typename F, typename P>
+__device__ __forceinline__ void rot_apply(const void* lane_base, uint4v (&rc)[2][4], F&& pair, P&& pin) {
+  constexpr int NB = NT / 4;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (b + 1 < NB) lds_wait_for4<4>(rc[b & 1]);
+    else lds_wait_for4<0>(rc[b & 1]);
+    float last = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4v raw = rc[b & 1][j];
+      const unsigned c0 = raw[0], s0 = raw[1], c1 = raw[2], s1 = raw[3];  // scalars first: see fa_swap16
+      pair(b * 4 + j, 0, __builtin_bit_cast(float, c0), __builtin_bit_cast(float, s0));
+      last = pair(b * 4 + j, 1, __builtin_bit_cast(float, c1), __builtin_bit_cast(float, s1));
+    }
+    pin(b);
+    if (b + 2 < NB) rot_issue_after(lane_base, b + 2, rc[b & 1], last);
+  }
+}
+
 template <typename E>
 struct MidParams {
   const E* q;
@@ -128,12 +209,11 @@ struct MidParams {
   float* pon;
   int B, Hq, Hkv, D, G, nbpg, N, L_m, T, n_split, tiles_per_split;
   float sm_log2e;
-  int dbg;  // profiling aid: bit 0 skips the stored-dim stream
 };
 
 // native sin/cos of 2*pi*((a*b) mod T)/T (hardware takes the angle in revolutions)
 __device__ __forceinline__ void fast_sincos_phase(int64_t a, int64_t b, int T, float* s, float* c) {
-  const float x = (float)((a * b) % (int64_t)T) / (float)T;
+  const float x = (float)fa_phase_mod(a, b, T) / (float)T;
   *s = __builtin_amdgcn_sinf(x);
   *c = __builtin_amdgcn_cosf(x);
 }
@@ -146,16 +226,21 @@ __device__ __forceinline__ void fast_sincos_phase(int64_t a, int64_t b, int T, f
 // Score wave i and value wave i own the same frequencies and stream the same batch element of the group.
 // KS: ksteps (32 coefficient rows) per slice = N / 64.  KMAX: ksteps of stored K dims a head may have
 // (dp_k / 32).  VMAX: V dim groups of 16 (dp_v / 16).
-template <typename E, int KS, int KMAX, int VMAX>
+// NST: page stages per wave in LDS; the K / V pages travel HBM -> LDS with global_load_lds (no registers
+// held while in flight), NST - 1 pages ahead of their use.
+template <typename E, int KS, int KMAX, int VMAX, int NST>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
   using M = Mma<E>;
   using vec8 = typename M::vec8;
+  constexpr int kFragsMax = (2 * KMAX > VMAX ? 2 * KMAX : VMAX);   // fragments (1 KiB) of one page of one wave
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[8][NST][kFragsMax * 1024];
   __shared__ float s_part[2][kFreqWaves][16 * kPart];
   __shared__ float s_max[kFreqWaves][16];
   __shared__ float4v s_rot[kFreqWaves * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
 
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, lg = lane >> 4, lc = lane & 15;
+  const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
   const bool score_wave = w < kFreqWaves;
   const int sl = w & 3;  // frequency slice and batch element of the group
   const int split = blockIdx.x, h = blockIdx.y, grp = blockIdx.z;
@@ -167,7 +252,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int bb_r = lc / G, g_r = lc - bb_r * G;
   const int64_t qrow = valid_r ? ((int64_t)(b0 + bb_r) * p.Hq + h * G + g_r) : 0;
   const int fbase = sl * 16 * KS;
-  const bool has_mn = sl < nb && !(p.dbg & 1);
+  const bool has_mn = sl < nb;
   const int my_b = b0 + (sl < nb ? sl : 0);
 
   const int n_tiles = (p.L_m + 31) >> 5;
@@ -216,49 +301,98 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float colscale = wmax > 0.f ? exp2f(ceilf(log2f(wmax))) : 1.f;
     const float colinv = 1.0f / colscale;
     const float c0col = (valid_r && sl == 0) ? p.c0[qrow] : 0.f;
+    {
+      // phases of the first page: exact for row tile 0, then stepped by the (exact) phase of 8 frequencies
+      float sn[2], co[2], s8, c8;
+      fast_sincos_phase(8, (int64_t)32 * t_beg, p.T, &s8, &c8);
 #pragma unroll
-    for (int rt = 0; rt < 2 * KS; ++rt)
+      for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), (int64_t)32 * t_beg, p.T, &sn[f2], &co[f2]);
 #pragma unroll
-      for (int f2 = 0; f2 < 2; ++f2) {
-        float sn, co;
-        fast_sincos_phase(fbase + freq_of(rt, lg, f2), (int64_t)32 * t_beg, p.T, &sn, &co);
-        const float wc = Wc[rt][f2] * colinv, ws = Ws[rt][f2] * colinv;
-        Wc[rt][f2] = co * wc + sn * ws;    // rotation by -phi: W'c = cos(phi) wc + sin(phi) ws
-        Ws[rt][f2] = -sn * wc + co * ws;   //                   W's = -sin(phi) wc + cos(phi) ws
-      }
+      for (int rt = 0; rt < 2 * KS; ++rt)
+#pragma unroll
+        for (int f2 = 0; f2 < 2; ++f2) {
+          const float wc = Wc[rt][f2] * colinv, ws = Ws[rt][f2] * colinv;
+          Wc[rt][f2] = co[f2] * wc + sn[f2] * ws;    // rotation by -phi: W'c = cos(phi) wc + sin(phi) ws
+          Ws[rt][f2] = -sn[f2] * wc + co[f2] * ws;   //                   W's = -sin(phi) wc + cos(phi) ws
+          const float cn = co[f2] * c8 - sn[f2] * s8;
+          sn[f2] = sn[f2] * c8 + co[f2] * s8;
+          co[f2] = cn;
+        }
+    }
 
     // stored K dims of batch element sl: both 16-token blocks of the page
     const int kn0 = p.kn_h[h], kn_len = p.kn_h[h + 1] - kn0;
     const int kp0 = p.kpad_h[h], dpk = p.kpad_h[h + 1] - kp0;
     const int nks = dpk >> 5;
+    // the gathered query dims: all index loads first, then all query loads (clamped so that none is
+    // conditional: conditional loads would be issued one round trip after the other)
     vec8 Qb[KMAX];
 #pragma unroll
     for (int s = 0; s < KMAX; ++s)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int j = s * 32 + 8 * lg + e;
-        typename M::elem val = (typename M::elem)0.f;
-        if (has_mn && valid_r && bb_r == sl && j < kn_len)
-          val = M::from_bits(p.q[qrow * p.D + (p.kn_list[kn0 + j] - h * p.D)]);
-        Qb[s][e] = val;
-      }
-    const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages + lane * 8;
-    vec8 K0[2 * KMAX], K1[2 * KMAX], K2[2 * KMAX];
-    auto load_k = [&](int t, vec8* kf) {
+      for (int e = 0; e < 8; ++e) Qb[s][e] = (typename M::elem)0.f;
+    if (kn_len > 0) {   // one branch around the whole gather; nothing inside is conditional
+      const bool mine = has_mn && valid_r && bb_r == sl;
+      const int32_t* kl = p.kn_list + kn0;
+      const E* qr = p.q + qrow * p.D - h * p.D;
+      int dim[KMAX][8];
+#pragma unroll
+      for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dim[s][e] = kl[min(s * 32 + 8 * lg + e, kn_len - 1)];
+      E qv[KMAX][8];
+#pragma unroll
+      for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[s][e] = qr[dim[s][e]];
+#pragma unroll
+      for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (mine && s * 32 + 8 * lg + e < kn_len) Qb[s][e] = M::from_bits(qv[s][e]);
+    }
+    const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
+    const bool has_k = has_mn && nks > 0;
+    // every page moves 2*KMAX fragments so that the number of loads in flight is a compile-time constant;
+    // a head with fewer stored dims repeats its first fragment into the unused slots
+    auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* kp = kbase + (int64_t)t * dpk * 32;
+      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-        for (int s = 0; s < KMAX; ++s)
-          if (s < nks) kf[tb * KMAX + s] = *(const vec8*)(kp + (tb * nks + s) * 512);
+        for (int ks = 0; ks < KMAX; ++ks)
+          load_frag_to_lds(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
     };
-    if (has_mn && n_it > 0) load_k(t_beg, K0);
-    if (has_mn && n_it > 1) load_k(t_beg + 1, K1);
+    // every table and weight load above must have landed before the page loads start: afterwards the
+    // only waits on vector memory in this wave are the explicit page waits
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
+    if (has_k) {
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i)
+        if (i < n_it) issue_k(t_beg + i);
+    }
+    const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
       if (it < n_it) {
         const int t = t_beg + it;
-        if (has_mn && it + 2 < n_it) load_k(t + 2, K2);
+        uint4v kraw[2 * KMAX];
+        uint4v rc[2][4];
+        if (has_k) {
+          // pages t+1 .. t+NST-2 may still be in flight; page t has landed: start its LDS reads now
+          if (it + NST - 2 < n_it) wait_vmcnt<(NST - 2) * 2 * KMAX>();
+          else wait_vmcnt<0>();
+          if (it + NST - 1 < n_it) issue_k(t + NST - 1);   // refills the stage read one page ago
+          const unsigned char* st = &s_stage[w][it % NST][0];
+#pragma unroll
+          for (int f = 0; f < 2 * KMAX; ++f) kraw[f] = lds_read_b128_async(st + (size_t)f * 1024 + lane * 16);
+        }
+        rot_issue(rot_lane, 0, rc[0]);
+        if (2 * KS > 4) rot_issue(rot_lane, 1, rc[1]);
         float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -271,13 +405,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           accf[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][s], wb, accf[0], 0, 0, 0);
           accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
         }
+        // advance W' by one page step
+        rot_apply<2 * KS>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
+          rot_pair(c, sn, Wc[rt][f2], Ws[rt][f2]);
+          return Ws[rt][f2];
+        }, [&](int b) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            asm volatile("" : "+v"(Wc[4 * b + j][0]), "+v"(Wc[4 * b + j][1]), "+v"(Ws[4 * b + j][0]), "+v"(Ws[4 * b + j][1]));
+        });
         float4v accm[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
-        if (has_mn) {
+        if (has_k) {
+#pragma unroll
+          for (int f = 0; f < 2 * KMAX; ++f) lds_wait_for(kraw[f]);
 #pragma unroll
           for (int s = 0; s < KMAX; ++s)
             if (s < nks) {
-              accm[0] = M::mma(K0[s], Qb[s], accm[0]);
-              accm[1] = M::mma(K0[KMAX + s], Qb[s], accm[1]);
+              accm[0] = M::mma(__builtin_bit_cast(vec8, kraw[s]), Qb[s], accm[0]);
+              accm[1] = M::mma(__builtin_bit_cast(vec8, kraw[KMAX + s]), Qb[s], accm[1]);
             }
         }
 #pragma unroll
@@ -287,27 +432,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int v = 0; v < 4; ++v) o[v] = accf[rb][v] * colscale + accm[rb][v] * p.sm_log2e + c0col;
           *(float4v*)&s_part[it & 1][sl][lc * kPart + rb * 16 + 4 * lg] = o;
         }
-        // advance W' by one page step
-#pragma unroll
-        for (int rt = 0; rt < 2 * KS; ++rt) {
-          const float4v cs = s_rot[(sl * 2 * KS + rt) * 4 + lg];
-#pragma unroll
-          for (int f2 = 0; f2 < 2; ++f2) {
-            const float c = cs[2 * f2], s = cs[2 * f2 + 1];
-            const float x = Wc[rt][f2], y = Ws[rt][f2];
-            Wc[rt][f2] = c * x + s * y;
-            Ws[rt][f2] = c * y - s * x;
-          }
-        }
-        if (has_mn) {
-#pragma unroll
-          for (int f = 0; f < 2 * KMAX; ++f) {
-            K0[f] = K1[f];
-            K1[f] = K2[f];
-          }
-        }
       }
-      __syncthreads();
+      barrier_lds_only();
     }
   } else {
     // =============================== value waves ===============================
@@ -316,16 +442,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
     const int vp0 = p.vpad_h[h], dpv = p.vpad_h[h + 1] - vp0;
     const int ndg = dpv >> 4;
-    const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages + lane * 8;
-    vec8 V0[VMAX], V1[VMAX], V2[VMAX];
-    auto load_v = [&](int t, vec8* vf) {
+    const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
+    const bool has_v = has_mn && ndg > 0;
+    // VMAX fragments per page whatever the head holds (see the score waves)
+    auto issue_v = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* vp = vbase + (int64_t)t * dpv * 32;
+      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
 #pragma unroll
-      for (int f = 0; f < VMAX; ++f)
-        if (f < ndg) vf[f] = *(const vec8*)(vp + f * 512);
+      for (int f = 0; f < VMAX; ++f) load_frag_to_lds(vp + (f < ndg ? f : 0) * 512 + lane * 8, st + f * 1024);
     };
-    if (has_mn && n_it > 0) load_v(t_beg, V0);
-    if (has_mn && n_it > 1) load_v(t_beg + 1, V1);
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -334,20 +459,66 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float m_run = -INFINITY, d_run = 0.f;
     const bool ragged_tail = (p.L_m & 31) != 0;
     __syncthreads();  // pairs with the score waves' column-scale exchange
+    // the table loads must have landed before the page loads start (see the score waves)
+#pragma unroll
+    for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
+    if (has_v) {
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i)
+        if (i < n_it) issue_v(t_beg + i);
+    }
+    const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
       if (it > 0) {
         const int t = t_beg + it - 1, buf = (it - 1) & 1;
-        if (has_mn && it + 1 < n_it) load_v(t + 2, V2);
-        // scores of the page in B-operand layout: column lc, tokens 8*lg + e
-        float4v a0 = *(const float4v*)&s_part[buf][0][lc * kPart + 8 * lg];
-        float4v a1 = *(const float4v*)&s_part[buf][0][lc * kPart + 8 * lg + 4];
-#pragma unroll
-        for (int ww = 1; ww < kFreqWaves; ++ww) {
-          a0 += *(const float4v*)&s_part[buf][ww][lc * kPart + 8 * lg];
-          a1 += *(const float4v*)&s_part[buf][ww][lc * kPart + 8 * lg + 4];
+        const int pg = it - 1;   // page index within the split
+        uint4v rc[2][4];
+        rot_issue(rot_lane, 0, rc[0]);
+        if (2 * KS > 4) rot_issue(rot_lane, 1, rc[1]);
+        if (has_v) {
+          if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
+          else wait_vmcnt<0>();
+          if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
         }
-        float sc[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+        // the g history moves into the frame of this page
+        rot_apply<2 * KS>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
+          float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
+          rot_pair(c, sn, x, y);
+          hacc[rt][2 * f2] = x;
+          hacc[rt][2 * f2 + 1] = y;
+          return y;
+        }, [&](int b) {
+          asm volatile("" : "+v"(hacc[4 * b]), "+v"(hacc[4 * b + 1]), "+v"(hacc[4 * b + 2]), "+v"(hacc[4 * b + 3]));
+        });
+        // scores of the page in B-operand layout (column lc, tokens 8*lg + e): four partials to sum
+        float sc[8];
+        {
+          uint4v part[kFreqWaves][2];
+#pragma unroll
+          for (int ww = 0; ww < kFreqWaves; ++ww) {
+            part[ww][0] = lds_read_b128_async(&s_part[buf][ww][lc * kPart + 8 * lg]);
+            part[ww][1] = lds_read_b128_async(&s_part[buf][ww][lc * kPart + 8 * lg + 4]);
+          }
+#pragma unroll
+          for (int ww = 0; ww < kFreqWaves; ++ww) {
+            lds_wait_for(part[ww][0]);
+            lds_wait_for(part[ww][1]);
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const uint4v p0 = part[0][e >> 2], p1 = part[1][e >> 2], p2 = part[2][e >> 2], p3 = part[3][e >> 2];
+            const unsigned u0 = p0[e & 3], u1 = p1[e & 3], u2 = p2[e & 3], u3 = p3[e & 3];
+            sc[e] = (__builtin_bit_cast(float, u0) + __builtin_bit_cast(float, u1)) +
+                    (__builtin_bit_cast(float, u2) + __builtin_bit_cast(float, u3));
+          }
+        }
+        uint4v vraw[VMAX];
+        if (has_v) {
+          const unsigned char* st = &s_stage[w][pg % NST][0];
+#pragma unroll
+          for (int f = 0; f < VMAX; ++f) vraw[f] = lds_read_b128_async(st + (size_t)f * 1024 + lane * 16);
+        }
         if (ragged_tail && t == n_tiles - 1) {
           const int tok0 = t * 32 + 8 * lg;
 #pragma unroll
@@ -371,40 +542,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         d_run = d_run * alpha + psum;
         m_run = m_new;
         const bool rescale = __any(alpha != 1.0f);
-        // the g history (rescaled by alpha) moves into the frame of this page
         if (rescale) {
 #pragma unroll
           for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] *= alpha;
-        }
 #pragma unroll
-        for (int rt = 0; rt < 2 * KS; ++rt) {
-          const float4v cs = s_rot[(sl * 2 * KS + rt) * 4 + lg];
-#pragma unroll
-          for (int f2 = 0; f2 < 2; ++f2) {
-            const float c = cs[2 * f2], s = cs[2 * f2 + 1];
-            const float hx = hacc[rt][2 * f2], hy = hacc[rt][2 * f2 + 1];
-            hacc[rt][2 * f2] = c * hx + s * hy;
-            hacc[rt][2 * f2 + 1] = c * hy - s * hx;
-          }
+          for (int f = 0; f < VMAX; ++f) oacc[f] *= alpha;
         }
 #pragma unroll
         for (int rt = 0; rt < 2 * KS; ++rt)
           hacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[rt], pf, hacc[rt], 0, 0, 0);
-        if (has_mn) {
+        if (has_v) {
+#pragma unroll
+          for (int f = 0; f < VMAX; ++f) lds_wait_for(vraw[f]);
 #pragma unroll
           for (int f = 0; f < VMAX; ++f)
-            if (f < ndg) {
-              if (rescale) oacc[f] *= alpha;
-              oacc[f] = M::mma(V0[f], pe, oacc[f]);
-            }
-#pragma unroll
-          for (int f = 0; f < VMAX; ++f) {
-            V0[f] = V1[f];
-            V1[f] = V2[f];
-          }
+            if (f < ndg) oacc[f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f]);
         }
       }
-      __syncthreads();
+      barrier_lds_only();
     }
 
     // ---- partials of this split ------------------------------------------------------
@@ -417,16 +572,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
       float* g = p.pg + base * 2 * N;
       const int64_t last = (int64_t)32 * (t_end > t_beg ? t_end - 1 : t_beg);
+      float sn[2], co[2], s8, c8;   // stepped phases, as for the first page
+      fast_sincos_phase(8, last, p.T, &s8, &c8);
+#pragma unroll
+      for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), last, p.T, &sn[f2], &co[f2]);
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt)
 #pragma unroll
         for (int f2 = 0; f2 < 2; ++f2) {
           const int f = fbase + freq_of(rt, lg, f2);
-          float sn, co;
-          fast_sincos_phase(f, last, p.T, &sn, &co);
           const float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
-          g[f] = co * x - sn * y;       // back from the page frame: rotation by +phi
-          g[N + f] = sn * x + co * y;
+          g[f] = co[f2] * x - sn[f2] * y;       // back from the page frame: rotation by +phi
+          g[N + f] = sn[f2] * x + co[f2] * y;
+          const float cn = co[f2] * c8 - sn[f2] * s8;
+          sn[f2] = sn[f2] * c8 + co[f2] * s8;
+          co[f2] = cn;
         }
       if (has_mn && bb_r == sl) {
         const int vn_len = p.vn_h[h + 1] - p.vn_h[h];
