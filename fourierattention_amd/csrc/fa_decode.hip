@@ -32,23 +32,45 @@ struct Seg {
 //       c0[b, hq]   = sm*log2e * sum_j q[b, hq, d_j] (avg_u - avg_d s)[b, kc0 + j]
 // block = 64 coefficient rows of one (b, KV head); thread = (row, one of 4 column classes):
 // a thread reads every 4th compressed dim of its row (up to 32 independent loads in flight),
-// four neighbouring lanes finish the dot product.  Block x == 0 also clears the merge tickets.
+// four neighbouring lanes finish the dot product.
 // ---------------------------------------------------------------------------
 constexpr int kPrepRows = 64;
 
 template <typename E>
-__global__ __launch_bounds__(256) void decode_prep_kernel(
-    const E* __restrict__ q, const float* __restrict__ k_mc, const float* __restrict__ avg_u,
-    const float* __restrict__ avg_d, const float* __restrict__ scale, const int32_t* __restrict__ kc_list,
-    const int32_t* __restrict__ kc_h, float* __restrict__ W, float* __restrict__ c0, unsigned* __restrict__ tickets,
-    int Hq, int Hkv, int D, int N, int Ck, float sm_log2e) {
+struct PrepArgs {
+  const E* q;
+  const float* k_mc;
+  const float* avg_u;
+  const float* avg_d;
+  const float* scale;
+  const int32_t* kc_list;
+  const int32_t* kc_h;
+  float* W;
+  float* c0;
+  int Hq, Hkv, D, N, Ck;
+  float sm_log2e;
+};
+
+// bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx
+template <typename E>
+__device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx) {
+  const E* __restrict__ q = pa.q;
+  const float* __restrict__ k_mc = pa.k_mc;
+  const float* __restrict__ avg_u = pa.avg_u;
+  const float* __restrict__ avg_d = pa.avg_d;
+  const float* __restrict__ scale = pa.scale;
+  const int32_t* __restrict__ kc_list = pa.kc_list;
+  const int32_t* __restrict__ kc_h = pa.kc_h;
+  float* __restrict__ W = pa.W;
+  float* __restrict__ c0 = pa.c0;
+  const int Hq = pa.Hq, Hkv = pa.Hkv, D = pa.D, N = pa.N, Ck = pa.Ck;
+  const float sm_log2e = pa.sm_log2e;
   __shared__ float s_qs[kGMax][128];
   __shared__ float s_qa[kGMax][128];
   const int tid = threadIdx.x;
   const int h = blockIdx.y, b = blockIdx.z;
   const int G = Hq / Hkv;
   const int kc0 = kc_h[h], kc_len = kc_h[h + 1] - kc0;
-  if (blockIdx.x == 0 && tid == 0) tickets[b * Hkv + h] = 0u;
   for (int e = tid; e < kGMax * 128; e += 256) {
     const int g = e >> 7, j = e & 127;
     float qs = 0.f, qa = 0.f;
@@ -64,13 +86,13 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(
     s_qa[g][j] = qa;
   }
   __syncthreads();
-  if (blockIdx.x == 0 && tid < 64) {
+  if (bx == 0 && tid < 64) {
     for (int g = 0; g < G; ++g) {
       float v = fa_wave_sum(s_qa[g][tid] + s_qa[g][tid + 64]);
       if (tid == 0) c0[(int64_t)b * Hq + h * G + g] = v * sm_log2e;
     }
   }
-  const int n = blockIdx.x * kPrepRows + (tid >> 2), jq = tid & 3;
+  const int n = bx * kPrepRows + (tid >> 2), jq = tid & 3;
   if (n >= 2 * N) return;
   const float* row = k_mc + ((int64_t)b * 2 * N + n) * Ck + kc0;
   float v[32];
@@ -89,6 +111,11 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(
     a = fa_group_sum<4>(a);
     if (jq == 0) W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = a * mul;
   }
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void decode_prep_kernel(const PrepArgs<E> pa) {
+  decode_prep_body<E>(pa, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -399,21 +426,53 @@ __global__ __launch_bounds__(256) void decode_mid_kernel(
 // merge: one block of 1024 threads per (b, KV head) combines, for the G query heads of that head,
 // the partials of every split and applies the V coefficients once:
 //   out_c = s_v * ((1/N) V_coef^T g - avg_d_v * P) + avg_u_v * P
-// Every phase issues its global loads in batches of 16 per thread before using them.
+// The kernel is a chain of short dependent phases, so its time is memory latency: every thread first
+// issues the loads of ALL phases (split maxima, its g / o partials, its V-coefficient rows) into
+// registers and only then starts the first phase; what does not fit the prefetch is looped afterwards.
 // ---------------------------------------------------------------------------
-// sum_s w[s] * ptr[s * stride] with the loads issued sixteen at a time
-__device__ __forceinline__ float weighted_sum(const float* __restrict__ ptr, int64_t stride, const float* w, int n) {
-  float a = 0.f;
-  for (int s0 = 0; s0 < n; s0 += 16) {
-    float v[16];
+constexpr int kMergePre = 16;    // splits held in registers per prefetched element
+constexpr int kMergeRows = 16;   // V-coefficient rows held in registers per thread
+constexpr int kMergeIl = 20;     // sink/window splits held in registers per output element
+
+// n > 0 loads from ptr[min(u, n - 1) * stride], u < CNT: clamped, so that none of them is conditional
+template <int CNT>
+__device__ __forceinline__ void prefetch_strided(float (&v)[CNT], const float* __restrict__ ptr, int64_t stride, int n) {
 #pragma unroll
-    for (int u = 0; u < 16; ++u) v[u] = (s0 + u < n) ? ptr[(int64_t)(s0 + u) * stride] : 0.f;
+  for (int u = 0; u < CNT; ++u) v[u] = ptr[(int64_t)min(u, n - 1) * stride];
+}
+// sum_s w[s] * x[s] over the prefetched head of a strided vector, the tail read from memory
+template <int CNT>
+__device__ __forceinline__ float weighted_sum_pre(const float (&v)[CNT], const float* __restrict__ ptr, int64_t stride,
+                                                  const float* w, int n) {
+  float a = 0.f;
+#pragma unroll
+  for (int u = 0; u < CNT; ++u)
+    if (u < n) a = fmaf(w[u], v[u], a);
+  for (int s0 = CNT; s0 < n; s0 += 16) {
+    float t[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) t[u] = ptr[(int64_t)min(s0 + u, n - 1) * stride];
 #pragma unroll
     for (int u = 0; u < 16; ++u)
-      if (s0 + u < n) a = fmaf(w[s0 + u], v[u], a);
+      if (s0 + u < n) a = fmaf(w[s0 + u], t[u], a);
   }
   return a;
 }
+// the same without a prefetched head
+__device__ __forceinline__ float weighted_sum(const float* __restrict__ ptr, int64_t stride, const float* w, int n) {
+  float a = 0.f;
+  for (int s0 = 0; s0 < n; s0 += 16) {
+    float t[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) t[u] = ptr[(int64_t)min(s0 + u, n - 1) * stride];
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (s0 + u < n) a = fmaf(w[s0 + u], t[u], a);
+  }
+  return a;
+}
+
+constexpr int kMergeChunks = 4;  // blocks per (b, KV head): each applies the V coefficients of a quarter of the dims
 
 __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
@@ -429,58 +488,143 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   float* s_w = s_g + G * 2 * N;          // [G][n_all]
   float* s_d = s_w + G * n_all;          // [G][n_all]
   float* s_sc = s_d + G * n_all;         // [2][kGMax]: sum of d, sum of d over the mid rows
-  float* s_part = s_sc + 2 * kGMax;      // [16][G][128]
-  float* s_o = s_part + 16 * G * 128;    // [G][D]
+  float* s_part = s_sc + 2 * kGMax;      // [parts][G][cwp] = 1024 * G
+  float* s_o = s_part + 1024 * G;        // [G][D]
+  int* s_own = (int*)(s_o + G * D);      // [D]: bit 0 = some list holds the dim, bit 1 = this block writes it
   const int tid = threadIdx.x;
-  const int h = blockIdx.x, b = blockIdx.y;
+  const int h = blockIdx.x, b = blockIdx.y, z = blockIdx.z;
   const int64_t r0 = (int64_t)b * Hq + h * G;
   const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
   const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
+  // this block's share of the compressed and of the stored dims (by position in the head's lists)
+  const int cw = (vc_len + kMergeChunks - 1) / kMergeChunks;
+  const int c_lo = min(vc_len, z * cw), cn = min(vc_len, c_lo + cw) - c_lo;
+  const int nw = (vn_len + kMergeChunks - 1) / kMergeChunks;
+  const int n_lo = min(vn_len, z * nw), nn = min(vn_len, n_lo + nw) - n_lo;
+  const bool has_coef = n_mid_split > 0 && cn > 0;
+  int cwp = 1;                           // power of two >= cw: threads = (dim, row class)
+  while (cwp < cw) cwp <<= 1;
+  const int parts = 1024 / cwp;          // cw <= 128 for head dims up to 512
 
-  for (int idx = tid; idx < G * n_all; idx += 1024) {
-    const int g = idx / n_all, s_ = idx - g * n_all;
+  // ---- every load this thread will need, issued before anything is waited for --------------------------
+  float m_raw = -INFINITY, d_raw = 0.f;            // split maxima / denominators (first G * n_all threads)
+  if (tid < G * n_all) {
+    const int g = tid / n_all, s_ = tid - g * n_all;
     const int64_t r = r0 + g;
     const bool il = s_ < n_il_split;
-    s_w[idx] = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
-    s_d[idx] = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
+    m_raw = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
+    d_raw = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
+  }
+  float g_pre[2][kMergePre];                        // g partials of elements tid and tid + 1024
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int idx = tid + k * 1024;
+    if (has_coef && idx < G * 2 * N) {
+      const int g = idx / (2 * N), n = idx - g * 2 * N;
+      prefetch_strided(g_pre[k], md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N, n_mid_split);
+    }
+  }
+  // V coefficients: rows part, part + parts, ... of dim c_lo + j
+  const int j = tid & (cwp - 1), part = tid / cwp;
+  const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + c_lo + j;
+  float v_pre[kMergeRows];
+  if (has_coef && j < cn) {
+#pragma unroll
+    for (int u = 0; u < kMergeRows; ++u) v_pre[u] = vp[(int64_t)min(part + u * parts, 2 * N - 1) * Cv];
+  }
+  float n_pre[kMergePre];                           // stored-dim outputs of the mid rows
+  if (n_mid_split > 0 && tid < G * nn) {
+    const int g = tid / nn, jj = n_lo + (tid - g * nn);
+    prefetch_strided(n_pre, md_on + (r0 + g) * n_mid_split * D + jj, D, n_mid_split);
+  }
+  float il_pre[kMergeIl];                           // sink/window outputs of element tid
+  if (n_il_split > 0 && tid < G * D) {
+    const int g = tid / D, d = tid - g * D;
+    prefetch_strided(il_pre, il_o + (r0 + g) * n_il_split * D + d, D, n_il_split);
+  }
+
+  // ---- split weights: one wave per query head ----------------------------------------------------------
+  for (int idx = tid; idx < G * n_all; idx += 1024) {
+    if (idx == tid) {
+      s_w[idx] = m_raw;
+      s_d[idx] = d_raw;
+    } else {
+      const int g = idx / n_all, s_ = idx - g * n_all;
+      const int64_t r = r0 + g;
+      const bool il = s_ < n_il_split;
+      s_w[idx] = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
+      s_d[idx] = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
+    }
   }
   for (int idx = tid; idx < G * D; idx += 1024) s_o[idx] = 0.f;
+  for (int idx = tid; idx < D; idx += 1024) s_own[idx] = 0;
   __syncthreads();
-  if (tid < G) {
-    float mstar = -INFINITY;
-    for (int s_ = 0; s_ < n_all; ++s_) mstar = fmaxf(mstar, s_w[tid * n_all + s_]);
-    float dsum = 0.f, pmid = 0.f;
-    for (int s_ = 0; s_ < n_all; ++s_) {
-      const float m = s_w[tid * n_all + s_];
-      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
-      s_w[tid * n_all + s_] = wgt;
-      if (s_ < n_il_split) dsum += wgt * s_d[tid * n_all + s_]; else pmid += wgt * s_d[tid * n_all + s_];
+  // which dims this block writes: its list shares; block 0 also takes dims that no list names
+  for (int idx = tid; idx < vc_len + vn_len; idx += 1024) {
+    const bool c = idx < vc_len;
+    const int pos = c ? idx : idx - vc_len;
+    const int d = (c ? vc_list[vc0 + pos] : vn_list[vn0 + pos]) - h * D;
+    const bool mine = c ? (pos >= c_lo && pos < c_lo + cn) : (pos >= n_lo && pos < n_lo + nn);
+    s_own[d] = mine ? 3 : 1;
+  }
+  {
+    const int g = tid >> 6, lane = tid & 63;
+    if (g < G) {
+      float mstar = -INFINITY;
+      for (int s_ = lane; s_ < n_all; s_ += 64) mstar = fmaxf(mstar, s_w[g * n_all + s_]);
+      mstar = fa_wave_max(mstar);
+      float dsum = 0.f, pmid = 0.f;
+      for (int s_ = lane; s_ < n_all; s_ += 64) {
+        const float m = s_w[g * n_all + s_];
+        const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+        s_w[g * n_all + s_] = wgt;
+        if (s_ < n_il_split) dsum += wgt * s_d[g * n_all + s_]; else pmid += wgt * s_d[g * n_all + s_];
+      }
+      dsum = fa_wave_sum(dsum);
+      pmid = fa_wave_sum(pmid);
+      if (lane == 0) {
+        s_sc[g] = dsum + pmid;
+        s_sc[kGMax + g] = pmid;
+      }
     }
-    s_sc[tid] = dsum + pmid;
-    s_sc[kGMax + tid] = pmid;
   }
   __syncthreads();
 
   if (n_mid_split > 0) {
-    if (vc_len > 0) {
+    if (cn > 0) {
       // g summed over the splits
-      for (int idx = tid; idx < G * 2 * N; idx += 1024) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int idx = tid + k * 1024;
+        if (idx < G * 2 * N) {
+          const int g = idx / (2 * N), n = idx - g * 2 * N;
+          s_g[idx] = weighted_sum_pre(g_pre[k], md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N,
+                                      s_w + g * n_all + n_il_split, n_mid_split);
+        }
+      }
+      for (int idx = tid + 2048; idx < G * 2 * N; idx += 1024) {
         const int g = idx / (2 * N), n = idx - g * 2 * N;
         s_g[idx] = weighted_sum(md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N, s_w + g * n_all + n_il_split, n_mid_split);
       }
       __syncthreads();
-      // g . V_coef: thread = (dim j, row class)
-      const int jw = vc_len > 64 ? 128 : 64, parts = 1024 / jw;
-      const int j = tid % jw, part = tid / jw;
+      // g . V_coef
       float acc[kGMax];
 #pragma unroll
       for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
-      if (j < vc_len) {
-        const float* vp = v_mc + (int64_t)b * 2 * N * Cv + vc0 + j;
-        for (int n0 = part; n0 < 2 * N; n0 += 16 * parts) {
+      if (j < cn) {
+#pragma unroll
+        for (int u = 0; u < kMergeRows; ++u) {
+          const int n = part + u * parts;
+          if (n < 2 * N) {
+#pragma unroll
+            for (int g = 0; g < kGMax; ++g)
+              if (g < G) acc[g] = fmaf(s_g[g * 2 * N + n], v_pre[u], acc[g]);
+          }
+        }
+        for (int n0 = part + kMergeRows * parts; n0 < 2 * N; n0 += 16 * parts) {
           float v[16];
 #pragma unroll
-          for (int u = 0; u < 16; ++u) v[u] = (n0 + u * parts < 2 * N) ? vp[(int64_t)(n0 + u * parts) * Cv] : 0.f;
+          for (int u = 0; u < 16; ++u) v[u] = vp[(int64_t)min(n0 + u * parts, 2 * N - 1) * Cv];
 #pragma unroll
           for (int u = 0; u < 16; ++u)
             if (n0 + u * parts < 2 * N) {
@@ -490,34 +634,55 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
             }
         }
       }
-      // fold the row classes pairwise down to 16 per dim, then finish below
-      if (part < 16 && j < 128) {
+      // the row classes of one dim meet in LDS
 #pragma unroll
-        for (int g = 0; g < kGMax; ++g)
-          if (g < G) s_part[(part * G + g) * 128 + j] = acc[g];
-      }
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) s_part[(part * G + g) * cwp + j] = acc[g];
       __syncthreads();
-      for (int idx = tid; idx < G * vc_len; idx += 1024) {
-        const int g = idx / vc_len, jj = idx - g * vc_len;
+      // 16 lanes per (head, dim) fold the row classes
+      for (int idx = tid; idx < G * cwp * 16; idx += 1024) {
+        const int sub = idx & 15, gj = idx >> 4;
+        const int g = gj / cwp, jj = gj - g * cwp;
         float a = 0.f;
-        for (int pp = 0; pp < parts; ++pp) a += s_part[(pp * G + g) * 128 + jj];
-        a /= (float)N;
-        const int64_t o = (int64_t)b * Cv + vc0 + jj;
-        const float pmid = s_sc[kGMax + g];
-        s_o[g * D + (vc_list[vc0 + jj] - h * D)] = scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid;
+        for (int pp = sub; pp < parts; pp += 16) a += s_part[(pp * G + g) * cwp + jj];
+        a = fa_group_sum<16>(a);
+        if (sub == 0 && jj < cn) {
+          a /= (float)N;
+          const int64_t o = (int64_t)b * Cv + vc0 + c_lo + jj;
+          const float pmid = s_sc[kGMax + g];
+          s_o[g * D + (vc_list[vc0 + c_lo + jj] - h * D)] = scale[o] * (a - avg_d[o] * pmid) + avg_u[o] * pmid;
+        }
       }
     }
-    for (int idx = tid; idx < G * vn_len; idx += 1024) {
-      const int g = idx / vn_len, jj = idx - g * vn_len;
+    if (tid < G * nn) {
+      const int g = tid / nn, jj = n_lo + (tid - g * nn);
+      s_o[g * D + (vn_list[vn0 + jj] - h * D)] = weighted_sum_pre(n_pre, md_on + (r0 + g) * n_mid_split * D + jj, D,
+                                                                  s_w + g * n_all + n_il_split, n_mid_split);
+    }
+    for (int idx = tid + 1024; idx < G * nn; idx += 1024) {
+      const int g = idx / nn, jj = n_lo + (idx - g * nn);
       s_o[g * D + (vn_list[vn0 + jj] - h * D)] =
           weighted_sum(md_on + (r0 + g) * n_mid_split * D + jj, D, s_w + g * n_all + n_il_split, n_mid_split);
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < G * D; idx += 1024) {
+  if (tid < G * D) {
+    const int g = tid / D, d = tid - g * D;
+    const int own = s_own[d];
+    if ((own & 2) || (z == 0 && own == 0)) {
+      float a = s_o[tid];
+      if (n_il_split > 0) a += weighted_sum_pre(il_pre, il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
+      out[(r0 + g) * D + d] = a / s_sc[g];
+    }
+  }
+  for (int idx = tid + 1024; idx < G * D; idx += 1024) {
     const int g = idx / D, d = idx - g * D;
-    const float a = s_o[idx] + weighted_sum(il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
-    out[(r0 + g) * D + d] = a / s_sc[g];
+    const int own = s_own[d];
+    if ((own & 2) || (z == 0 && own == 0)) {
+      float a = s_o[idx];
+      if (n_il_split > 0) a += weighted_sum(il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
+      out[(r0 + g) * D + d] = a / s_sc[g];
+    }
   }
 }
 
@@ -529,17 +694,34 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kIlFastTile = 64;
 
+template <typename E>
+struct IlArgs {
+  const E* q;
+  Seg s0, s1;
+  float* pm;
+  float* pd;
+  float* po;
+  int Hq, Hkv, n_split;
+  float sm_log2e;
+};
+
+// bx: block index along x (tile of kIlFastTile rows); y, z come from blockIdx
 template <typename E, int D, int GM>
-__global__ __launch_bounds__(256) void decode_il_fast_kernel(
-    const E* __restrict__ q, Seg s0, Seg s1, float* __restrict__ pm, float* __restrict__ pd,
-    float* __restrict__ po, int Hq, int Hkv, int n_split, float sm_log2e) {
+__device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx) {
+  const E* __restrict__ q = ia.q;
+  const Seg s0 = ia.s0, s1 = ia.s1;
+  float* __restrict__ pm = ia.pm;
+  float* __restrict__ pd = ia.pd;
+  float* __restrict__ po = ia.po;
+  const int Hq = ia.Hq, Hkv = ia.Hkv, n_split = ia.n_split;
+  const float sm_log2e = ia.sm_log2e;
   constexpr int LPT = D / 8, TPW = 64 / LPT, ITERS = kIlFastTile / 4 / TPW;
   __shared__ float s_m[4][GM], s_d[4][GM];
   __shared__ float s_o[4][GM][D];
   const int G = Hq / Hkv;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int sub = lane % LPT, tl = lane / LPT;
-  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int split = bx, h = blockIdx.y, b = blockIdx.z;
   const int n_il = s0.rows + s1.rows;
   const int base = split * kIlFastTile + w * (kIlFastTile / 4);
   uint4 kraw[ITERS], vraw[ITERS];
@@ -655,6 +837,20 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(
   }
 }
 
+template <typename E, int D, int GM>
+__global__ __launch_bounds__(256) void decode_il_fast_kernel(const IlArgs<E> ia) {
+  decode_il_fast_body<E, D, GM>(ia, blockIdx.x);
+}
+
+// The coefficient-domain query and the sink/window rows do not depend on each other and are both short,
+// latency-bound pieces of work: one launch runs them side by side (blocks [0, n_prep) prepare the query,
+// the rest attend over sink/window tiles).
+template <typename E, int D, int GM>
+__global__ __launch_bounds__(256) void decode_prep_il_kernel(const PrepArgs<E> pa, const IlArgs<E> ia, int n_prep) {
+  if ((int)blockIdx.x < n_prep) decode_prep_body<E>(pa, blockIdx.x);
+  else decode_il_fast_body<E, D, GM>(ia, blockIdx.x - n_prep);
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -678,7 +874,7 @@ struct Plan {
   Path path;
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
   int n_merge_chunks;
-  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, off_tick, total;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, total;
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
@@ -731,7 +927,6 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
   p.n_merge_chunks = 1;
   p.off_cpart = take(256);
-  p.off_tick = take((size_t)B * Hkv * 4);
   p.total = o;
   return p;
 }
@@ -781,13 +976,28 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   float* mg = (float*)(ws + p.off_mg);
   float* mon = (float*)(ws + p.off_mon);
   float* cpart = (float*)(ws + p.off_cpart);
-  unsigned* tickets = (unsigned*)(ws + p.off_tick);
   const int G = a.Hq / a.Hkv;
   const float sm_log2e = sm_scale * kLog2e;
+  Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
+  Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
+  IlArgs<E> ia{(const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e};
+  // sink/window tiles ride in the query-preparation launch when both exist and the fast tile kernel applies
+  const bool fuse_il = sizeof(E) == 2 && p_il_fast && p.n_il_split > 0 && p.n_mid_split > 0;
   if (p.n_mid_split > 0) {
-    decode_prep_kernel<E><<<dim3(fa_cdiv(2 * a.N, kPrepRows), a.Hkv, a.B), 256, 0, st>>>(
-        (const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0, tickets, a.Hq, a.Hkv,
-        a.D, a.N, a.Ck, sm_log2e);
+    PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
+                   a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e};
+    const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
+    if (fuse_il) {
+      if constexpr (sizeof(E) == 2) {
+        dim3 grid(n_prep + p.n_il_split, a.Hkv, a.B);
+        if (a.D == 128 && G <= 4) decode_prep_il_kernel<E, 128, 4><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        else if (a.D == 128) decode_prep_il_kernel<E, 128, kGMax><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        else if (G <= 4) decode_prep_il_kernel<E, 64, 4><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        else decode_prep_il_kernel<E, 64, kGMax><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+      }
+    } else {
+      decode_prep_kernel<E><<<dim3(n_prep, a.Hkv, a.B), 256, 0, st>>>(pa);
+    }
     if (p.path == Path::Mfma) {
       if constexpr (sizeof(E) == 2) {
         using namespace fa_mfma;
@@ -839,22 +1049,16 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   }
   if (ev && (p.n_mid_split == 0 || p.path != Path::Mfma)) hipEventRecord(ev[1], st);
   if (ev) hipEventRecord(ev[2], st);
-  if (p.n_il_split > 0) {
-    Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
-    Seg s1{a.k_il[1], a.v_il[1], a.il_rows[1], a.il_batch_stride[1], a.il_row_stride[1]};
+  if (p.n_il_split > 0 && !fuse_il) {
     dim3 grid(p.n_il_split, a.Hkv, a.B);
     bool launched = false;
     if constexpr (sizeof(E) == 2) {
       if (p_il_fast) {
         launched = true;
-        if (a.D == 128 && G <= 4)
-          decode_il_fast_kernel<E, 128, 4><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
-        else if (a.D == 128)
-          decode_il_fast_kernel<E, 128, kGMax><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
-        else if (G <= 4)
-          decode_il_fast_kernel<E, 64, 4><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
-        else
-          decode_il_fast_kernel<E, 64, kGMax><<<grid, 256, 0, st>>>((const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e);
+        if (a.D == 128 && G <= 4) decode_il_fast_kernel<E, 128, 4><<<grid, 256, 0, st>>>(ia);
+        else if (a.D == 128) decode_il_fast_kernel<E, 128, kGMax><<<grid, 256, 0, st>>>(ia);
+        else if (G <= 4) decode_il_fast_kernel<E, 64, 4><<<grid, 256, 0, st>>>(ia);
+        else decode_il_fast_kernel<E, 64, kGMax><<<grid, 256, 0, st>>>(ia);
       }
     }
     if (!launched) {
@@ -865,13 +1069,13 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   if (ev) hipEventRecord(ev[3], st);
   {
     const int n_all = p.n_il_split + p.n_mid_split;
-    size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 16 * (size_t)G * 128 + (size_t)G * a.D) * sizeof(float);
+    size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 1024 * (size_t)G + (size_t)G * a.D + a.D) * sizeof(float);
     if (lds > 64 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_merge_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
     }
-    decode_merge_kernel<<<dim3(a.Hkv, a.B), 1024, lds, st>>>(
+    decode_merge_kernel<<<dim3(a.Hkv, a.B, kMergeChunks), 1024, lds, st>>>(
         ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
         a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv);
   }
