@@ -716,8 +716,8 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
   const int Hq = ia.Hq, Hkv = ia.Hkv, n_split = ia.n_split;
   const float sm_log2e = ia.sm_log2e;
   constexpr int LPT = D / 8, TPW = 64 / LPT, ITERS = kIlFastTile / 4 / TPW;
-  __shared__ float s_m[4][GM], s_d[4][GM];
-  __shared__ float s_o[4][GM][D];
+  __shared__ float s_m[4][GM], s_d[4][TPW / 2][GM];
+  __shared__ __attribute__((aligned(16))) float s_o[4][TPW / 2][GM][D];
   const int G = Hq / Hkv;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int sub = lane % LPT, tl = lane / LPT;
@@ -734,89 +734,91 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
     kraw[it] = *(const uint4*)((in0 ? (const E*)s0.k : (const E*)s1.k) + off + h * D + sub * 8);
     vraw[it] = *(const uint4*)((in0 ? (const E*)s0.v : (const E*)s1.v) + off + h * D + sub * 8);
   }
-  float qv[GM][8];
+  // the query slices: one unconditional 16-byte load per head (a head index past G repeats the last one)
+  uint4 qraw[GM];
 #pragma unroll
   for (int g = 0; g < GM; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      qv[g][e] = g < G ? fa_to_float(q[((int64_t)b * Hq + h * G + g) * D + sub * 8 + e]) * sm_log2e : 0.f;
-  float m[GM], d[GM], o[GM][8];
+    qraw[g] = *(const uint4*)(q + ((int64_t)b * Hq + h * G + min(g, G - 1)) * D + sub * 8);
+  float qv[GM][8];
 #pragma unroll
   for (int g = 0; g < GM; ++g) {
-    m[g] = -INFINITY;
+    const E* qe = (const E*)&qraw[g];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[g][e] = g < G ? fa_to_float(qe[e]) * sm_log2e : 0.f;
+  }
+  // The wave holds only ITERS * TPW rows, so it takes one softmax block: all scores first, one maximum,
+  // then the weighted sum (no running maximum, no rescaling).
+  float sc[ITERS][GM], m[GM];
+#pragma unroll
+  for (int g = 0; g < GM; ++g) m[g] = -INFINITY;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const bool ok = base + it * TPW + tl < n_il;
+    const E* ke = (const E*)&kraw[it];
+    float kf[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) kf[e] = fa_to_float(ke[e]);
+#pragma unroll
+    for (int g = 0; g < GM; ++g) {
+      float a = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a = fmaf(kf[e], qv[g][e], a);
+      a = fa_group_sum<LPT>(a);
+      sc[it][g] = (ok && g < G) ? a : -INFINITY;
+      m[g] = fmaxf(m[g], sc[it][g]);
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < GM; ++g) {
+    if (LPT == 8) m[g] = fmaxf(m[g], fa_dpp<FA_DPP_ROR8>(m[g]));
+    m[g] = fa_rows_max(m[g]);
+  }
+  float d[GM], o[GM][8];
+#pragma unroll
+  for (int g = 0; g < GM; ++g) {
     d[g] = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
   }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const bool ok = base + it * TPW + tl < n_il;
-    const E* ke = (const E*)&kraw[it];
     const E* ve = (const E*)&vraw[it];
-    float kf[8], vf[8];
+    float vf[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      kf[e] = fa_to_float(ke[e]);
-      vf[e] = fa_to_float(ve[e]);
-    }
-    float sc[GM], mx[GM];
-    bool changed = false;
+    for (int e = 0; e < 8; ++e) vf[e] = fa_to_float(ve[e]);
 #pragma unroll
     for (int g = 0; g < GM; ++g) {
-      if (g < G) {
-        float a = 0.f;
+      const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[it][g] - m[g]);
+      d[g] += pv;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a = fmaf(kf[e], qv[g][e], a);
-        a = fa_group_sum<LPT>(a);
-        sc[g] = ok ? a : -INFINITY;
-        float t = sc[g];
-        if (LPT == 8) t = fmaxf(t, fa_dpp<FA_DPP_ROR8>(t));
-        t = fa_rows_max(t);
-        mx[g] = fmaxf(m[g], t);
-        changed |= mx[g] != m[g];
-      }
+      for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pv, vf[e], o[g][e]);
     }
-    if (changed) {  // wave-uniform: every lane sees the same maxima
-#pragma unroll
-      for (int g = 0; g < GM; ++g)
-        if (g < G) {
-          const float al = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[g] - mx[g]);
-          d[g] *= al;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) o[g][e] *= al;
-          m[g] = mx[g];
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < GM; ++g)
-      if (g < G) {
-        const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[g] - m[g]);
-        d[g] += pv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pv, vf[e], o[g][e]);
-      }
   }
-  // reduce over the rows a wave holds side by side, then over the four waves
+  // rows held side by side in the wave: lanes i and i + 32 meet in registers, the rest in LDS together
+  // with the four waves
 #pragma unroll
-  for (int g = 0; g < GM; ++g)
-    if (g < G) {
-      if (LPT == 8) {
-        d[g] += fa_dpp<FA_DPP_ROR8>(d[g]);
+  for (int g = 0; g < GM; ++g) {
+    float lo, hi;
+    fa_swap32(d[g], &lo, &hi);
+    d[g] = lo + hi;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[g][e] += fa_dpp<FA_DPP_ROR8>(o[g][e]);
-      }
-      d[g] = fa_rows_sum(d[g]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[g][e] = fa_rows_sum(o[g][e]);
-      if (tl == 0) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_o[w][g][sub * 8 + e] = o[g][e];
-        if (sub == 0) {
-          s_m[w][g] = m[g];
-          s_d[w][g] = d[g];
-        }
-      }
+    for (int e = 0; e < 8; ++e) {
+      fa_swap32(o[g][e], &lo, &hi);
+      o[g][e] = lo + hi;
     }
+  }
+  if (lane < 32) {
+#pragma unroll
+    for (int g = 0; g < GM; ++g) {
+      *(float4*)&s_o[w][tl][g][sub * 8] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+      *(float4*)&s_o[w][tl][g][sub * 8 + 4] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+      if (sub == 0) s_d[w][tl][g] = d[g];
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int g = 0; g < GM; ++g) s_m[w][g] = m[g];
+    }
+  }
   __syncthreads();
   for (int idx = tid; idx < G * D; idx += 256) {
     const int g = idx / D, dim = idx % D;
@@ -825,8 +827,14 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
 #pragma unroll
     for (int ww = 0; ww < 4; ++ww) {
       const float wgt = s_m[ww][g] == -INFINITY ? 0.f : exp2f(s_m[ww][g] - mm);
-      acc = fmaf(wgt, s_o[ww][g][dim], acc);
-      dd = fmaf(wgt, s_d[ww][g], dd);
+      float os = 0.f, ds = 0.f;
+#pragma unroll
+      for (int t = 0; t < TPW / 2; ++t) {
+        os += s_o[ww][t][g][dim];
+        ds += s_d[ww][t][g];
+      }
+      acc = fmaf(wgt, os, acc);
+      dd = fmaf(wgt, ds, dd);
     }
     const int64_t r = ((int64_t)b * Hq + h * G + g) * n_split + split;
     po[r * D + dim] = acc;
@@ -933,6 +941,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
 
 bool il_fast_ok(const fa_decode_args& a) {
   if (a.dtype == FA_FP32 || (a.D != 64 && a.D != 128)) return false;
+  if ((uintptr_t)a.q & 15) return false;   // query rows are read 16 bytes at a time
   for (int i = 0; i < 2; ++i) {
     if (a.il_rows[i] == 0) continue;
     if (((uintptr_t)a.k_il[i] & 15) || ((uintptr_t)a.v_il[i] & 15)) return false;
