@@ -271,6 +271,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   if (score_wave) {
     // =============================== score waves ===============================
+    // stored K dims of batch element sl: both 16-token blocks of the page.  The first pages are requested
+    // before anything else, so that HBM is busy while the tables and the query are being set up.
+    const int kn0 = p.kn_h[h], kn_len = p.kn_h[h + 1] - kn0;
+    const int kp0 = p.kpad_h[h], dpk = p.kpad_h[h + 1] - kp0;
+    const int nks = dpk >> 5;
+    const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
+    const bool has_k = has_mn && nks > 0;
+    // every page moves 2*KMAX fragments so that the number of loads in flight is a compile-time constant;
+    // a head with fewer stored dims repeats its first fragment into the unused slots
+    auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
+      const E* kp = kbase + (int64_t)t * dpk * 32;
+      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int ks = 0; ks < KMAX; ++ks)
+          load_frag_to_lds(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
+    };
+    if (has_k) {
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i)
+        if (i < n_it) issue_k(t_beg + i);
+    }
     half8 Ea[2][KS];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
@@ -286,8 +309,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) {
         const int f = fbase + freq_of(rt, lg, 0);
-        float2v c2 = valid_r ? *(const float2v*)(wr + f) : float2v{0.f, 0.f};
-        float2v s2 = valid_r ? *(const float2v*)(wr + N + f) : float2v{0.f, 0.f};
+        float2v c2 = *(const float2v*)(wr + f);      // row 0 stands in for columns past the group
+        float2v s2 = *(const float2v*)(wr + N + f);
+        if (!valid_r) c2 = s2 = float2v{0.f, 0.f};
         Wc[rt][0] = c2[0]; Wc[rt][1] = c2[1];
         Ws[rt][0] = s2[0]; Ws[rt][1] = s2[1];
         wmax = fmaxf(wmax, fmaxf(fmaxf(fabsf(c2[0]), fabsf(c2[1])), fmaxf(fabsf(s2[0]), fabsf(s2[1]))));
@@ -320,10 +344,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
-    // stored K dims of batch element sl: both 16-token blocks of the page
-    const int kn0 = p.kn_h[h], kn_len = p.kn_h[h + 1] - kn0;
-    const int kp0 = p.kpad_h[h], dpk = p.kpad_h[h + 1] - kp0;
-    const int nks = dpk >> 5;
     // the gathered query dims: all index loads first, then all query loads (clamped so that none is
     // conditional: conditional loads would be issued one round trip after the other)
     vec8 Qb[KMAX];
@@ -351,30 +371,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int e = 0; e < 8; ++e)
           if (mine && s * 32 + 8 * lg + e < kn_len) Qb[s][e] = M::from_bits(qv[s][e]);
     }
-    const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
-    const bool has_k = has_mn && nks > 0;
-    // every page moves 2*KMAX fragments so that the number of loads in flight is a compile-time constant;
-    // a head with fewer stored dims repeats its first fragment into the unused slots
-    auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
-      const E* kp = kbase + (int64_t)t * dpk * 32;
-      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-        for (int ks = 0; ks < KMAX; ++ks)
-          load_frag_to_lds(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
-    };
-    // every table and weight load above must have landed before the page loads start: afterwards the
-    // only waits on vector memory in this wave are the explicit page waits
+    // every table and weight load above must have landed before the loop starts: inside it the only
+    // waits on vector memory in this wave are the explicit page waits
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
-    if (has_k) {
-#pragma unroll
-      for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_k(t_beg + i);
-    }
     const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
@@ -437,9 +439,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
   } else {
     // =============================== value waves ===============================
-    half8 ETa[2 * KS];
-#pragma unroll
-    for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
     const int vp0 = p.vpad_h[h], dpv = p.vpad_h[h + 1] - vp0;
     const int ndg = dpv >> 4;
     const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
@@ -451,6 +450,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int f = 0; f < VMAX; ++f) load_frag_to_lds(vp + (f < ndg ? f : 0) * 512 + lane * 8, st + f * 1024);
     };
+    if (has_v) {   // first pages requested before the tables (see the score waves)
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i)
+        if (i < n_it) issue_v(t_beg + i);
+    }
+    half8 ETa[2 * KS];
+#pragma unroll
+    for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -459,14 +466,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float m_run = -INFINITY, d_run = 0.f;
     const bool ragged_tail = (p.L_m & 31) != 0;
     __syncthreads();  // pairs with the score waves' column-scale exchange
-    // the table loads must have landed before the page loads start (see the score waves)
+    // the table loads must have landed before the loop starts (see the score waves)
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
-    if (has_v) {
-#pragma unroll
-      for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_v(t_beg + i);
-    }
     const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
