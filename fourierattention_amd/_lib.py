@@ -61,7 +61,8 @@ _SIGNATURES = {
     "fa_abi_version": (c_int, []),
     "fa_decode_args_size": (c_size_t, []),
     "fa_mat_fourier": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                               c_int64, c_int, c_void_p]),
+                               c_int64, c_int, c_void_p, c_size_t, c_void_p]),
+    "fa_mat_fourier_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "fa_mat_avg_std": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                c_int, c_void_p, c_size_t, c_void_p]),
     "fa_mat_fourier_avg_std": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,

@@ -24,6 +24,13 @@ int fa_check_launch(const char* what);
     }                                    \
   } while (0)
 
+// matrix-core spectral compression (fa_spectral_mfma.hip)
+bool fa_spectral_mfma_ok(int a_dtype, int K, int Mc, int N);
+size_t fa_spectral_mfma_workspace(int B, int K, int Mc, int N);
+int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols, float* c, int B,
+                            int K, int Mc, int N, int T, int64_t k_start, int accumulate, void* workspace,
+                            hipStream_t st);
+
 static inline hipStream_t fa_hip_stream(fa_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 static inline int fa_cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 static inline size_t fa_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -18,35 +18,11 @@
 // ready-made MFMA A operands (see the page layout in the public header).
 #pragma once
 
-#include "fa_common.h"
+#include "fa_mfma_util.h"
 
 namespace fa_mfma {
 
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
-typedef float float2v __attribute__((ext_vector_type(2)));
-
 constexpr int kPart = 36;  // padded row (tokens) of the LDS score partials, floats
-
-template <typename E> struct Mma;
-template <> struct Mma<bf16_t> {
-  using vec8 = bf16x8;
-  using elem = __bf16;
-  static __device__ __forceinline__ float4v mma(vec8 a, vec8 b, float4v c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ elem from_bits(bf16_t x) { return __builtin_bit_cast(__bf16, x.bits); }
-};
-template <> struct Mma<f16_t> {
-  using vec8 = half8;
-  using elem = _Float16;
-  static __device__ __forceinline__ float4v mma(vec8 a, vec8 b, float4v c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ elem from_bits(f16_t x) { return x.v; }
-};
 
 // frequency owned by (kstep s, lane group lg, register v) of the score GEMM's K dimension and by
 // (row tile rt = 2s + v/2, lane group lg, pair v%2) of the g GEMM's rows: per lane the same set
@@ -105,38 +81,6 @@ static inline size_t tables_bytes(int N) {
   return (size_t)(2 * kFreqWaves * 2 * KS * 64) * 16 + (size_t)N * 8;
 }
 
-
-// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt 15 << 8 | vmcnt[5:4] << 14)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-// one fragment (64 lanes x 16 bytes) from global memory straight into LDS at lds_frag + lane * 16
-template <typename E>
-__device__ __forceinline__ void load_frag_to_lds(const E* g_lane_ptr, void* lds_frag) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g_lane_ptr,
-                                   (__attribute__((address_space(3))) void*)lds_frag, 16, 0, 0);
-}
-
-// LDS accesses that the compiler must not tie to the asynchronous page loads (it would otherwise wait
-// for every outstanding global_load_lds before each read and before each barrier)
-typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4v lds_read_b128_async(const void* lds_ptr) {
-  uint4v r;
-  const unsigned addr = (unsigned)(size_t)(const __attribute__((address_space(3))) void*)lds_ptr;
-  asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
-  return r;
-}
-// the read above completes asynchronously: tie the wait to the value so no use can be scheduled before it
-__device__ __forceinline__ void lds_wait_for(uint4v& r) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r)::"memory"); }
-// same for a batch of four reads, leaving the AFTER LDS operations issued after the batch in flight (LDS
-// operations complete in issue order, so a count is enough; later LDS traffic only makes the wait longer)
-template <int AFTER>
-__device__ __forceinline__ void lds_wait_for4(uint4v (&r)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(AFTER) : "memory");
-}
-// workgroup barrier that orders LDS traffic only (global loads stay in flight)
-__device__ __forceinline__ void barrier_lds_only() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // ---- page-step rotation of coefficient-domain state ---------------------------------------------------
 // Both wave roles turn 2*KS row tiles of (cos, sin) pairs by the per-frequency angle of one page.  The
@@ -210,13 +154,6 @@ struct MidParams {
   int B, Hq, Hkv, D, G, nbpg, N, L_m, T, n_split, tiles_per_split;
   float sm_log2e;
 };
-
-// native sin/cos of 2*pi*((a*b) mod T)/T (hardware takes the angle in revolutions)
-__device__ __forceinline__ void fast_sincos_phase(int64_t a, int64_t b, int T, float* s, float* c) {
-  const float x = (float)fa_phase_mod(a, b, T) / (float)T;
-  *s = __builtin_amdgcn_sinf(x);
-  *c = __builtin_amdgcn_cosf(x);
-}
 
 // The workgroup is a two-stage pipeline over the pages of its split, one barrier per page:
 //   waves 0-3 ("score waves")  page t+1: S partial = E . W' (their frequency slice) + K_mn . Q_n (their batch

@@ -273,10 +273,17 @@ extern "C" size_t fa_stats_workspace_bytes(int B, int Mc, int K) {
 
 extern "C" int fa_mat_fourier(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols,
                               float* c, int B, int K, int Mc, int N, int T, int64_t k_start, int accumulate,
-                              fa_stream_t stream) {
+                              void* workspace, size_t workspace_bytes, fa_stream_t stream) {
   FA_REQUIRE(a && c, FA_ERR_NULL_POINTER, "fa_mat_fourier: null pointer");
   FA_REQUIRE(B > 0 && K >= 0 && Mc > 0 && N > 0 && T > 0, FA_ERR_BAD_SHAPE,
              "fa_mat_fourier: bad shape B=%d K=%d Mc=%d N=%d T=%d", B, K, Mc, N, T);
+  FA_REQUIRE(a_dtype == FA_BF16 || a_dtype == FA_FP16 || a_dtype == FA_FP32, FA_ERR_BAD_DTYPE, "fa_mat_fourier: dtype %d",
+             a_dtype);
+  if (workspace && fa_spectral_mfma_ok(a_dtype, K, Mc, N) && workspace_bytes >= fa_spectral_mfma_workspace(B, K, Mc, N)) {
+    FA_REQUIRE(((uintptr_t)workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_mat_fourier: workspace not 256-byte aligned");
+    return fa_spectral_mfma_launch(a, a_dtype, a_bs, a_rs, cols, c, B, K, Mc, N, T, k_start, accumulate, workspace,
+                                   fa_hip_stream(stream));
+  }
   constexpr int MT = 4, NT = 8;
   dim3 grid(fa_cdiv(Mc, 64 * MT), fa_cdiv(N, 4 * NT), B), block(256);
   hipStream_t s = fa_hip_stream(stream);
@@ -294,6 +301,11 @@ extern "C" int fa_mat_fourier(const void* a, int a_dtype, int64_t a_bs, int64_t 
       FA_REQUIRE(false, FA_ERR_BAD_DTYPE, "fa_mat_fourier: dtype %d", a_dtype);
   }
   return fa_check_launch("fa_mat_fourier");
+}
+
+extern "C" size_t fa_mat_fourier_workspace_bytes(int a_dtype, int B, int K, int Mc, int N) {
+  if (B <= 0 || K <= 0 || Mc <= 0 || N <= 0 || !fa_spectral_mfma_ok(a_dtype, K, Mc, N)) return 0;
+  return fa_spectral_mfma_workspace(B, K, Mc, N);
 }
 
 extern "C" int fa_mat_avg_std(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols,

@@ -67,11 +67,13 @@ def as_i32(t: torch.Tensor) -> torch.Tensor:
 
 # --------------------------------------------------------------------------- K1
 def mat_fourier(a: torch.Tensor, N: int, T: int, K_start: int = 0, cols: Optional[torch.Tensor] = None,
-                out: Optional[torch.Tensor] = None, accumulate: bool = False, K: Optional[int] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None, accumulate: bool = False, K: Optional[int] = None,
+                matrix_cores: bool = True) -> torch.Tensor:
     """``c[b, n, m] (+)= sum_k cos(2 pi (k + K_start) n / T) a[b, k, cols[m]]`` and the sin rows.
 
     ``a (B, K, width)`` may be a strided view as long as its last dim is contiguous; ``cols``
-    (int32, GPU) selects columns; ``K`` limits the rows read."""
+    (int32, GPU) selects columns; ``K`` limits the rows read.  Long 16-bit inputs run on the matrix
+    cores (fp16 basis, fp32 accumulation) unless ``matrix_cores`` is false."""
     _require_gpu(a, "a")
     assert a.dim() == 3 and a.stride(2) == 1, "a must be (B, K, M) with a contiguous last dim"
     B, rows, width = a.shape
@@ -84,8 +86,10 @@ def mat_fourier(a: torch.Tensor, N: int, T: int, K_start: int = 0, cols: Optiona
     if Mc == 0 or B == 0:
         return out
     lib = _lib.load()
+    ws_bytes = int(lib.fa_mat_fourier_workspace_bytes(dtype_code(a.dtype), B, K, Mc, N)) if matrix_cores else 0
+    ws = workspace(a.device, ws_bytes, "spectral") if ws_bytes else None
     check(lib.fa_mat_fourier(a.data_ptr(), dtype_code(a.dtype), a.stride(0), a.stride(1), _ptr(cols), out.data_ptr(), B, K,
-                             Mc, N, int(T), int(K_start), int(accumulate), _stream(a.device)))
+                             Mc, N, int(T), int(K_start), int(accumulate), _ptr(ws), ws_bytes, _stream(a.device)))
     return out
 
 

@@ -55,10 +55,18 @@ int fa_abi_version(void);
  * a_batch_stride (elements); if `cols` is non-NULL it holds Mc int32 column
  * indices into the row (the gather `x[:, :, idx]` of CACHE:561 fused in),
  * otherwise columns 0..Mc-1 are read.  c: (B, 2N, Mc) fp32 contiguous.
- * accumulate != 0 adds into c (the `base_input + ...` of TRI:856). */
+ * accumulate != 0 adds into c (the `base_input + ...` of TRI:856).
+ * workspace (optional): with at least fa_mat_fourier_workspace_bytes(B, K, Mc, N)
+ * bytes (256-byte aligned), 16-bit inputs of K >= 512 rows with N % 8 == 0 and
+ * Mc even run on the matrix cores (basis rounded to fp16, fp32 accumulation);
+ * without it, and for every other shape, an fp32 vector kernel is used. */
 int fa_mat_fourier(const void* a, int a_dtype, int64_t a_batch_stride, int64_t a_row_stride,
                    const int32_t* cols, float* c, int B, int K, int Mc, int N, int T,
-                   int64_t k_start, int accumulate, fa_stream_t stream);
+                   int64_t k_start, int accumulate, void* workspace, size_t workspace_bytes,
+                   fa_stream_t stream);
+
+/* 0 when the matrix-core path does not apply to the shape. */
+size_t fa_mat_fourier_workspace_bytes(int a_dtype, int B, int K, int Mc, int N);
 
 /* mat_avg_std_triton(a) (TRI:433-461): per (b, m) mean over k and
  * max(max - mean, mean - min).  Outputs fp32 (B, Mc); when round_dtype is

@@ -141,9 +141,9 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_decode_attn(ctypes.byref(a), None) == -4          # workspace missing
     a.Hq, a.Hkv = 64, 2
     assert lib.fa_decode_attn(ctypes.byref(a), None) == -5          # 32 query heads per KV head
-    assert lib.fa_mat_fourier(None, 0, 0, 0, None, None, 1, 1, 1, 1, 1, 0, 0, None) == -1
-    assert lib.fa_mat_fourier(p, 0, 0, 0, None, p, 1, 1, 1, 0, 1, 0, 0, None) == -2
-    assert lib.fa_mat_fourier(p, 7, 0, 0, None, p, 1, 1, 1, 1, 1, 0, 0, None) == -3
+    assert lib.fa_mat_fourier(None, 0, 0, 0, None, None, 1, 1, 1, 1, 1, 0, 0, None, 0, None) == -1
+    assert lib.fa_mat_fourier(p, 0, 0, 0, None, p, 1, 1, 1, 0, 1, 0, 0, None, 0, None) == -2
+    assert lib.fa_mat_fourier(p, 7, 0, 0, None, p, 1, 1, 1, 1, 1, 0, 0, None, 0, None) == -3
     assert lib.fa_mat_avg_std(p, 0, 0, 0, None, p, p, 1, 4, 4, 2, None, 0, None) == -4
     assert lib.fa_coeff_update(p, None, 0, 0, None, 1, 1, 1, 0, 1, None) == -1
     assert lib.fa_stats_workspace_bytes(2, 10, 1000) == 3 * 2 * 4 * 10 * 4

@@ -144,3 +144,33 @@ def test_decode_attention_window_only_and_errors():
                             tuple(ops.as_i32(g[k]) for k in ("kc_list", "kc_h_list", "kn_list", "kn_h_list", "vc_list", "vc_h_list", "vn_list", "vn_h_list")),
                             8, 2, 0, 1)
     assert ei.value.code == -2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,K,Mc,N,T,k0,gather", [
+    (2, 1500, 96, 40, 1501, 0, True),       # ragged everything: last step partly empty, 5 row tiles, 6 column tiles
+    (1, 4096, 512, 128, 4096, 0, True),     # whole tiles, several chunks
+    (1, 700, 30, 8, 9000, 12345, False),    # phase offset, fewer columns than one workgroup tile
+])
+def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
+    """Long 16-bit inputs take the matrix-core kernels (basis in fp16, fp32 accumulation): checked against the
+    oracle and against the fp32 vector kernel on the same input.  Bound: the fp16 basis carries a relative
+    rounding error of at most 2^-11 per entry, about 1.5e-4 rms, which is what the result inherits."""
+    from fourierattention_amd import ops
+    r = np.random.default_rng(5)
+    width = Mc + 37 if gather else Mc
+    x = H.to_dtype_np(r.standard_normal((B, K, width)), dtype)
+    cols = np.sort(r.choice(width, Mc, replace=False)) if gather else None
+    xs = x[:, :, cols] if gather else x
+    xg = H.to_gpu(x, dtype)
+    cg = torch.from_numpy(cols).int().cuda() if gather else None
+    got = ops.mat_fourier(xg, N, T, k0, cols=cg)
+    ref = ops.mat_fourier(xg, N, T, k0, cols=cg, matrix_cores=False)
+    assert rel_err(got.cpu().numpy(), ref.cpu().numpy()) <= 5e-4
+    if k0 == 0:
+        want = fo.compress_prefill(xs, N, T)
+        assert rel_err(got.cpu().numpy(), want) <= 5e-4
+    # accumulate adds onto what is there
+    got2 = got.clone()
+    ops.mat_fourier(xg, N, T, k0, cols=cg, out=got2, accumulate=True)
+    assert rel_err(got2.cpu().numpy(), 2 * got.cpu().numpy()) <= 1e-6
