@@ -68,6 +68,7 @@ _SIGNATURES = {
     "fa_mat_fourier_avg_std": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
                                        c_size_t, c_void_p]),
     "fa_stats_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "fa_mat_fourier_avg_std_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fa_reconstruct": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                c_void_p]),
     "fa_coeff_update": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_void_p, c_int, c_int, c_int, c_int64, c_int,

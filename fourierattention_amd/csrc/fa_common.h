@@ -26,6 +26,11 @@ int fa_check_launch(const char* what);
 
 // matrix-core spectral compression (fa_spectral_mfma.hip)
 bool fa_spectral_mfma_ok(int a_dtype, int K, int Mc, int N);
+bool fa_recon_stats_mfma_ok(int N, int Mc, int K);
+size_t fa_recon_stats_mfma_workspace(int B, int N, int Mc, int K);
+// partial sums / maxima / minima of the reconstruction, [B][row blocks][Mc] each; returns the number of row blocks
+int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int T, void* workspace, float** psum,
+                               float** pmax, float** pmin, hipStream_t st);
 size_t fa_spectral_mfma_workspace(int B, int K, int Mc, int N);
 int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols, float* c, int B,
                             int K, int Mc, int N, int T, int64_t k_start, int accumulate, void* workspace,
@@ -137,6 +142,13 @@ __device__ __forceinline__ float fa_rows_max(float x) {
   x = fmaxf(a, b);
   fa_swap32(x, &a, &b);
   return fmaxf(a, b);
+}
+__device__ __forceinline__ float fa_rows_min(float x) {
+  float a, b;
+  fa_swap16(x, &a, &b);
+  x = fminf(a, b);
+  fa_swap32(x, &a, &b);
+  return fminf(a, b);
 }
 __device__ __forceinline__ float fa_rows_sum(float x) {
   float a, b;

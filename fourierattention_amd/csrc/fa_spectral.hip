@@ -338,6 +338,16 @@ extern "C" int fa_mat_avg_std(const void* a, int a_dtype, int64_t a_bs, int64_t 
   return fa_check_launch("fa_mat_avg_std");
 }
 
+extern "C" size_t fa_mat_fourier_avg_std_workspace_bytes(int B, int N, int Mc, int K) {
+  if (B <= 0 || N <= 0 || Mc <= 0 || K <= 0) return 0;
+  size_t a = fa_stats_workspace_bytes(B, Mc, K);
+  if (fa_recon_stats_mfma_ok(N, Mc, K)) {
+    const size_t m = fa_recon_stats_mfma_workspace(B, N, Mc, K);
+    if (m > a) a = m;
+  }
+  return a;
+}
+
 extern "C" int fa_mat_fourier_avg_std(const float* c, float* avg, float* max_dev, int B, int N, int Mc, int K,
                                       int T, int round_dtype, void* workspace, size_t workspace_bytes,
                                       fa_stream_t stream) {
@@ -346,12 +356,19 @@ extern "C" int fa_mat_fourier_avg_std(const float* c, float* avg, float* max_dev
              "fa_mat_fourier_avg_std: bad shape B=%d N=%d Mc=%d K=%d T=%d", B, N, Mc, K, T);
   FA_REQUIRE(workspace && workspace_bytes >= fa_stats_workspace_bytes(B, Mc, K), FA_ERR_WORKSPACE,
              "fa_mat_fourier_avg_std: workspace %zu < %zu", workspace_bytes, fa_stats_workspace_bytes(B, Mc, K));
+  hipStream_t s = fa_hip_stream(stream);
+  if (fa_recon_stats_mfma_ok(N, Mc, K) && workspace_bytes >= fa_recon_stats_mfma_workspace(B, N, Mc, K)) {
+    FA_REQUIRE(((uintptr_t)workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_mat_fourier_avg_std: workspace not 256-byte aligned");
+    float *ps, *px, *pn;
+    const int rb = fa_recon_stats_mfma_launch(c, B, N, Mc, K, T, workspace, &ps, &px, &pn, s);
+    stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 256), B), 256, 0, s>>>(ps, px, pn, avg, max_dev, K, Mc, rb, round_dtype);
+    return fa_check_launch("fa_mat_fourier_avg_std");
+  }
   const int nsplit = stats_splits(K);
   float* psum = (float*)workspace;
   float* pmax = psum + (size_t)B * nsplit * Mc;
   float* pmin = pmax + (size_t)B * nsplit * Mc;
   constexpr int MB = 32;
-  hipStream_t s = fa_hip_stream(stream);
   reconstruct_kernel<true, MB><<<dim3(fa_cdiv(Mc, MB), nsplit, B), 256, 0, s>>>(
       c, N, Mc, K, T, psum, pmax, pmin, nsplit, nullptr, nullptr, nullptr, nullptr);
   stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 256), B), 256, 0, s>>>(psum, pmax, pmin, avg, max_dev, K, Mc, nsplit, round_dtype);

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void spectral_table_kernel(half8* __restrict__
 template <typename E>
 __global__ __launch_bounds__(256) void spectral_pack_kernel(
     const E* __restrict__ a, int64_t a_bs, int64_t a_rs, const int32_t* __restrict__ cols,
-    half8* __restrict__ out, int K, int Mc, int CT, int KS32) {
+    const float* __restrict__ col_inv_scale, half8* __restrict__ out, int K, int Mc, int CT, int KS32) {
   constexpr int kPitch = 256 + 4;   // f16 elements per LDS row: 8 rows apart = 16 banks apart
   __shared__ _Float16 tile[32][kPitch];
   const int tid = threadIdx.x;
@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void spectral_pack_kernel(
   const bool mok = m < Mc;
   const int col = mok ? (cols ? cols[m] : m) : 0;
   const E* ab = a + (int64_t)b * a_bs + col;
+  const float mul = (col_inv_scale && mok) ? col_inv_scale[(int64_t)b * Mc + m] : 1.f;
   float v[32];
 #pragma unroll
   for (int kk = 0; kk < 32; ++kk) {
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(256) void spectral_pack_kernel(
   for (int kk = 0; kk < 32; ++kk) {
     const int k = ks * 32 + kk;
     // f16 holds every bf16 / f16 value of magnitude below 65504 exactly (tiny ones as subnormals)
-    const float x = (mok && k < K) ? fminf(fmaxf(v[kk], -65504.f), 65504.f) : 0.f;
+    const float x = (mok && k < K) ? fminf(fmaxf(v[kk] * mul, -65504.f), 65504.f) : 0.f;
     tile[kk][tid] = (_Float16)x;
   }
   __syncthreads();
@@ -210,6 +211,177 @@ __global__ __launch_bounds__(256) void spectral_reduce_kernel(const float* __res
   *(float4*)(c + i) = a;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Statistics of the reconstruction (mat_fourier_avg_std_triton, TRI:285-326) on the same machinery.
+//   r[k, m] = (1/N) sum_n cos(theta k n) c[n, m] + sin(theta k n) c[N + n, m] = (1/N) Re sum_n e^{i theta k n} (c - i s)
+// is the compression GEMM with the roles of position and frequency exchanged: the rows are the positions k,
+// the "tokens" are the N coefficient indices.  A workgroup owns 128 positions, keeps their basis rows in
+// registers, and walks over every block of 64 columns: one pass over the cos coefficients (keeps the real part),
+// one over the sin coefficients (adds the imaginary part), then folds its positions into sum / max / min.
+// The coefficients travel as f16 scaled by a power of two per column (their range is not bounded).
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void coef_colscale_kernel(const float* __restrict__ c, float* __restrict__ scale,
+                                                            float* __restrict__ inv_scale, int N2, int Mc) {
+  __shared__ float s_mx[4][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int m = blockIdx.x * 64 + lane, b = blockIdx.y;
+  float mx = 0.f;
+  if (m < Mc)
+    for (int n = g; n < N2; n += 4) mx = fmaxf(mx, fabsf(c[((int64_t)b * N2 + n) * Mc + m]));
+  s_mx[g][lane] = mx;
+  __syncthreads();
+  if (g == 0 && m < Mc) {
+    mx = fmaxf(fmaxf(s_mx[0][lane], s_mx[1][lane]), fmaxf(s_mx[2][lane], s_mx[3][lane]));
+    const float sc = mx > 0.f ? exp2f(ceilf(log2f(mx))) : 1.f;   // power of two: scaling is exact
+    scale[(int64_t)b * Mc + m] = sc;
+    inv_scale[(int64_t)b * Mc + m] = 1.0f / sc;
+  }
+}
+
+struct ReconStatsParams {
+  const half8* tab;        // basis rows of the positions: [ceil(K/8)][kStepK][64]
+  const half8* packed[2];  // cos / sin coefficients, [B][CT][KS32][64] fragments
+  const float* scale;      // [B][Mc]
+  float* psum;
+  float* pmax;
+  float* pmin;             // [B][RB][Mc]
+  int B, N, Mc, CT, KS32, K, T, n_steps, RB;
+};
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void spectral_recon_stats_kernel(
+    const ReconStatsParams p) {
+  constexpr int NST = 4;
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[NST][4][kStepK][1024];
+  __shared__ float s_red[3][4][kWgCols];
+  const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rb = blockIdx.x, b = blockIdx.y;
+  const int rt0 = (rb * 4 + w) * 4;
+  const int n_rt = (p.K + 7) / 8;
+  const int S = p.n_steps;
+  const int n_cb = (p.Mc + kWgCols - 1) / kWgCols;
+  const int Q = n_cb * 2 * S;   // steps of this workgroup: column block, pass (cos, sin), step (last to first)
+
+  auto issue = [&](int q, int stage) {
+    const int cb = q / (2 * S), rem = q - cb * 2 * S;
+    const int pass = rem / S, s = S - 1 - (rem - pass * S);
+    const int ct = min(cb * 4 + w, p.CT - 1);
+    const _Float16* src = (const _Float16*)(p.packed[pass] + (((int64_t)b * p.CT + ct) * p.KS32) * 64) + lane * 8;
+#pragma unroll
+    for (int ks = 0; ks < kStepK; ++ks)
+      load_frag_to_lds(src + (int64_t)(s * kStepK + ks) * 512, &s_stage[stage][w][ks][0]);
+  };
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i)
+    if (i < Q) issue(i, i);
+
+  half8 Ea[4][kStepK];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int ks = 0; ks < kStepK; ++ks) Ea[i][ks] = p.tab[((int64_t)min(rt0 + i, n_rt - 1) * kStepK + ks) * 64 + lane];
+  float rc[4][2], rs[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(min(rt0 + i, n_rt - 1) * 8 + lg * 2 + f2, kStepTokens, p.T, &rs[i][f2], &rc[i][f2]);
+  float4v acc[4][4];
+  float re[4][4][2];   // real part left by the cos pass
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int ks = 0; ks < kStepK; ++ks) asm volatile("" ::"v"(Ea[i][ks]));
+
+  const float inv_n = 1.0f / (float)p.N;
+  for (int q = 0; q < Q; ++q) {
+    const int cb = q / (2 * S), rem = q - cb * 2 * S;
+    const int pass = rem / S, it = rem - pass * S;
+    const int stage = q % NST;
+    if (q + NST - 2 < Q) wait_vmcnt<(NST - 2) * kStepK>();
+    else wait_vmcnt<0>();
+    barrier_lds_only();
+    if (q + NST - 1 < Q) issue(q + NST - 1, (q + NST - 1) % NST);
+    if (it == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int f2 = 0; f2 < 2; ++f2) {
+            const float c = acc[i][j][2 * f2], sn = acc[i][j][2 * f2 + 1];
+            acc[i][j][2 * f2] = rc[i][f2] * c - rs[i][f2] * sn;
+            acc[i][j][2 * f2 + 1] = rs[i][f2] * c + rc[i][f2] * sn;
+          }
+    }
+#pragma unroll
+    for (int ks = 0; ks < kStepK; ++ks) {
+      uint4v braw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) braw[j] = lds_read_b128_async(&s_stage[stage][j][ks][lane * 16]);
+      lds_wait_for4<0>(braw);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[i][ks], __builtin_bit_cast(half8, braw[j]), acc[i][j], 0, 0, 0);
+    }
+    if (it != S - 1) continue;
+    if (pass == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          re[i][j][0] = acc[i][j][0];
+          re[i][j][1] = acc[i][j][2];
+        }
+      continue;
+    }
+    // both passes done for this column block: r = (re + im) * scale / N at this lane's 8 positions per column
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = (cb * 4 + j) * 16 + lc;
+      const float sc = m < p.Mc ? p.scale[(int64_t)b * p.Mc + m] * inv_n : 0.f;
+      float sum = 0.f, mx = -INFINITY, mn = INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int f2 = 0; f2 < 2; ++f2) {
+          const int k = (rt0 + i) * 8 + lg * 2 + f2;
+          const float r = (re[i][j][f2] + acc[i][j][2 * f2 + 1]) * sc;
+          if (k < p.K) {
+            sum += r;
+            mx = fmaxf(mx, r);
+            mn = fminf(mn, r);
+          }
+        }
+      sum = fa_rows_sum(sum);
+      mx = fa_rows_max(mx);
+      mn = fa_rows_min(mn);
+      if (lg == 0) {
+        s_red[0][w][j * 16 + lc] = sum;
+        s_red[1][w][j * 16 + lc] = mx;
+        s_red[2][w][j * 16 + lc] = mn;
+      }
+    }
+    __syncthreads();
+    if (tid < kWgCols) {
+      const int m = cb * kWgCols + tid;
+      if (m < p.Mc) {
+        const int64_t o = ((int64_t)b * p.RB + rb) * p.Mc + m;
+        p.psum[o] = (s_red[0][0][tid] + s_red[0][1][tid]) + (s_red[0][2][tid] + s_red[0][3][tid]);
+        p.pmax[o] = fmaxf(fmaxf(s_red[1][0][tid], s_red[1][1][tid]), fmaxf(s_red[1][2][tid], s_red[1][3][tid]));
+        p.pmin[o] = fminf(fminf(s_red[2][0][tid], s_red[2][1][tid]), fminf(s_red[2][2][tid], s_red[2][3][tid]));
+      }
+    }
+    // the next barrier (top of the loop) orders these reads before s_red is written again
+  }
+}
+
 }  // namespace fa_mfma
 
 namespace {
@@ -258,9 +430,9 @@ int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_
   spectral_table_kernel<<<fa_cdiv((N / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, N, T);
   dim3 pgrid(pl.KS32, fa_cdiv(Mc, 256), B);
   if (a_dtype == FA_BF16)
-    spectral_pack_kernel<bf16_t><<<pgrid, 256, 0, st>>>((const bf16_t*)a, a_bs, a_rs, cols, packed, K, Mc, pl.CT, pl.KS32);
+    spectral_pack_kernel<bf16_t><<<pgrid, 256, 0, st>>>((const bf16_t*)a, a_bs, a_rs, cols, nullptr, packed, K, Mc, pl.CT, pl.KS32);
   else
-    spectral_pack_kernel<f16_t><<<pgrid, 256, 0, st>>>((const f16_t*)a, a_bs, a_rs, cols, packed, K, Mc, pl.CT, pl.KS32);
+    spectral_pack_kernel<f16_t><<<pgrid, 256, 0, st>>>((const f16_t*)a, a_bs, a_rs, cols, nullptr, packed, K, Mc, pl.CT, pl.KS32);
   SpectralGemmParams gp{};
   gp.tab = tab; gp.packed = packed; gp.part = part;
   gp.B = B; gp.N = N; gp.Mc = Mc; gp.CT = pl.CT; gp.KS32 = pl.KS32; gp.T = T;
@@ -271,4 +443,63 @@ int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_
   const int64_t total = (int64_t)B * 2 * N * Mc;
   spectral_reduce_kernel<<<fa_cdiv(total / 4, 256), 256, 0, st>>>(part, c, total, pl.n_chunks, accumulate);
   return fa_check_launch("fa_mat_fourier");
+}
+
+namespace {
+struct ReconPlan {
+  int CT, KS32, n_steps, RB;
+  size_t off_tab, off_pc, off_ps, off_scale, off_inv, off_sum, off_max, off_min, total;
+};
+ReconPlan recon_plan(int B, int N, int Mc, int K) {
+  using namespace fa_mfma;
+  ReconPlan p{};
+  p.CT = fa_cdiv(Mc, 16);
+  p.n_steps = fa_cdiv(N, kStepTokens);
+  p.KS32 = p.n_steps * kStepK;
+  p.RB = fa_cdiv(K, kWgFreqs);
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o += fa_align_up(bytes, 256); return at; };
+  p.off_tab = take((size_t)fa_cdiv(K, 8) * kStepK * 64 * 16);
+  p.off_pc = take((size_t)B * p.CT * p.KS32 * 1024);
+  p.off_ps = take((size_t)B * p.CT * p.KS32 * 1024);
+  p.off_scale = take((size_t)B * Mc * 4);
+  p.off_inv = take((size_t)B * Mc * 4);
+  p.off_sum = take((size_t)B * p.RB * Mc * 4);
+  p.off_max = take((size_t)B * p.RB * Mc * 4);
+  p.off_min = take((size_t)B * p.RB * Mc * 4);
+  p.total = o;
+  return p;
+}
+}  // namespace
+
+bool fa_recon_stats_mfma_ok(int N, int Mc, int K) { return N >= 32 && Mc >= 16 && K >= 1024; }
+
+size_t fa_recon_stats_mfma_workspace(int B, int N, int Mc, int K) { return recon_plan(B, N, Mc, K).total; }
+
+int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int T, void* workspace, float** psum,
+                               float** pmax, float** pmin, hipStream_t st) {
+  using namespace fa_mfma;
+  const ReconPlan pl = recon_plan(B, N, Mc, K);
+  char* ws = (char*)workspace;
+  half8* tab = (half8*)(ws + pl.off_tab);
+  half8* pc = (half8*)(ws + pl.off_pc);
+  half8* ps = (half8*)(ws + pl.off_ps);
+  float* scale = (float*)(ws + pl.off_scale);
+  float* inv = (float*)(ws + pl.off_inv);
+  *psum = (float*)(ws + pl.off_sum);
+  *pmax = (float*)(ws + pl.off_max);
+  *pmin = (float*)(ws + pl.off_min);
+  const int kp8 = fa_cdiv(K, 8) * 8;
+  spectral_table_kernel<<<fa_cdiv((kp8 / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, kp8, T);
+  coef_colscale_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, st>>>(c, scale, inv, 2 * N, Mc);
+  dim3 pgrid(pl.KS32, fa_cdiv(Mc, 256), B);
+  spectral_pack_kernel<float><<<pgrid, 256, 0, st>>>(c, (int64_t)2 * N * Mc, Mc, nullptr, inv, pc, N, Mc, pl.CT, pl.KS32);
+  spectral_pack_kernel<float><<<pgrid, 256, 0, st>>>(c + (int64_t)N * Mc, (int64_t)2 * N * Mc, Mc, nullptr, inv, ps, N, Mc,
+                                                     pl.CT, pl.KS32);
+  ReconStatsParams rp{};
+  rp.tab = tab; rp.packed[0] = pc; rp.packed[1] = ps; rp.scale = scale;
+  rp.psum = *psum; rp.pmax = *pmax; rp.pmin = *pmin;
+  rp.B = B; rp.N = N; rp.Mc = Mc; rp.CT = pl.CT; rp.KS32 = pl.KS32; rp.K = K; rp.T = T; rp.n_steps = pl.n_steps; rp.RB = pl.RB;
+  spectral_recon_stats_kernel<<<dim3(pl.RB, B), 256, 0, st>>>(rp);
+  return pl.RB;
 }

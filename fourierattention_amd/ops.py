@@ -127,7 +127,11 @@ def mat_avg_std_triton(a: torch.Tensor):
 
 
 # --------------------------------------------------------------------------- K3
-def mat_fourier_avg_std(c: torch.Tensor, K: int, T: int, round_dtype: Optional[torch.dtype] = torch.float16):
+def mat_fourier_avg_std(c: torch.Tensor, K: int, T: int, round_dtype: Optional[torch.dtype] = torch.float16,
+                        matrix_cores: bool = True):
+    """Mean and maximum deviation, per column, of the signal reconstructed from ``c`` at positions 0..K-1.
+    Long reconstructions run on the matrix cores (fp16 operands, fp32 accumulation) unless
+    ``matrix_cores`` is false."""
     _require_gpu(c, "c")
     assert c.is_contiguous() and c.dtype == torch.float32 and c.dim() == 3
     B, N2, Mc = c.shape
@@ -136,11 +140,14 @@ def mat_fourier_avg_std(c: torch.Tensor, K: int, T: int, round_dtype: Optional[t
     if Mc == 0 or B == 0:
         return avg, dev
     lib = _lib.load()
-    nbytes = lib.fa_stats_workspace_bytes(B, Mc, int(K))
-    ws = workspace(c.device, nbytes)
+    if matrix_cores:
+        nbytes = lib.fa_mat_fourier_avg_std_workspace_bytes(B, N2 // 2, Mc, int(K))
+    else:
+        nbytes = lib.fa_stats_workspace_bytes(B, Mc, int(K))
+    ws = workspace(c.device, nbytes, "spectral")
     rd = FA_FP32 if round_dtype is None else dtype_code(round_dtype)
     check(lib.fa_mat_fourier_avg_std(c.data_ptr(), avg.data_ptr(), dev.data_ptr(), B, N2 // 2, Mc, int(K), int(T), rd,
-                                     ws.data_ptr(), ws.numel(), _stream(c.device)))
+                                     ws.data_ptr(), int(nbytes), _stream(c.device)))
     return avg, dev
 
 

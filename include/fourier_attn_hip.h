@@ -81,12 +81,16 @@ int fa_mat_avg_std(const void* a, int a_dtype, int64_t a_batch_stride, int64_t a
  * reconstructed from c (B, 2N, Mc) fp32 at positions 0..K-1 with period T:
  *   r[b,k,m] = (1/N) sum_n cos(2 pi k n / T) c[b,n,m] + sin(...) c[b,N+n,m].
  * Outputs fp32 (B, Mc) rounded through round_dtype (the reference returns
- * fp16, TRI:326).  workspace: fa_stats_workspace_bytes(B, Mc, K). */
+ * fp16, TRI:326).  workspace: at least fa_stats_workspace_bytes(B, Mc, K);
+ * with fa_mat_fourier_avg_std_workspace_bytes(B, N, Mc, K) bytes (256-byte
+ * aligned) long reconstructions (K >= 1024) run on the matrix cores (basis and
+ * per-column scaled coefficients in fp16, fp32 accumulation). */
 int fa_mat_fourier_avg_std(const float* c, float* avg, float* max_dev, int B, int N, int Mc,
                            int K, int T, int round_dtype, void* workspace, size_t workspace_bytes,
                            fa_stream_t stream);
 
 size_t fa_stats_workspace_bytes(int B, int Mc, int K);
+size_t fa_mat_fourier_avg_std_workspace_bytes(int B, int N, int Mc, int K);
 
 /* Reconstruction r (B, K, Mc) fp32 from coefficients (mat_fourier_inv_torch,
  * TRI:782-791); with stats pointers non-NULL also applies

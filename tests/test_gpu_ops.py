@@ -174,3 +174,24 @@ def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
     got2 = got.clone()
     ops.mat_fourier(xg, N, T, k0, cols=cg, out=got2, accumulate=True)
     assert rel_err(got2.cpu().numpy(), 2 * got.cpu().numpy()) <= 1e-6
+
+
+@pytest.mark.parametrize("B,L,C,N,T", [(2, 1500, 70, 40, 1533), (1, 4100, 128, 128, 4100), (1, 1100, 16, 200, 5000)])
+def test_stats_reconstructed_matrix_cores(B, L, C, N, T):
+    """Long reconstructions take the matrix-core kernel (fp16 basis and per-column scaled fp16 coefficients, fp32
+    accumulation): statistics against the oracle and against the fp32 vector kernel.  Bound: each operand carries
+    up to 2^-11 relative rounding, the results are rounded through fp16 (2^-11 again)."""
+    from fourierattention_amd import ops
+    r = np.random.default_rng(6)
+    x = r.standard_normal((B, L, C)) * r.uniform(0.2, 30.0, (1, 1, C)) + r.uniform(-3, 3, (1, 1, C))   # mixed column ranges
+    coef = fo.compress_prefill(x, N, T).astype(np.float32)
+    cg = torch.from_numpy(coef).cuda()
+    avg, dev = ops.mat_fourier_avg_std(cg, L, T, torch.float16)
+    avg0, dev0 = ops.mat_fourier_avg_std(cg, L, T, torch.float16, matrix_cores=False)
+    wa, wd = fo.stats_reconstructed(coef, L, T)
+    scale = np.abs(wd).max(axis=None)
+    for got, ref, want in ((avg, avg0, wa), (dev, dev0, wd)):
+        g = got.cpu().numpy()
+        # relative to the size of the reconstructed signal of the column (its deviation), not of the value itself
+        assert np.max(np.abs(g - want) / (np.abs(wd) + np.abs(wa))) <= 2e-3
+        assert np.max(np.abs(g - ref.cpu().numpy()) / (np.abs(wd) + np.abs(wa))) <= 2e-3
