@@ -20,22 +20,64 @@ __device__ __forceinline__ int64_t page_elem_offset(bool is_v, int dp, int64_t t
   return page * dp * 32 + (int64_t)frag * 512 + lane * 8 + e;
 }
 
-// one thread per (token, padded dim) of one (b, h): grid (ceil(L*dp/256), Hkv, B)
+// one block per page (32 tokens) of one (b, h): the gather reads run along the stored dims of a token row,
+// the page is assembled in LDS and leaves as whole fragments (16 bytes per lane); grid (pages, Hkv, B)
 template <typename E>
 __global__ __launch_bounds__(256) void mid_pack_kernel(
     const E* __restrict__ src, int64_t src_bs, int64_t src_rs, int64_t row0, int L, E* __restrict__ store,
     int64_t st_bs, int cap_pages, const int32_t* __restrict__ n_list, const int32_t* __restrict__ n_h,
     const int32_t* __restrict__ pad_h, int is_v) {
-  const int h = blockIdx.y, b = blockIdx.z;
+  constexpr int kMaxDp = 256;                       // padded stored dims of a head
+  constexpr int kPitch = kMaxDp + 8;                // elements; keeps rows 16-byte aligned
+  struct alignas(sizeof(E) * 8) Piece { E v[8]; };  // what one lane of a fragment holds
+  __shared__ __attribute__((aligned(32))) E tile[32][kPitch];
+  const int page = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int n0 = n_h[h], n_len = n_h[h + 1] - n0;
   const int p0 = pad_h[h], dp = pad_h[h + 1] - p0;
   if (n_len == 0) return;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)L * n_len) return;
-  const int64_t token = idx / n_len;
-  const int j = (int)(idx % n_len);
-  const E v = src[(int64_t)b * src_bs + (row0 + token) * src_rs + n_list[n0 + j]];
-  store[(int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + page_elem_offset(is_v, dp, token, j)] = v;
+  const int tid = threadIdx.x;
+  __shared__ int s_col[kMaxDp];
+  for (int j = tid; j < dp; j += 256) s_col[j] = n_list[n0 + min(j, n_len - 1)];
+  __syncthreads();
+  // gather: consecutive threads take consecutive stored dims of one token; eight loads in flight per thread,
+  // all unconditional (clamped to the last real dim / row, masked afterwards)
+  const E* sb = src + (int64_t)b * src_bs + row0 * src_rs;
+  const int64_t last = (int64_t)L - 1;
+  for (int base = tid; base < 32 * dp; base += 256 * 8) {
+    E v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int idx = min(base + 256 * u, 32 * dp - 1);
+      const int t = idx / dp, j = idx - t * dp;
+      const int64_t token = (int64_t)page * 32 + t;
+      v[u] = sb[(token < last ? token : last) * src_rs + s_col[j]];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int idx = base + 256 * u;
+      if (idx < 32 * dp) {
+        const int t = idx / dp, j = idx - t * dp;
+        const bool ok = j < n_len && (int64_t)page * 32 + t < L;
+        tile[t][j] = ok ? v[u] : E{};
+      }
+    }
+  }
+  __syncthreads();
+  Piece* out = (Piece*)(store + (int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + (int64_t)page * dp * 32);
+  const int n_pieces = dp * 32 / 8;
+  for (int piece = tid; piece < n_pieces; piece += 256) {
+    const int frag = piece >> 6, lane = piece & 63;
+    Piece o;
+    if (!is_v) {
+      const int nks = dp >> 5;
+      const int tb = frag / nks, s_ = frag - tb * nks;
+      o = *(const Piece*)&tile[tb * 16 + (lane & 15)][s_ * 32 + 8 * (lane >> 4)];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o.v[i] = tile[8 * (lane >> 4) + i][frag * 16 + (lane & 15)];
+    }
+    out[piece] = o;
+  }
 }
 
 template <typename E>
@@ -91,7 +133,8 @@ extern "C" int fa_mid_pack(const void* src, int dtype, int64_t src_bs, int64_t s
   if (L == 0) return FA_OK;
   hipStream_t st = fa_hip_stream(stream);
   FA_REQUIRE(D > 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: head_dim %d", D);
-  dim3 grid(fa_cdiv((int64_t)L * D, 256), Hkv, B);  // a head stores at most D dims
+  FA_REQUIRE(D <= 256, FA_ERR_UNSUPPORTED, "fa_mid_pack: head_dim %d above 256", D);
+  dim3 grid(fa_cdiv(L, 32), Hkv, B);
   int rc = dispatch16(dtype, "fa_mid_pack", [&](auto tag) {
     using E = decltype(tag);
     mid_pack_kernel<E><<<grid, 256, 0, st>>>((const E*)src, src_bs, src_rs, row0, L, (E*)store, st_bs, cap_pages, n_list,

@@ -129,14 +129,39 @@ __global__ __launch_bounds__(256) void col_stats_partial_kernel(
 __global__ __launch_bounds__(256) void stats_finalize_kernel(
     const float* __restrict__ psum, const float* __restrict__ pmax, const float* __restrict__ pmin,
     float* __restrict__ avg, float* __restrict__ dev, int K, int Mc, int nsplit, int round_dtype) {
-  const int m = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
-  if (m >= Mc) return;
+  // block = 64 columns x 4 classes of splits, eight splits in flight per thread
+  __shared__ float s_red[3][4][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int m = blockIdx.x * 64 + lane, b = blockIdx.y;
   float sum = 0.f, mx = -INFINITY, mn = INFINITY;
-  for (int s = 0; s < nsplit; ++s) {
-    int64_t o = ((int64_t)b * nsplit + s) * Mc + m;
-    sum += psum[o];
-    mx = fmaxf(mx, pmax[o]);
-    mn = fminf(mn, pmin[o]);
+  if (m < Mc) {
+    for (int s0 = g; s0 < nsplit; s0 += 4 * 8) {
+      float a[8], x[8], n[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int64_t o = ((int64_t)b * nsplit + min(s0 + 4 * u, nsplit - 1)) * Mc + m;
+        a[u] = psum[o];
+        x[u] = pmax[o];
+        n[u] = pmin[o];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + 4 * u < nsplit) {
+          sum += a[u];
+          mx = fmaxf(mx, x[u]);
+          mn = fminf(mn, n[u]);
+        }
+    }
+  }
+  s_red[0][g][lane] = sum;
+  s_red[1][g][lane] = mx;
+  s_red[2][g][lane] = mn;
+  __syncthreads();
+  if (g != 0 || m >= Mc) return;
+  for (int i = 1; i < 4; ++i) {
+    sum += s_red[0][i][lane];
+    mx = fmaxf(mx, s_red[1][i][lane]);
+    mn = fminf(mn, s_red[2][i][lane]);
   }
   float av = sum / (float)K;
   float dv = fmaxf(mx - av, av - mn);
@@ -334,7 +359,7 @@ extern "C" int fa_mat_avg_std(const void* a, int a_dtype, int64_t a_bs, int64_t 
     default:
       FA_REQUIRE(false, FA_ERR_BAD_DTYPE, "fa_mat_avg_std: dtype %d", a_dtype);
   }
-  stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 256), B), 256, 0, s>>>(psum, pmax, pmin, avg, max_dev, K, Mc, nsplit, round_dtype);
+  stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, s>>>(psum, pmax, pmin, avg, max_dev, K, Mc, nsplit, round_dtype);
   return fa_check_launch("fa_mat_avg_std");
 }
 
@@ -361,7 +386,7 @@ extern "C" int fa_mat_fourier_avg_std(const float* c, float* avg, float* max_dev
     FA_REQUIRE(((uintptr_t)workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_mat_fourier_avg_std: workspace not 256-byte aligned");
     float *ps, *px, *pn;
     const int rb = fa_recon_stats_mfma_launch(c, B, N, Mc, K, T, workspace, &ps, &px, &pn, s);
-    stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 256), B), 256, 0, s>>>(ps, px, pn, avg, max_dev, K, Mc, rb, round_dtype);
+    stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, s>>>(ps, px, pn, avg, max_dev, K, Mc, rb, round_dtype);
     return fa_check_launch("fa_mat_fourier_avg_std");
   }
   const int nsplit = stats_splits(K);
@@ -371,7 +396,7 @@ extern "C" int fa_mat_fourier_avg_std(const float* c, float* avg, float* max_dev
   constexpr int MB = 32;
   reconstruct_kernel<true, MB><<<dim3(fa_cdiv(Mc, MB), nsplit, B), 256, 0, s>>>(
       c, N, Mc, K, T, psum, pmax, pmin, nsplit, nullptr, nullptr, nullptr, nullptr);
-  stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 256), B), 256, 0, s>>>(psum, pmax, pmin, avg, max_dev, K, Mc, nsplit, round_dtype);
+  stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, s>>>(psum, pmax, pmin, avg, max_dev, K, Mc, nsplit, round_dtype);
   return fa_check_launch("fa_mat_fourier_avg_std");
 }
 

@@ -220,18 +220,27 @@ __global__ __launch_bounds__(256) void spectral_reduce_kernel(const float* __res
 // one over the sin coefficients (adds the imaginary part), then folds its positions into sum / max / min.
 // The coefficients travel as f16 scaled by a power of two per column (their range is not bounded).
 // ---------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void coef_colscale_kernel(const float* __restrict__ c, float* __restrict__ scale,
-                                                            float* __restrict__ inv_scale, int N2, int Mc) {
-  __shared__ float s_mx[4][64];
-  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+__global__ __launch_bounds__(1024) void coef_colscale_kernel(const float* __restrict__ c, float* __restrict__ scale,
+                                                             float* __restrict__ inv_scale, int N2, int Mc) {
+  __shared__ float s_mx[16][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;   // 64 columns x 16 row classes
   const int m = blockIdx.x * 64 + lane, b = blockIdx.y;
   float mx = 0.f;
-  if (m < Mc)
-    for (int n = g; n < N2; n += 4) mx = fmaxf(mx, fabsf(c[((int64_t)b * N2 + n) * Mc + m]));
+  if (m < Mc) {
+    const float* cp = c + (int64_t)b * N2 * Mc + m;
+    for (int n0 = g; n0 < N2; n0 += 16 * 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = cp[(int64_t)min(n0 + 16 * u, N2 - 1) * Mc];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) mx = fmaxf(mx, fabsf(v[u]));
+    }
+  }
   s_mx[g][lane] = mx;
   __syncthreads();
   if (g == 0 && m < Mc) {
-    mx = fmaxf(fmaxf(s_mx[0][lane], s_mx[1][lane]), fmaxf(s_mx[2][lane], s_mx[3][lane]));
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s_mx[i][lane]);
     const float sc = mx > 0.f ? exp2f(ceilf(log2f(mx))) : 1.f;   // power of two: scaling is exact
     scale[(int64_t)b * Mc + m] = sc;
     inv_scale[(int64_t)b * Mc + m] = 1.0f / sc;
@@ -491,7 +500,7 @@ int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int 
   *pmin = (float*)(ws + pl.off_min);
   const int kp8 = fa_cdiv(K, 8) * 8;
   spectral_table_kernel<<<fa_cdiv((kp8 / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, kp8, T);
-  coef_colscale_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, st>>>(c, scale, inv, 2 * N, Mc);
+  coef_colscale_kernel<<<dim3(fa_cdiv(Mc, 64), B), 1024, 0, st>>>(c, scale, inv, 2 * N, Mc);
   dim3 pgrid(pl.KS32, fa_cdiv(Mc, 256), B);
   spectral_pack_kernel<float><<<pgrid, 256, 0, st>>>(c, (int64_t)2 * N * Mc, Mc, nullptr, inv, pc, N, Mc, pl.CT, pl.KS32);
   spectral_pack_kernel<float><<<pgrid, 256, 0, st>>>(c + (int64_t)N * Mc, (int64_t)2 * N * Mc, Mc, nullptr, inv, ps, N, Mc,
