@@ -133,6 +133,32 @@ def cpu_baseline():
                       f"{nbytes} algorithmic bytes; host has {os.cpu_count()} logical CPUs"}
 
 
+def compress_bench(device, reps=20):
+    """Spectral compression of one tensor of a 32k prompt (B=1, 32768 tokens, 8 KV heads x 128 dims of which
+    64 per head are compressed, 1024 coefficient rows, bf16): matrix-core roofline of the whole call
+    (basis table, gather/pack, GEMM, chunk reduction)."""
+    from fourierattention_amd import ops
+    L, HD, Mc, N = 32768, 1024, 512, 512
+    g = torch.Generator(device=device).manual_seed(0)
+    x = torch.randn((1, L, HD), device=device, generator=g).to(torch.bfloat16)
+    cols = torch.sort(torch.randperm(HD, device=device, generator=g)[:Mc])[0].int()
+    out = torch.empty((1, 2 * N, Mc), device=device)
+    for _ in range(3):
+        ops.mat_fourier(x, N, L, 0, cols=cols, out=out)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        ops.mat_fourier(x, N, L, 0, cols=cols, out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    flops = 2.0 * (2 * N) * L * Mc
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"workload": "config2_compress_32k", "ms_per_tensor": round(ms, 5), "bound": "mfma", "achieved": round(tf, 1),
+            "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4), "algorithmic_flops": flops,
+            "operand_dtype": "f16 (basis and data), fp32 accumulation"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -199,20 +225,23 @@ def main():
         cache.decode_attention(q, 0, Hq, Hkv, timings=tm)
         per += np.array(tm)
     per /= reps
-    kernel_ms = {"coeff_query": per[0], "mid_rows": per[1], "sink_window": per[2], "merge": per[3]}
+    # three launches: the coefficient-domain query shares one with the sink/window tiles (the third slot is the
+    # gap left between the event pairs, a few microseconds of event overhead)
+    kernel_ms = {"query_and_sink_window": per[0] + per[2], "mid_rows": per[1], "merge": per[3]}
     # algorithmic bytes of each kernel's own launch
     kbytes = {
-        "coeff_query": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4,
+        "query_and_sink_window": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4 + w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,
         "mid_rows": w["B"] * 2 * L * (hd - ck) * 2,
-        "sink_window": w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,
         "merge": w["B"] * w["M"] * ck * 4,
     }
     dom = max(kernel_ms, key=kernel_ms.get)
     dom_gbs = kbytes[dom] / (kernel_ms[dom] * 1e-3) / 1e9
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "decode_mid_rows_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "decode_mid_rows_traffic.txt")
     if dom == "mid_rows" and args.workload.startswith("config3") and os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        for line in open(tpath):   # counter summary kept with the profiles: "hbm_bytes_per_launch: <bytes>"
+            if line.startswith("hbm_bytes_per_launch:"):
+                traffic = int(float(line.split(":", 1)[1]))
     full = 2 * w["ctx"] * hd * 2
     fourier = 2 * (w["I"] + w["W"]) * hd * 2 + 2 * L * (hd - ck) * 2 + 2 * w["M"] * ck * 4
     result = {
@@ -235,6 +264,8 @@ def main():
                      "algorithmic_bytes_per_launch": kbytes[dom], "kernel_ms": round(float(kernel_ms[dom]), 5),
                      "whole_step_frac": round(gbs / HBM_PEAK_GBS, 4)},
     }
+    del cache
+    result["prefill_compress"] = compress_bench(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
