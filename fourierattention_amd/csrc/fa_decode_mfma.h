@@ -173,7 +173,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int kFragsMax = (2 * KMAX > VMAX ? 2 * KMAX : VMAX);   // fragments (1 KiB) of one page of one wave
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[8][NST][kFragsMax * 1024];
   __shared__ float s_part[2][kFreqWaves][16 * kPart];
-  __shared__ float s_max[kFreqWaves][16];
   __shared__ float4v s_rot[kFreqWaves * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
 
   const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
@@ -255,10 +254,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
     wmax = fa_rows_max(wmax);
-    if (lg == 0) s_max[sl][lc] = wmax;
-    __syncthreads();
-    wmax = fmaxf(fmaxf(s_max[0][lc], s_max[1][lc]), fmaxf(s_max[2][lc], s_max[3][lc]));
-    // power-of-two column scale keeps the f16 operand in [-1, 1] without rounding
+    // power-of-two scale per column and frequency slice (the partial scores are rescaled in fp32 before they
+    // are summed): keeps the f16 operand in [-1, 1] without rounding
     const float colscale = wmax > 0.f ? exp2f(ceilf(log2f(wmax))) : 1.f;
     const float colinv = 1.0f / colscale;
     const float c0col = (valid_r && sl == 0) ? p.c0[qrow] : 0.f;
@@ -314,6 +311,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
+    __syncthreads();   // the rotation constants in LDS are complete
     const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
@@ -402,10 +400,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int f = 0; f < VMAX; ++f) oacc[f] = float4v{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, d_run = 0.f;
     const bool ragged_tail = (p.L_m & 31) != 0;
-    __syncthreads();  // pairs with the score waves' column-scale exchange
     // the table loads must have landed before the loop starts (see the score waves)
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
+    __syncthreads();   // the rotation constants in LDS are complete
     const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
 
     for (int it = 0; it <= n_it; ++it) {
