@@ -1,8 +1,8 @@
 // MFMA path of decode attention over the mid rows (gfx950, wave64).
 //
-// One workgroup (4 waves, one per SIMD, up to 512 VGPRs each) owns one KV head, one group
-// of batch elements whose query rows fill the 16 MFMA columns (R = nb * G <= 16), and one
-// contiguous range of 32-token pages.  Per page:
+// One workgroup (8 waves, two per SIMD, 256 VGPRs each) owns one KV head, one group of batch
+// elements whose query rows fill the 16 MFMA columns (R = nb * G <= 16), and one contiguous
+// range of 32-token pages.  Per page:
 //
 //   scores  S[32 x 16] = E[32 x 2N] . W'[2N x 16]      (f16 MFMA; E = cos/sin of the token offset
 //                        + K_mn[32 x dims] . Q_n        inside the page, W' = coefficient-domain
@@ -12,9 +12,10 @@
 //                                                        current page: rotated by one page step first)
 //   o_n[dims x 16] += V_mn^T[dims x 32] . P              (bf16 / f16 MFMA on the stored dims)
 //
-// The 2N coefficient rows are split over the 4 waves (each keeps its slice of E, E^T, W' and
-// g' in registers); the partial scores are summed through LDS with one barrier per page.
-// Wave w also streams the stored dims of batch element w of the group.  K/V pages arrive as
+// The 2N coefficient rows are split four ways; slice i belongs to score wave i (E, W') and to
+// value wave i (E^T, g'), which share a SIMD.  The score waves work one page ahead of the value
+// waves; the partial scores cross through LDS with one barrier per page.  Waves i and 4 + i also
+// stream the stored K resp. V dims of batch element i of the group.  K/V pages arrive as
 // ready-made MFMA A operands (see the page layout in the public header).
 #pragma once
 
