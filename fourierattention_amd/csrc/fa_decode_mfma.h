@@ -224,7 +224,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
         for (int ks = 0; ks < KMAX; ++ks)
-          load_frag_to_lds(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
+          load_frag_to_lds<2>(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
     };
     if (has_k) {
 #pragma unroll
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const E* vp = vbase + (int64_t)t * dpv * 32;
       unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
 #pragma unroll
-      for (int f = 0; f < VMAX; ++f) load_frag_to_lds(vp + (f < ndg ? f : 0) * 512 + lane * 8, st + f * 1024);
+      for (int f = 0; f < VMAX; ++f) load_frag_to_lds<2>(vp + (f < ndg ? f : 0) * 512 + lane * 8, st + f * 1024);
     };
     if (has_v) {   // first pages requested before the tables (see the score waves)
 #pragma unroll

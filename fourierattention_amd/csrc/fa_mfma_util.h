@@ -35,10 +35,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 // one fragment (64 lanes x 16 bytes) from global memory straight into LDS at lds_frag + lane * 16
-template <typename E>
+// AUX: cache-policy bits of the load (0 = default, 2 = non-temporal: data that is read once should not
+// displace what the neighbouring kernels want to find in the last-level cache)
+template <int AUX = 0, typename E>
 __device__ __forceinline__ void load_frag_to_lds(const E* g_lane_ptr, void* lds_frag) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g_lane_ptr,
-                                   (__attribute__((address_space(3))) void*)lds_frag, 16, 0, 0);
+                                   (__attribute__((address_space(3))) void*)lds_frag, 16, 0, AUX);
 }
 
 // LDS accesses that the compiler must not tie to the asynchronous page loads (it would otherwise wait
