@@ -41,6 +41,7 @@ MFMA_CASES = [
     (torch.bfloat16, 2, 8, 2, 128, 4, 32, 512, 1100, 2, [0, 128], [127, 5]),         # ragged: nothing / everything stored
     (torch.float16, 3, 4, 4, 64, 2, 16, 256, 420, 2, [10, 30, 64, 1], [3, 64, 33, 17]),  # MHA, head_dim 64, fp16
     (torch.bfloat16, 2, 32, 8, 128, 4, 64, 1024, 2200, 2, [64] * 8, [64] * 8),       # the benchmark's geometry, short
+    (torch.bfloat16, 3, 16, 2, 128, 4, 200, 256, 900, 3, [64, 40], [64, 96]),        # 8:1 grouping, window of several tiles
 ]
 
 
@@ -82,3 +83,34 @@ def test_mfma_decode_matches_oracle_and_generic(case):
         # on the matrix cores land well inside it
         assert e_mfma <= 2e-2, e_mfma
         assert e_mfma <= 5e-3, e_mfma
+
+
+def test_full_size_properties():
+    """BASELINE config 3 at full size (B=8, 32k context): properties that need no CPU oracle.
+    (1) the matrix-core path and the generic path (independent kernels, each checked against the oracle at
+    small sizes) agree; (2) swapping two batch elements of the query and of the cache-independent inputs
+    swaps the output rows only where the cache rows are swapped too: here the query alone is permuted across
+    the heads of a KV group, which must permute the output heads the same way (GQA heads share K/V)."""
+    import bench
+    w = bench.WORKLOADS["config3_decode_attn_8b_32k"]
+    dev = torch.device("cuda", 0)
+    cache, q, kn, vn = bench.build_cache(w, torch.bfloat16, dev)
+    Hq, Hkv = w["Hq"], w["Hkv"]
+    assert cache._tables is not None
+    out = cache.decode_attention(q, 0, Hq, Hkv)
+    cache.force_generic = True
+    ref = cache.decode_attention(q, 0, Hq, Hkv)
+    cache.force_generic = False
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max().item() <= 5e-3
+    G = Hq // Hkv
+    perm = torch.arange(Hq, device=dev).view(Hkv, G).flip(1).reshape(-1)     # reverse the heads inside every group
+    out_p = cache.decode_attention(q[:, perm].contiguous(), 0, Hq, Hkv)
+    # same rows, other MFMA columns: equal up to the accumulation order of the split merge (identical here)
+    assert (out_p - out[:, perm]).abs().max().item() <= 1e-5
+    # a streaming step keeps everything consistent: sequence length grows by one, output stays finite
+    n0 = cache.get_seq_length(0)
+    cache.update(kn, vn, 0)
+    assert cache.get_seq_length(0) == n0 + 1
+    out2 = cache.decode_attention(q, 0, Hq, Hkv)
+    assert torch.isfinite(out2).all() and (out2 - out).abs().max().item() < 1.0
