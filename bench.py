@@ -264,6 +264,22 @@ def main():
                      "algorithmic_bytes_per_launch": kbytes[dom], "kernel_ms": round(float(kernel_ms[dom]), 5),
                      "whole_step_frac": round(gbs / HBM_PEAK_GBS, 4)},
     }
+    # the streaming update that precedes every decode-attention pass in use (one launch: rank-1 coefficient
+    # update, evicted row into the page store, new token into the window); read + write of the coefficients
+    for _ in range(5):
+        cache.update(kn, vn, 0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(50):
+        cache.update(kn, vn, 0)
+    stop.record()
+    torch.cuda.synchronize()
+    upd_wall = (time.perf_counter() - t0) / 50
+    upd_ms = start.elapsed_time(stop) / 50
+    upd_bytes = w["B"] * 2 * 2 * w["M"] * ck * 4
+    result["stream_update"] = {"ms_per_step": round(upd_ms, 5), "wall_ms_per_step": round(upd_wall * 1e3, 5),
+                               "algorithmic_bytes": upd_bytes, "GB_s": round(upd_bytes / (upd_ms * 1e-3) / 1e9, 1)}
     del cache
     result["prefill_compress"] = compress_bench(device)
     if not args.no_cpu_baseline:

@@ -56,10 +56,28 @@ class DecodeArgs(ctypes.Structure):
     ]
 
 
+class StreamArgs(ctypes.Structure):
+    """Mirror of ``fa_stream_args``."""
+    _fields_ = [
+        ("k_new", c_void_p), ("v_new", c_void_p), ("new_batch_stride", c_int64),
+        ("k_ring", c_void_p), ("v_ring", c_void_p), ("ring_batch_stride", c_int64), ("ring_row_stride", c_int64),
+        ("evict_slot", c_int32), ("write_slot", c_int32),
+        ("k_coef", c_void_p), ("v_coef", c_void_p), ("kc_list", c_void_p), ("vc_list", c_void_p),
+        ("Ck", c_int32), ("Cv", c_int32), ("N", c_int32), ("T", c_int32), ("phase", c_int64),
+        ("k_mid", c_void_p), ("v_mid", c_void_p), ("k_mid_batch_stride", c_int64), ("v_mid_batch_stride", c_int64),
+        ("cap_pages", c_int32), ("mid_pos", c_int64),
+        ("kn_list", c_void_p), ("kn_h_list", c_void_p), ("k_pad_h_list", c_void_p),
+        ("vn_list", c_void_p), ("vn_h_list", c_void_p), ("v_pad_h_list", c_void_p),
+        ("Cnk", c_int32), ("Cnv", c_int32), ("B", c_int32), ("Hkv", c_int32), ("width", c_int32), ("dtype", c_int32),
+    ]
+
+
 _SIGNATURES = {
     "fa_last_error_string": (c_char_p, []),
     "fa_abi_version": (c_int, []),
     "fa_decode_args_size": (c_size_t, []),
+    "fa_stream_args_size": (c_size_t, []),
+    "fa_stream_update": (c_int, [ctypes.POINTER(StreamArgs), c_void_p]),
     "fa_mat_fourier": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                c_int64, c_int, c_void_p, c_size_t, c_void_p]),
     "fa_mat_fourier_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
@@ -105,6 +123,9 @@ def load():
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
+    if lib.fa_stream_args_size() != ctypes.sizeof(StreamArgs):
+        raise ImportError(f"fa_stream_args is {lib.fa_stream_args_size()} bytes in the library but "
+                          f"{ctypes.sizeof(StreamArgs)} in the Python mirror")
     if lib.fa_decode_args_size() != ctypes.sizeof(DecodeArgs):
         raise ImportError(f"fa_decode_args is {lib.fa_decode_args_size()} bytes in the library but "
                           f"{ctypes.sizeof(DecodeArgs)} in the binding")

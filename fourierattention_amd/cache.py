@@ -41,8 +41,9 @@ class _Tensor:
     """Per-layer state of one of K / V."""
 
     def __init__(self):
-        self.init: Optional[torch.Tensor] = None        # (B, I, HD)
-        self.ring: Optional[torch.Tensor] = None        # (B, W, HD) when compressed, else growing (B, cap, HD)
+        self.il: Optional[torch.Tensor] = None          # (B, I + W + 1, HD): sink rows, then the window slots
+        self.init: Optional[torch.Tensor] = None        # view il[:, :I]
+        self.ring: Optional[torch.Tensor] = None        # view il[:, I:] (W + 1 slots) when compressed, else growing (B, cap, HD)
         self.coef: Optional[torch.Tensor] = None        # (B, 2N, C) fp32
         self.mid: Optional[MidStore] = None             # paged store of the stored dims of the mid rows
         self.stats32: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None  # avg_u, avg_d, scale fp32
@@ -55,7 +56,7 @@ class _Layer:
         self.compressed = False   # sink / coefficients / mid store exist
         self.window_only = True   # attention reads the window only (short prompt, or the append branch)
         self.growing = True       # the window is a plain growing buffer rather than a ring
-        self.ring_head = 0        # index of the oldest window row (ring mode)
+        self.spare = 0            # the window slot that holds no row (ring mode: W + 1 slots for W rows)
         self.n_local = 0
         self.n_mid = 0
         self.version = 0        # bumped by every update; lets views detect staleness
@@ -213,21 +214,33 @@ class DynamicCache:
         return self.maxtokens - self.numinittokens - self.maxlocallen
 
     def _window_in_order(self, layer: _Layer, t: _Tensor) -> torch.Tensor:
-        if layer.growing or layer.ring_head == 0:
+        if layer.growing:
             return t.ring[:, : layer.n_local, :]
-        return torch.cat([t.ring[:, layer.ring_head:, :], t.ring[:, : layer.ring_head, :]], dim=1)
+        sp = layer.spare      # oldest row sits right after the spare slot
+        if sp == t.ring.shape[1] - 1:
+            return t.ring[:, :sp, :]
+        return torch.cat([t.ring[:, sp + 1:, :], t.ring[:, :sp, :]], dim=1)
 
     def _window_segments(self, layer: _Layer):
-        """The window as up to two (k, v) views whose union is the window (order irrelevant to attention)."""
+        """The window as (k, v) views whose union is the window (order irrelevant to attention)."""
         return [(layer.k.ring[:, : layer.n_local, :], layer.v.ring[:, : layer.n_local, :])]
+
+    def _il_segments(self, layer: _Layer):
+        """Sink + window of a compressed layer as two views of the one buffer: the rows before and the rows
+        after the spare window slot."""
+        cut = self.numinittokens + layer.spare
+        return [(layer.k.il[:, :cut, :], layer.v.il[:, :cut, :]), (layer.k.il[:, cut + 1:, :], layer.v.il[:, cut + 1:, :])]
 
     def _compress_tensor(self, t: _Tensor, states: torch.Tensor, c32: torch.Tensor, n32: torch.Tensor, nh32: torch.Tensor,
                          nh_host, is_v: bool, L: int, fft_rows: int, n_f: int):
         I, W = self.numinittokens, self.maxlocallen
         B, S, HD = states.shape
         mid = states[:, I: S - W, :]
-        t.init = states[:, :I, :].contiguous()
-        t.ring = states[:, S - W:, :].contiguous()
+        t.il = torch.empty((B, I + W + 1, HD), dtype=states.dtype, device=states.device)
+        t.init, t.ring = t.il[:, :I, :], t.il[:, I:, :]
+        t.init.copy_(states[:, :I, :])
+        t.ring[:, :W, :].copy_(states[:, S - W:, :])
+        t.ring[:, W, :].zero_()
         cap = max(self._book.t_x, L) + 1
         t.mid = MidStore(B, n32, nh32, nh_host, self.heads, self.head_dim, cap, states.dtype, states.device, is_v)
         t.mid.pack(states, I, L)
@@ -282,18 +295,18 @@ class DynamicCache:
                                                    step.fft_rows, n_f)
                 if self._tables is None and layer_idx == 0:
                     self._tables = ops.decode_tables(n_f, self.period_reconstruct, self.device)
-                layer.compressed, layer.window_only, layer.growing, layer.ring_head = True, False, False, 0
+                layer.compressed, layer.window_only, layer.growing, layer.spare = True, False, False, self.maxlocallen
                 layer.n_local, layer.n_mid = self.maxlocallen, step.mid_rows
                 self._store_stats(layer_idx, ks, ku, kd, vs, vu, vd)
                 kview, vview = CacheParts(self, layer_idx, "k"), CacheParts(self, layer_idx, "v")
             else:
-                layer.compressed, layer.window_only, layer.growing, layer.ring_head = False, True, True, 0
+                layer.compressed, layer.window_only, layer.growing, layer.spare = False, True, True, 0
                 layer.n_local, layer.n_mid = q_len, 0
                 cap = q_len + max(int(self.maxnewtokens), 16)
                 for t, s in ((layer.k, k), (layer.v, v)):
                     t.ring = torch.empty((bsz, cap, s.shape[2]), dtype=s.dtype, device=s.device)
                     t.ring[:, :q_len, :].copy_(s)
-                    t.init, t.coef, t.mid, t.stats32 = None, None, None, None
+                    t.il, t.init, t.coef, t.mid, t.stats32 = None, None, None, None, None
                 kview, vview = self._placeholder_parts(layer_idx, bsz, heads * head_dim)
             if len(self.key_cache) <= layer_idx:
                 self.key_cache.append(kview)
@@ -311,7 +324,7 @@ class DynamicCache:
                 # by turning the ring into a growing buffer
                 for t in (layer.k, layer.v):
                     t.ring = self._window_in_order(layer, t).contiguous()
-                layer.ring_head, layer.growing, layer.window_only = 0, True, True
+                layer.spare, layer.growing, layer.window_only = 0, True, True
             for t, s in ((layer.k, k), (layer.v, v)):
                 need = layer.n_local + q_len
                 if need > t.ring.shape[1]:
@@ -339,16 +352,17 @@ class DynamicCache:
         self.curr_tokennum[layer_idx] = lb.curr_tokennum
         p = step.phase
         l32 = self._lists32[layer_idx]
-        h = layer.ring_head
-        for t, new, c32 in ((layer.k, k, l32[0]), (layer.v, v, l32[4])):
-            oldest = t.ring[:, h, :]
-            ops.coeff_update_(t.coef, oldest, c32, p, self._book.t_c)
+        slots = self.maxlocallen + 1
+        sp = layer.spare
+        oldest = (sp + 1) % slots
+        for t in (layer.k, layer.v):
             if layer.n_mid >= t.mid.cap_tokens:
                 t.mid.grow(layer.n_mid, 2 * t.mid.cap_tokens)
-            t.mid.append(oldest, layer.n_mid)
-            t.ring[:, h, :].copy_(new[:, 0, :])
+        # one launch: coefficients and page store take the oldest row, the new token takes the spare slot
+        ops.stream_update(k[:, 0, :], v[:, 0, :], layer.k.ring, layer.v.ring, oldest, sp, layer.k.coef, layer.v.coef,
+                          l32[0], l32[4], p, self._book.t_c, layer.k.mid, layer.v.mid, layer.n_mid)
         layer.n_mid += 1
-        layer.ring_head = (h + 1) % self.maxlocallen
+        layer.spare = oldest
         kview, vview = CacheParts(self, layer_idx, "k"), CacheParts(self, layer_idx, "v")
         self.key_cache[layer_idx], self.value_cache[layer_idx] = kview, vview
         return kview, vview
@@ -386,7 +400,7 @@ class DynamicCache:
         if layer.window_only:
             return ops.decode_attn_raw(q, self._window_segments(layer), None, None, None, None, None, None, l32, num_heads,
                                        num_kv_heads, 0, 1, sm_scale, timings=timings)
-        segs = [(layer.k.init, layer.v.init)] + self._window_segments(layer)
+        segs = self._il_segments(layer)
         return ops.decode_attn_raw(q, segs, layer.k.coef, layer.v.coef, layer.k.mid, layer.v.mid, layer.k.stats32,
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
                                    sm_scale, tables=self._tables, force_generic=self.force_generic, timings=timings)

@@ -188,6 +188,37 @@ def coeff_update_(c: torch.Tensor, row: torch.Tensor, cols: Optional[torch.Tenso
     return c
 
 
+def stream_update(k_new: torch.Tensor, v_new: torch.Tensor, k_ring: torch.Tensor, v_ring: torch.Tensor, evict_slot: int,
+                  write_slot: int, k_coef: torch.Tensor, v_coef: torch.Tensor, kc_list: torch.Tensor, vc_list: torch.Tensor,
+                  phase: int, T: int, k_mid, v_mid, mid_pos: int) -> None:
+    """One streaming step of one layer in one launch (the body of cache_utils_fourier.py:731-748 for K and V):
+    the rows in window slot ``evict_slot`` enter the coefficients (rank-1 update at ``phase``) and the page
+    stores (at token ``mid_pos``); ``k_new, v_new (B, width)`` are written to window slot ``write_slot``.
+    ``k_ring, v_ring (B, slots, width)`` share their strides; ``k_mid, v_mid`` are ``MidStore`` objects."""
+    _require_gpu(k_ring, "k_ring")
+    assert k_new.dim() == 2 and k_new.stride(1) == 1 and v_new.stride() == k_new.stride()
+    assert k_ring.stride(2) == 1 and v_ring.stride() == k_ring.stride() and k_ring.shape == v_ring.shape
+    assert evict_slot != write_slot and k_mid.cap_pages == v_mid.cap_pages
+    a = _lib.StreamArgs()
+    a.k_new, a.v_new, a.new_batch_stride = k_new.data_ptr(), v_new.data_ptr(), k_new.stride(0)
+    a.k_ring, a.v_ring = k_ring.data_ptr(), v_ring.data_ptr()
+    a.ring_batch_stride, a.ring_row_stride = k_ring.stride(0), k_ring.stride(1)
+    a.evict_slot, a.write_slot = int(evict_slot), int(write_slot)
+    a.k_coef, a.v_coef = _ptr(k_coef), _ptr(v_coef)
+    a.kc_list, a.vc_list = _ptr(kc_list), _ptr(vc_list)
+    a.Ck, a.Cv = int(kc_list.numel()), int(vc_list.numel())
+    a.N, a.T, a.phase = int(k_coef.shape[1] // 2), int(T), int(phase)
+    a.k_mid, a.v_mid = k_mid.data.data_ptr(), v_mid.data.data_ptr()
+    a.k_mid_batch_stride, a.v_mid_batch_stride = int(k_mid.batch_stride), int(v_mid.batch_stride)
+    a.cap_pages, a.mid_pos = int(k_mid.cap_pages), int(mid_pos)
+    a.kn_list, a.kn_h_list, a.k_pad_h_list = _ptr(k_mid.n_list32), k_mid.n_h32.data_ptr(), k_mid.pad_h32.data_ptr()
+    a.vn_list, a.vn_h_list, a.v_pad_h_list = _ptr(v_mid.n_list32), v_mid.n_h32.data_ptr(), v_mid.pad_h32.data_ptr()
+    a.Cnk, a.Cnv = int(k_mid.Cn), int(v_mid.Cn)
+    a.B, a.Hkv, a.width, a.dtype = int(k_ring.shape[0]), int(k_mid.Hkv), int(k_ring.shape[2]), dtype_code(k_ring.dtype)
+    import ctypes
+    check(_lib.load().fa_stream_update(ctypes.byref(a), _stream(k_ring.device)))
+
+
 class MultiDimHiPPO2(torch.nn.Module):
     """Same call contract as the reference class (TRI:840-865): without ``slice_input`` the
     whole ``base_input (B, L, C)`` is projected (period and length ``int(1/dt)``: longer inputs

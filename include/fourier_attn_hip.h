@@ -110,6 +110,38 @@ int fa_reconstruct(const float* c, const float* avg_u, const float* avg_d, const
 int fa_coeff_update(float* c, const void* row, int row_dtype, int64_t row_batch_stride,
                     const int32_t* cols, int B, int N, int Mc, int64_t p, int T, fa_stream_t stream);
 
+/* One streaming step of one layer in a single launch (the body of CACHE:731-748 for
+ * K and V): the row in window slot evict_slot leaves the window -- rank-1
+ * coefficient update at `phase` over its compressed columns (fa_coeff_update),
+ * its stored columns appended at token position mid_pos of the page store
+ * (fa_mid_append) -- and the new token is written to window slot write_slot.
+ * The window buffers are (B, slots, width) with batch / row strides in elements;
+ * evict_slot != write_slot (keep one slot more than the window is long), so
+ * the three pieces of work are independent.  Pointers of a tensor whose column
+ * count is 0 may be NULL. */
+typedef struct fa_stream_args {
+  const void* k_new; const void* v_new;      /* (B, width) new token rows, batch stride new_batch_stride */
+  int64_t new_batch_stride;
+  void* k_ring; void* v_ring;                /* window buffers */
+  int64_t ring_batch_stride, ring_row_stride;
+  int32_t evict_slot, write_slot;
+  float* k_coef; float* v_coef;              /* (B, 2N, Ck) / (B, 2N, Cv) fp32 */
+  const int32_t* kc_list; const int32_t* vc_list;
+  int32_t Ck, Cv, N, T;
+  int64_t phase;
+  void* k_mid; void* v_mid;                  /* page stores (see below) */
+  int64_t k_mid_batch_stride, v_mid_batch_stride;
+  int32_t cap_pages;
+  int64_t mid_pos;
+  const int32_t* kn_list; const int32_t* kn_h_list; const int32_t* k_pad_h_list;
+  const int32_t* vn_list; const int32_t* vn_h_list; const int32_t* v_pad_h_list;
+  int32_t Cnk, Cnv;
+  int32_t B, Hkv, width, dtype;
+} fa_stream_args;
+
+int fa_stream_update(const fa_stream_args* args, fa_stream_t stream);
+size_t fa_stream_args_size(void);
+
 /* ---------------------------------------------------------------------------
  * Decode attention (triton_fourier_attn, TRI:684-779; kernel TRI:464-681)
  * ------------------------------------------------------------------------- */
