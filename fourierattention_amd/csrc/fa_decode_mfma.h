@@ -88,19 +88,21 @@ static inline size_t tables_bytes(int N) {
 // constants sit in LDS as float4 {c, s, c', s'} per (row tile, lane group), 64 bytes between row tiles.
 // They are fetched in batches of four tiles, two batches in flight, so that the LDS latency hides behind
 // the arithmetic of the previous batch instead of being paid once per tile.
-__device__ __forceinline__ void rot_issue(const void* lane_base, int batch, uint4v (&buf)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) buf[j] = lds_read_b128_async((const char*)lane_base + (batch * 4 + j) * 64);
+template <int BATCH>
+__device__ __forceinline__ void rot_issue(unsigned lane_base, uint4v (&buf)[4]) {
+  buf[0] = lds_read_b128_async_at<(BATCH * 4 + 0) * 64>(lane_base);
+  buf[1] = lds_read_b128_async_at<(BATCH * 4 + 1) * 64>(lane_base);
+  buf[2] = lds_read_b128_async_at<(BATCH * 4 + 2) * 64>(lane_base);
+  buf[3] = lds_read_b128_async_at<(BATCH * 4 + 3) * 64>(lane_base);
 }
 // the same, issued only once `after` has been computed: keeps a refill of a constant buffer behind the
 // arithmetic that consumed its previous contents (otherwise all batches are hoisted and held at once)
-__device__ __forceinline__ void rot_issue_after(const void* lane_base, int batch, uint4v (&buf)[4], float after) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const unsigned addr =
-        (unsigned)(size_t)(const __attribute__((address_space(3))) void*)((const char*)lane_base + (batch * 4 + j) * 64);
-    asm volatile("ds_read_b128 %0, %1 ; after %2" : "=v"(buf[j]) : "v"(addr), "v"(after));
-  }
+template <int BATCH>
+__device__ __forceinline__ void rot_issue_after(unsigned lane_base, uint4v (&buf)[4], float after) {
+  asm volatile("ds_read_b128 %0, %1 offset:%3 ; after %2" : "=v"(buf[0]) : "v"(lane_base), "v"(after), "n"((BATCH * 4 + 0) * 64));
+  asm volatile("ds_read_b128 %0, %1 offset:%3 ; after %2" : "=v"(buf[1]) : "v"(lane_base), "v"(after), "n"((BATCH * 4 + 1) * 64));
+  asm volatile("ds_read_b128 %0, %1 offset:%3 ; after %2" : "=v"(buf[2]) : "v"(lane_base), "v"(after), "n"((BATCH * 4 + 2) * 64));
+  asm volatile("ds_read_b128 %0, %1 offset:%3 ; after %2" : "=v"(buf[3]) : "v"(lane_base), "v"(after), "n"((BATCH * 4 + 3) * 64));
 }
 __device__ __forceinline__ void rot_pair(float c, float s, float& x, float& y) {
   const float sy = s * y, sx = s * x;
@@ -110,25 +112,30 @@ __device__ __forceinline__ void rot_pair(float c, float s, float& x, float& y) {
 // pair(rt, f2, c, s) applies one rotation and returns one of its results; pin(b) passes the results of
 // batch b (row tiles 4b .. 4b+3) through an empty asm volatile, which keeps their arithmetic above the
 // next wait (it is otherwise sunk to its uses, and every batch of constants is then held at once);
-// batches 0 and 1 must already be in flight in rc[0], rc[1]
-template <int NT, typename F, typename P>
-__device__ __forceinline__ void rot_apply(const void* lane_base, uint4v (&rc)[2][4], F&& pair, P&& pin) {
+// the first NBUF batches must already be in flight in rc[0 .. NBUF-1] (NBUF = 2 hides the LDS latency of a batch
+// behind the arithmetic of the one before; NBUF = 1 saves 16 registers and pays the latency)
+template <int NT, int NBUF, int B, typename F, typename P>
+__device__ __forceinline__ void rot_apply_from(unsigned lane_base, uint4v (&rc)[NBUF][4], F&& pair, P&& pin) {
   constexpr int NB = NT / 4;
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    if (b + 1 < NB) lds_wait_for4<4>(rc[b & 1]);
-    else lds_wait_for4<0>(rc[b & 1]);
+  if constexpr (B < NB) {
+    if (NBUF == 2 && B + 1 < NB) lds_wait_for4<4>(rc[B % NBUF]);
+    else lds_wait_for4<0>(rc[B % NBUF]);
     float last = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint4v raw = rc[b & 1][j];
+      const uint4v raw = rc[B % NBUF][j];
       const unsigned c0 = raw[0], s0 = raw[1], c1 = raw[2], s1 = raw[3];  // scalars first: see fa_swap16
-      pair(b * 4 + j, 0, __builtin_bit_cast(float, c0), __builtin_bit_cast(float, s0));
-      last = pair(b * 4 + j, 1, __builtin_bit_cast(float, c1), __builtin_bit_cast(float, s1));
+      pair(B * 4 + j, 0, __builtin_bit_cast(float, c0), __builtin_bit_cast(float, s0));
+      last = pair(B * 4 + j, 1, __builtin_bit_cast(float, c1), __builtin_bit_cast(float, s1));
     }
-    pin(b);
-    if (b + 2 < NB) rot_issue_after(lane_base, b + 2, rc[b & 1], last);
+    pin(B);
+    if constexpr (B + NBUF < NB) rot_issue_after<B + NBUF>(lane_base, rc[B % NBUF], last);
+    rot_apply_from<NT, NBUF, B + 1>(lane_base, rc, pair, pin);
   }
+}
+template <int NT, int NBUF, typename F, typename P>
+__device__ __forceinline__ void rot_apply(unsigned lane_base, uint4v (&rc)[NBUF][4], F&& pair, P&& pin) {
+  rot_apply_from<NT, NBUF, 0>(lane_base, rc, pair, pin);
 }
 
 template <typename E>
@@ -215,8 +222,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int nks = dpk >> 5;
     const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
     const bool has_k = has_mn && nks > 0;
-    // every page moves 2*KMAX fragments so that the number of loads in flight is a compile-time constant;
-    // a head with fewer stored dims repeats its first fragment into the unused slots
+    // a page moves the fragments the head really has (two stages: the page wait below is always "all landed")
     auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* kp = kbase + (int64_t)t * dpk * 32;
       unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
@@ -224,7 +230,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
         for (int ks = 0; ks < KMAX; ++ks)
-          load_frag_to_lds<2>(kp + (ks < nks ? tb * nks + ks : 0) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
+          if (ks < nks) load_frag_to_lds<2>(kp + (tb * nks + ks) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
     };
     if (has_k) {
 #pragma unroll
@@ -313,24 +319,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
     __syncthreads();   // the rotation constants in LDS are complete
-    const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
+    const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
 
     for (int it = 0; it <= n_it; ++it) {
       if (it < n_it) {
         const int t = t_beg + it;
-        uint4v kraw[2 * KMAX];
+        uint4v kraw[4];   // two ksteps of both token blocks at a time
+        const unsigned kst = lds_addr_of(&s_stage[w][it % NST][0]) + lane * 16;
         uint4v rc[2][4];
         if (has_k) {
           // pages t+1 .. t+NST-2 may still be in flight; page t has landed: start its LDS reads now
           if (it + NST - 2 < n_it) wait_vmcnt<(NST - 2) * 2 * KMAX>();
           else wait_vmcnt<0>();
           if (it + NST - 1 < n_it) issue_k(t + NST - 1);   // refills the stage read one page ago
-          const unsigned char* st = &s_stage[w][it % NST][0];
-#pragma unroll
-          for (int f = 0; f < 2 * KMAX; ++f) kraw[f] = lds_read_b128_async(st + (size_t)f * 1024 + lane * 16);
+          // ksteps 0, 1: issued early, consumed after the coefficient-domain product
+          kraw[0] = lds_read_b128_async_at<0>(kst);
+          kraw[1] = lds_read_b128_async_at<1024>(kst);
+          kraw[2] = lds_read_b128_async_at<KMAX * 1024>(kst);
+          kraw[3] = lds_read_b128_async_at<(KMAX + 1) * 1024>(kst);
         }
-        rot_issue(rot_lane, 0, rc[0]);
-        if (2 * KS > 4) rot_issue(rot_lane, 1, rc[1]);
+        rot_issue<0>(rot_lane, rc[0]);
+        if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
         float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -344,7 +353,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
         }
         // advance W' by one page step
-        rot_apply<2 * KS>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
+        rot_apply<2 * KS, 2>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
           rot_pair(c, sn, Wc[rt][f2], Ws[rt][f2]);
           return Ws[rt][f2];
         }, [&](int b) {
@@ -355,13 +364,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         float4v accm[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
         if (has_k) {
 #pragma unroll
-          for (int f = 0; f < 2 * KMAX; ++f) lds_wait_for(kraw[f]);
-#pragma unroll
-          for (int s = 0; s < KMAX; ++s)
-            if (s < nks) {
-              accm[0] = M::mma(__builtin_bit_cast(vec8, kraw[s]), Qb[s], accm[0]);
-              accm[1] = M::mma(__builtin_bit_cast(vec8, kraw[KMAX + s]), Qb[s], accm[1]);
+          for (int s0 = 0; s0 < KMAX; s0 += 2) {
+            if (s0 > 0) {
+              if (s0 >= nks) break;
+              kraw[0] = lds_read_b128_async_at<0>(kst + s0 * 1024);
+              kraw[1] = lds_read_b128_async_at<1024>(kst + s0 * 1024);
+              kraw[2] = lds_read_b128_async_at<KMAX * 1024>(kst + s0 * 1024);
+              kraw[3] = lds_read_b128_async_at<(KMAX + 1) * 1024>(kst + s0 * 1024);
             }
+            lds_wait_for4<0>(kraw);
+#pragma unroll
+            for (int ss = 0; ss < 2; ++ss)
+              if (s0 + ss < nks) {
+                accm[0] = M::mma(__builtin_bit_cast(vec8, kraw[ss]), Qb[s0 + ss], accm[0]);
+                accm[1] = M::mma(__builtin_bit_cast(vec8, kraw[2 + ss]), Qb[s0 + ss], accm[1]);
+              }
+          }
         }
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
@@ -379,12 +397,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int ndg = dpv >> 4;
     const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
     const bool has_v = has_mn && ndg > 0;
-    // VMAX fragments per page whatever the head holds (see the score waves)
     auto issue_v = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* vp = vbase + (int64_t)t * dpv * 32;
       unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
 #pragma unroll
-      for (int f = 0; f < VMAX; ++f) load_frag_to_lds<2>(vp + (f < ndg ? f : 0) * 512 + lane * 8, st + f * 1024);
+      for (int f = 0; f < VMAX; ++f)
+        if (f < ndg) load_frag_to_lds<2>(vp + f * 512 + lane * 8, st + f * 1024);
     };
     if (has_v) {   // first pages requested before the tables (see the score waves)
 #pragma unroll
@@ -405,22 +423,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
     __syncthreads();   // the rotation constants in LDS are complete
-    const float4v* rot_lane = &s_rot[(sl * 2 * KS) * 4 + lg];
+    const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
 
     for (int it = 0; it <= n_it; ++it) {
       if (it > 0) {
         const int t = t_beg + it - 1, buf = (it - 1) & 1;
         const int pg = it - 1;   // page index within the split
-        uint4v rc[2][4];
-        rot_issue(rot_lane, 0, rc[0]);
-        if (2 * KS > 4) rot_issue(rot_lane, 1, rc[1]);
+        constexpr int RCB = VMAX > 4 ? 1 : 2;   // the wide variant has no registers to spare for a second batch
+        uint4v rc[RCB][4];
+        rot_issue<0>(rot_lane, rc[0]);
+        if (RCB == 2 && 2 * KS > 4) rot_issue<1>(rot_lane, rc[RCB - 1]);
         if (has_v) {
           if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
           else wait_vmcnt<0>();
           if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
         }
         // the g history moves into the frame of this page
-        rot_apply<2 * KS>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
+        rot_apply<2 * KS, RCB>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
           float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
           rot_pair(c, sn, x, y);
           hacc[rt][2 * f2] = x;
@@ -433,11 +452,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         float sc[8];
         {
           uint4v part[kFreqWaves][2];
-#pragma unroll
-          for (int ww = 0; ww < kFreqWaves; ++ww) {
-            part[ww][0] = lds_read_b128_async(&s_part[buf][ww][lc * kPart + 8 * lg]);
-            part[ww][1] = lds_read_b128_async(&s_part[buf][ww][lc * kPart + 8 * lg + 4]);
-          }
+          const unsigned pst = lds_addr_of(&s_part[buf][0][lc * kPart + 8 * lg]);
+          constexpr int kW = 16 * kPart * 4;   // bytes between the partials of two score waves
+          part[0][0] = lds_read_b128_async_at<0>(pst);
+          part[0][1] = lds_read_b128_async_at<16>(pst);
+          part[1][0] = lds_read_b128_async_at<kW>(pst);
+          part[1][1] = lds_read_b128_async_at<kW + 16>(pst);
+          part[2][0] = lds_read_b128_async_at<2 * kW>(pst);
+          part[2][1] = lds_read_b128_async_at<2 * kW + 16>(pst);
+          part[3][0] = lds_read_b128_async_at<3 * kW>(pst);
+          part[3][1] = lds_read_b128_async_at<3 * kW + 16>(pst);
 #pragma unroll
           for (int ww = 0; ww < kFreqWaves; ++ww) {
             lds_wait_for(part[ww][0]);
@@ -451,11 +475,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     (__builtin_bit_cast(float, u2) + __builtin_bit_cast(float, u3));
           }
         }
-        uint4v vraw[VMAX];
+        uint4v vraw[4];   // four dim groups at a time
+        const unsigned vst = lds_addr_of(&s_stage[w][pg % NST][0]) + lane * 16;
         if (has_v) {
-          const unsigned char* st = &s_stage[w][pg % NST][0];
-#pragma unroll
-          for (int f = 0; f < VMAX; ++f) vraw[f] = lds_read_b128_async(st + (size_t)f * 1024 + lane * 16);
+          vraw[0] = lds_read_b128_async_at<0>(vst);
+          vraw[1] = lds_read_b128_async_at<1024>(vst);
+          vraw[2] = lds_read_b128_async_at<2048>(vst);
+          vraw[3] = lds_read_b128_async_at<3072>(vst);
         }
         if (ragged_tail && t == n_tiles - 1) {
           const int tok0 = t * 32 + 8 * lg;
@@ -491,10 +517,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           hacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[rt], pf, hacc[rt], 0, 0, 0);
         if (has_v) {
 #pragma unroll
-          for (int f = 0; f < VMAX; ++f) lds_wait_for(vraw[f]);
+          for (int f0 = 0; f0 < VMAX; f0 += 4) {
+            if (f0 > 0) {
+              if (f0 >= ndg) break;
+              vraw[0] = lds_read_b128_async_at<0>(vst + f0 * 1024);
+              vraw[1] = lds_read_b128_async_at<1024>(vst + f0 * 1024);
+              vraw[2] = lds_read_b128_async_at<2048>(vst + f0 * 1024);
+              vraw[3] = lds_read_b128_async_at<3072>(vst + f0 * 1024);
+            }
+            lds_wait_for4<0>(vraw);
 #pragma unroll
-          for (int f = 0; f < VMAX; ++f)
-            if (f < ndg) oacc[f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f]);
+            for (int f = 0; f < 4; ++f)
+              if (f0 + f < ndg) oacc[f0 + f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f0 + f]);
+          }
         }
       }
       barrier_lds_only();

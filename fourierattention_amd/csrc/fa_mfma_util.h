@@ -52,6 +52,18 @@ __device__ __forceinline__ uint4v lds_read_b128_async(const void* lds_ptr) {
   asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
   return r;
 }
+// the same at lds_addr + OFF with OFF in the instruction's immediate field: reads of one structure share one
+// address register instead of computing (and keeping) an address each
+__device__ __forceinline__ unsigned lds_addr_of(const void* lds_ptr) {
+  return (unsigned)(size_t)(const __attribute__((address_space(3))) void*)lds_ptr;
+}
+template <int OFF>
+__device__ __forceinline__ uint4v lds_read_b128_async_at(unsigned lds_addr) {
+  static_assert(OFF >= 0 && OFF < 65536 && OFF % 16 == 0, "immediate offset of ds_read_b128");
+  uint4v r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(lds_addr), "n"(OFF));
+  return r;
+}
 // the read above completes asynchronously: tie the wait to the value so no use can be scheduled before it
 __device__ __forceinline__ void lds_wait_for(uint4v& r) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r)::"memory"); }
 // same for a batch of four reads, leaving the AFTER LDS operations issued after the batch in flight (LDS
