@@ -955,8 +955,8 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
   const int KS = N / 64;
   half8* tabE = (half8*)tables;
   half8* tabET = tabE + kFreqWaves * 2 * KS * 64;
-  float2v* rot = (float2v*)(tabET + kFreqWaves * 2 * KS * 64);
-  const int total = 2 * kFreqWaves * 2 * KS * 64 + N;
+  float2v* rot = (float2v*)(tabET + 2 * kFreqWaves * 2 * KS * 64);
+  const int total = 3 * kFreqWaves * 2 * KS * 64 + 2 * N;
   decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N);
 }
 
@@ -1021,7 +1021,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.vn_h = a.vn_h_list; mp.vpad_h = a.v_pad_h_list;
         mp.tabE = (const half8*)tables;
         mp.tabET = mp.tabE + kFreqWaves * 2 * KS * 64;
-        mp.rot = (const float2v*)(mp.tabET + kFreqWaves * 2 * KS * 64);
+        mp.rot = (const float2v*)(mp.tabET + 2 * kFreqWaves * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;

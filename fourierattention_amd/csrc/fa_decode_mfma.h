@@ -20,6 +20,7 @@
 #pragma once
 
 #include "fa_mfma_util.h"
+#include <type_traits>
 
 namespace fa_mfma {
 
@@ -34,13 +35,15 @@ constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one 
 // ---------------------------------------------------------------------------
 // constant operand tables (depend on T and N only); KS = N / 64 ksteps per frequency slice
 //   tabE  [4 slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM
-//   tabET [4 slices][2*KS row tiles][64 lanes]  x half8 : A operand of the g GEMM
-//   rot   [N] float2 : (cos, sin)(2 pi f 32 / T), the per-page frame rotation
+//   tabET [2 pages][4 slices][2*KS row tiles][64 lanes] x half8 : A operand of the g GEMM for the tokens of
+//         a page (0) and for the tokens of the page after it seen from the same page start (1)
+//   rot   [2][N] float2 : (cos, sin)(2 pi f 32 / T) and (cos, sin)(2 pi f 64 / T), the frame rotation of one
+//         page step and of two
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ tabE, half8* __restrict__ tabET,
                                                             float2v* __restrict__ rot, int KS, int T, int N) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  const int nE = kFreqWaves * 2 * KS * 64, nET = kFreqWaves * 2 * KS * 64;
+  const int nE = kFreqWaves * 2 * KS * 64, nET = 2 * kFreqWaves * 2 * KS * 64;
   if (idx < nE) {
     const int lane = idx & 63, s = (idx >> 6) % KS, rb = ((idx >> 6) / KS) & 1, w = (idx >> 6) / (2 * KS);
     const int lg = lane >> 4, lc = lane & 15;
@@ -57,7 +60,8 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
     tabE[idx] = out;
   } else if (idx < nE + nET) {
     const int k = idx - nE;
-    const int lane = k & 63, rt = (k >> 6) % (2 * KS), w = (k >> 6) / (2 * KS);
+    const int lane = k & 63, rt = (k >> 6) % (2 * KS), w = ((k >> 6) / (2 * KS)) % kFreqWaves;
+    const int page = (k >> 6) / (2 * KS * kFreqWaves);
     const int lg = lane >> 4, rho = lane & 15;
     const int f = w * 16 * KS + freq_of(rt, rho >> 2, (rho & 3) >> 1);
     const int cs = rho & 1;
@@ -65,21 +69,21 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float sn, co;
-      fa_sincos_phase(f, 8 * lg + e, T, &sn, &co);
+      fa_sincos_phase(f, 32 * page + 8 * lg + e, T, &sn, &co);
       out[e] = (_Float16)(cs ? sn : co);
     }
     tabET[k] = out;
-  } else if (idx < nE + nET + N) {
-    const int f = idx - nE - nET;
+  } else if (idx < nE + nET + 2 * N) {
+    const int f = (idx - nE - nET) % N, two = (idx - nE - nET) / N;
     float sn, co;
-    fa_sincos_phase(f, 32, T, &sn, &co);
-    rot[f] = float2v{co, sn};
+    fa_sincos_phase(f, 32 * (1 + two), T, &sn, &co);
+    rot[two * N + f] = float2v{co, sn};
   }
 }
 
 static inline size_t tables_bytes(int N) {
   const int KS = N / 64;
-  return (size_t)(2 * kFreqWaves * 2 * KS * 64) * 16 + (size_t)N * 8;
+  return (size_t)(3 * kFreqWaves * 2 * KS * 64) * 16 + (size_t)2 * N * 8;
 }
 
 
@@ -138,6 +142,23 @@ __device__ __forceinline__ void rot_apply(unsigned lane_base, uint4v (&rc)[NBUF]
   rot_apply_from<NT, NBUF, 0>(lane_base, rc, pair, pin);
 }
 
+// hacc[rt] += A[rt] . pf for the second page of a frame: the A operands (E^T of token offsets 32..63) come from
+// LDS four row tiles at a time (1 KiB apart per row tile)
+template <int NT, int RT0>
+__device__ __forceinline__ void et1_accumulate(unsigned lane_base, half8 pf, float4v (&hacc)[NT], uint4v (&a)[4]) {
+  if constexpr (RT0 < NT) {
+    a[0] = lds_read_b128_async_at<(RT0 + 0) * 1024>(lane_base);
+    a[1] = lds_read_b128_async_at<(RT0 + 1) * 1024>(lane_base);
+    a[2] = lds_read_b128_async_at<(RT0 + 2) * 1024>(lane_base);
+    a[3] = lds_read_b128_async_at<(RT0 + 3) * 1024>(lane_base);
+    lds_wait_for4<0>(a);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      hacc[RT0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a[j]), pf, hacc[RT0 + j], 0, 0, 0);
+    et1_accumulate<NT, RT0 + 4>(lane_base, pf, hacc, a);
+  }
+}
+
 template <typename E>
 struct MidParams {
   const E* q;
@@ -182,6 +203,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[8][NST][kFragsMax * 1024];
   __shared__ float s_part[2][kFreqWaves][16 * kPart];
   __shared__ float4v s_rot[kFreqWaves * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
+  // Narrow pages leave LDS for a second g operand: the value waves then accumulate two pages per frame (the second
+  // through E^T of the token offsets 32..63, read from LDS) and rotate their history every other page only.
+  constexpr bool TWO = kFragsMax <= 4;
+  __shared__ float4v s_rot2[TWO ? kFreqWaves * 2 * KS * 4 : 1];   // the same for a step of two pages
+  __shared__ uint4v s_et1[TWO ? kFreqWaves * 2 * KS * 64 : 1];    // [slice][row tile][lane]
 
   const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
@@ -210,6 +236,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const float2v a = p.rot[fbase + freq_of(rt, lg, 0)];
       const float2v b = p.rot[fbase + freq_of(rt, lg, 1)];
       s_rot[(sl * 2 * KS + rt) * 4 + lg] = float4v{a[0], a[1], b[0], b[1]};
+      if (TWO) {
+        const float2v a2 = p.rot[N + fbase + freq_of(rt, lg, 0)];
+        const float2v b2 = p.rot[N + fbase + freq_of(rt, lg, 1)];
+        s_rot2[(sl * 2 * KS + rt) * 4 + lg] = float4v{a2[0], a2[1], b2[0], b2[1]};
+      }
     }
   }
 
@@ -412,6 +443,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     half8 ETa[2 * KS];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
+    if (TWO) {
+      const uint4v* src = (const uint4v*)(p.tabET + (kFreqWaves + sl) * 2 * KS * 64) + lane;
+#pragma unroll
+      for (int rt = 0; rt < 2 * KS; ++rt) s_et1[(sl * 2 * KS + rt) * 64 + lane] = src[rt * 64];
+    }
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -423,22 +459,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
     __syncthreads();   // the rotation constants in LDS are complete
-    const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
+    const unsigned rot_lane = lds_addr_of(TWO ? &s_rot2[(sl * 2 * KS) * 4 + lg] : &s_rot[(sl * 2 * KS) * 4 + lg]);
+    const unsigned et1_lane = lds_addr_of(&s_et1[TWO ? (sl * 2 * KS) * 64 + lane : 0]);
 
-    for (int it = 0; it <= n_it; ++it) {
-      if (it > 0) {
+    // one page of the value stage (page it - 1 of the split)
+    auto value_page = [&](int it, auto first_tag) {
         const int t = t_beg + it - 1, buf = (it - 1) & 1;
         const int pg = it - 1;   // page index within the split
         constexpr int RCB = VMAX > 4 ? 1 : 2;   // the wide variant has no registers to spare for a second batch
+        constexpr bool first_of_frame = decltype(first_tag)::value;   // first page of a frame (rotates), or second
         uint4v rc[RCB][4];
-        rot_issue<0>(rot_lane, rc[0]);
-        if (RCB == 2 && 2 * KS > 4) rot_issue<1>(rot_lane, rc[RCB - 1]);
+        if constexpr (first_of_frame) {
+          rot_issue<0>(rot_lane, rc[0]);
+          if (RCB == 2 && 2 * KS > 4) rot_issue<1>(rot_lane, rc[RCB - 1]);
+        }
         if (has_v) {
           if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
           else wait_vmcnt<0>();
           if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
         }
-        // the g history moves into the frame of this page
+        // the g history moves into the frame of this page (of this pair of pages)
+        if constexpr (first_of_frame)
         rot_apply<2 * KS, RCB>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
           float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
           rot_pair(c, sn, x, y);
@@ -512,9 +553,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int f = 0; f < VMAX; ++f) oacc[f] *= alpha;
         }
+        if constexpr (first_of_frame) {
 #pragma unroll
-        for (int rt = 0; rt < 2 * KS; ++rt)
-          hacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[rt], pf, hacc[rt], 0, 0, 0);
+          for (int rt = 0; rt < 2 * KS; ++rt)
+            hacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[rt], pf, hacc[rt], 0, 0, 0);
+        } else {
+          et1_accumulate<2 * KS, 0>(et1_lane, pf, hacc, rc[0]);   // the constant buffer is idle on these pages
+        }
         if (has_v) {
 #pragma unroll
           for (int f0 = 0; f0 < VMAX; f0 += 4) {
@@ -531,8 +576,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
               if (f0 + f < ndg) oacc[f0 + f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f0 + f]);
           }
         }
+    };
+    barrier_lds_only();   // iteration 0: the score waves are one page ahead
+    if constexpr (TWO) {
+      for (int it = 1; it <= n_it; it += 2) {
+        value_page(it, std::true_type{});
+        barrier_lds_only();
+        if (it + 1 <= n_it) {
+          value_page(it + 1, std::false_type{});
+          barrier_lds_only();
+        }
       }
-      barrier_lds_only();
+    } else {
+      for (int it = 1; it <= n_it; ++it) {
+        value_page(it, std::true_type{});
+        barrier_lds_only();
+      }
     }
 
     // ---- partials of this split ------------------------------------------------------
@@ -544,7 +603,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         p.pd[base] = dsum;
       }
       float* g = p.pg + base * 2 * N;
-      const int64_t last = (int64_t)32 * (t_end > t_beg ? t_end - 1 : t_beg);
+      const int64_t last = (int64_t)32 * (t_end > t_beg ? t_beg + (TWO ? ((n_it - 1) & ~1) : n_it - 1) : t_beg);
       float sn[2], co[2], s8, c8;   // stepped phases, as for the first page
       fast_sincos_phase(8, last, p.T, &s8, &c8);
 #pragma unroll
