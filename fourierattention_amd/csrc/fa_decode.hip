@@ -515,14 +515,17 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     m_raw = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
     d_raw = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
   }
-  float g_pre[2][kMergePre];                        // g partials of elements tid and tid + 1024
+  // g partials: two neighbouring threads share four consecutive coefficient rows of one head, one takes the even
+  // splits, the other the odd ones (16-byte loads: a quarter of the load instructions of a row-per-thread map)
+  constexpr int kGPre = kMergePre / 2;
+  const int g_items = G * 2 * N / 4;                 // 2N is a multiple of 4
+  const int g_item = tid >> 1, g_half = tid & 1;
+  float4 g_pre[kGPre];
+  if (has_coef && g_item < g_items) {
+    const int g = g_item / (2 * N / 4), n4 = g_item - g * (2 * N / 4);
+    const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const int idx = tid + k * 1024;
-    if (has_coef && idx < G * 2 * N) {
-      const int g = idx / (2 * N), n = idx - g * 2 * N;
-      prefetch_strided(g_pre[k], md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N, n_mid_split);
-    }
+    for (int u = 0; u < kGPre; ++u) g_pre[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * u, n_mid_split - 1) * 2 * N);
   }
   // V coefficients: rows part, part + parts, ... of dim c_lo + j
   const int j = tid & (cwp - 1), part = tid / cwp;
@@ -593,18 +596,35 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   if (n_mid_split > 0) {
     if (cn > 0) {
       // g summed over the splits
-#pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        const int idx = tid + k * 1024;
-        if (idx < G * 2 * N) {
-          const int g = idx / (2 * N), n = idx - g * 2 * N;
-          s_g[idx] = weighted_sum_pre(g_pre[k], md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N,
-                                      s_w + g * n_all + n_il_split, n_mid_split);
+      auto fold1 = [&](const float4& v, int sp, const float* wg, float4& a) {
+        if (sp < n_mid_split) {
+          const float wt = wg[sp];
+          a.x = fmaf(wt, v.x, a.x); a.y = fmaf(wt, v.y, a.y);
+          a.z = fmaf(wt, v.z, a.z); a.w = fmaf(wt, v.w, a.w);
         }
-      }
-      for (int idx = tid + 2048; idx < G * 2 * N; idx += 1024) {
-        const int g = idx / (2 * N), n = idx - g * 2 * N;
-        s_g[idx] = weighted_sum(md_g + (r0 + g) * n_mid_split * 2 * N + n, 2 * N, s_w + g * n_all + n_il_split, n_mid_split);
+      };
+      for (int item = g_item; item < g_items; item += 512) {   // same trip count for both threads of a pair
+        const int g = item / (2 * N / 4), n4 = item - g * (2 * N / 4);
+        const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
+        const float* wg = s_w + g * n_all + n_il_split;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        int u0 = 0;
+        if (item == g_item) {   // the prefetched head
+#pragma unroll
+          for (int u = 0; u < kGPre; ++u) fold1(g_pre[u], g_half + 2 * u, wg, a);
+          u0 = kGPre;
+        }
+        for (; g_half + 2 * u0 < n_mid_split; u0 += 4) {
+          float4 v[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            v[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * (u0 + u), n_mid_split - 1) * 2 * N);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) fold1(v[u], g_half + 2 * (u0 + u), wg, a);
+        }
+        a.x += fa_dpp<FA_DPP_XOR1>(a.x); a.y += fa_dpp<FA_DPP_XOR1>(a.y);
+        a.z += fa_dpp<FA_DPP_XOR1>(a.z); a.w += fa_dpp<FA_DPP_XOR1>(a.w);
+        if (g_half == 0) *(float4*)(s_g + g * 2 * N + 4 * n4) = a;
       }
       __syncthreads();
       // g . V_coef
