@@ -5,7 +5,9 @@ hipcc and links ``fourierattention_amd/libfourier_attn_hip.so`` in-tree.
 """
 from __future__ import annotations
 
+import glob
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -28,12 +30,77 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def audit_async_lds_reads(asm_text: str):
+    """Find instructions that touch the destination of an inline-asm LDS read before it has been waited for.
+
+    The matrix-core kernels issue ``ds_read`` from inline asm and tie the ``s_waitcnt`` to the result later, so
+    that the compiler does not wait for the asynchronous page loads at every read.  Until that wait the
+    registers do not hold the data, but the compiler believes they do and is free to copy them (it does when a
+    read under a condition is merged with the other path).  The copy reads stale registers and nothing fails at
+    build time, so every build checks the generated assembly: between such a read and the ``lgkmcnt`` wait
+    that covers it, no instruction outside an asm block may name its registers.  Returns the violations."""
+    def regs(text):
+        out = set()
+        for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
+            out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+        for m in re.finditer(r"\bv(\d+)\b", text):
+            out.add(int(m.group(1)))
+        return out
+
+    kernel, in_asm, pending, found = None, False, [], []   # pending: (registers, line) in issue order
+    for no, line in enumerate(asm_text.split("\n"), 1):
+        mk = re.match(r"^(_Z\S+):", line)
+        if mk:
+            kernel, pending = mk.group(1), []
+        s = line.strip()
+        if "ASMSTART" in s:
+            in_asm = True
+            continue
+        if "ASMEND" in s:
+            in_asm = False
+            continue
+        if not s or s[0] in ";.":
+            continue
+        m = re.match(r"(\S+)\s*(.*)", s.split(";")[0])
+        if not m:
+            continue
+        op, args = m.group(1), m.group(2)
+        if op == "s_waitcnt":
+            mm = re.search(r"lgkmcnt\((\d+)\)", args)
+            if mm:   # LDS operations complete in issue order: all but the last n are done
+                n = int(mm.group(1))
+                pending = pending[len(pending) - n:] if n else []
+            continue
+        if in_asm and op.startswith("ds_read"):
+            pending.append((regs(args.split(",")[0]), no))
+            continue
+        if op.startswith("ds_") or op.startswith("s_load") or op.startswith("s_buffer_load"):
+            pending.append((set(), no))   # shares the counter
+        if in_asm:
+            continue
+        used = regs(args)
+        for dst, at in pending:
+            if dst & used:
+                found.append(f"{kernel}: line {no} `{s[:80]}` touches v{sorted(dst & used)} of the read at line {at}")
+                break
+    return found
+
+
 def _compile(src: str, obj_dir: str, extra) -> str:
-    obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, "-c", src, "-o", obj]
+    base = os.path.basename(src)[:-4]
+    obj = os.path.join(obj_dir, base + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, "-save-temps=obj", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
+    found = []
+    for tmp in glob.glob(os.path.join(obj_dir, base + "-*")) + glob.glob(os.path.join(obj_dir, base + ".hip-*")):
+        if tmp.endswith("gfx950.s"):
+            with open(tmp) as f:
+                found = audit_async_lds_reads(f.read())
+        os.remove(tmp)   # intermediate files of the compile
+    if found:
+        raise RuntimeError(f"{src}: results of asynchronous LDS reads are used before their wait:\n" + "\n".join(found))
     return obj
 
 

@@ -902,13 +902,13 @@ struct Plan {
   Path path;
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
   int n_merge_chunks;
-  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, total;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, off_scores, total;
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
   const int G = Hq / Hkv;
   return layout == FA_MID_PAGED && (dtype == FA_BF16 || dtype == FA_FP16) && G <= 16 && D <= 128 &&
-         (N == 128 || N == 256 || N == 512);
+         (N == 128 || N == 256 || N == 512 || N == 1024);
 }
 
 Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma, bool il_fast) {
@@ -920,7 +920,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     p.nbpg = 16 / G < 4 ? 16 / G : 4;       // one wave streams one batch element of the group
     if (p.nbpg > B) p.nbpg = B;
     p.n_groups = fa_cdiv(B, p.nbpg);
-    p.ks = N / 64;
+    p.ks = N / (16 * fa_mfma::table_slices(N));
     const int tiles = fa_cdiv(L_m, 32);
     int want = fa_cdiv(device_cu_count(), (int64_t)Hkv * p.n_groups);
     if (want < 1) want = 1;
@@ -955,6 +955,8 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
   p.n_merge_chunks = 1;
   p.off_cpart = take(256);
+  // two-pass mid rows (eight frequency slices): the scores of every page travel through memory
+  p.off_scores = take(mfma && fa_mfma::table_slices(N) > 4 ? (size_t)p.n_groups * Hkv * fa_cdiv(L_m, 32) * 512 * 4 : 0);
   p.total = o;
   return p;
 }
@@ -972,12 +974,25 @@ bool il_fast_ok(const fa_decode_args& a) {
 
 void launch_tables(void* tables, int N, int T, hipStream_t st) {
   using namespace fa_mfma;
-  const int KS = N / 64;
+  const int NSL = table_slices(N), KS = N / (16 * NSL);
   half8* tabE = (half8*)tables;
-  half8* tabET = tabE + kFreqWaves * 2 * KS * 64;
-  float2v* rot = (float2v*)(tabET + 2 * kFreqWaves * 2 * KS * 64);
-  const int total = 3 * kFreqWaves * 2 * KS * 64 + 2 * N;
-  decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N);
+  half8* tabET = tabE + NSL * 2 * KS * 64;
+  float2v* rot = (float2v*)(tabET + 2 * NSL * 2 * KS * 64);
+  const int total = 3 * NSL * 2 * KS * 64 + 2 * N;
+  decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N, NSL);
+}
+
+// eight frequency slices: a score pass, then a value pass over the same pages
+template <typename E>
+void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
+  dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
+  if (wide) {
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 2><<<grid, 512, 0, st>>>(mp);
+  } else {
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 1><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 2><<<grid, 512, 0, st>>>(mp);
+  }
 }
 
 template <typename E, int KS>
@@ -1040,15 +1055,18 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.kn_list = a.kn_list; mp.kn_h = a.kn_h_list; mp.kpad_h = a.k_pad_h_list;
         mp.vn_h = a.vn_h_list; mp.vpad_h = a.v_pad_h_list;
         mp.tabE = (const half8*)tables;
-        mp.tabET = mp.tabE + kFreqWaves * 2 * KS * 64;
-        mp.rot = (const float2v*)(mp.tabET + 2 * kFreqWaves * 2 * KS * 64);
+        const int NSL = table_slices(a.N);
+        mp.tabET = mp.tabE + NSL * 2 * KS * 64;
+        mp.rot = (const float2v*)(mp.tabET + 2 * NSL * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
+        mp.scores = (float*)(ws + p.off_scores);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
         mp.sm_log2e = sm_log2e;
         if (ev) hipEventRecord(ev[1], st);
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
-        switch (KS) {
+        if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, st);
+        else switch (KS) {
           case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, st); break;
           case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, st); break;
           default: launch_mid_mfma_ks<E, 8>(mp, p, wide, st); break;

@@ -33,17 +33,17 @@ __device__ __forceinline__ int freq_of(int rt, int lg, int fi2) { return rt * 8 
 constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one slice per SIMD)
 
 // ---------------------------------------------------------------------------
-// constant operand tables (depend on T and N only); KS = N / 64 ksteps per frequency slice
-//   tabE  [4 slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM
-//   tabET [2 pages][4 slices][2*KS row tiles][64 lanes] x half8 : A operand of the g GEMM for the tokens of
+// constant operand tables (depend on T and N only); KS = N / (16 * slices) ksteps per frequency slice
+//   tabE  [slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM
+//   tabET [2 pages][slices][2*KS row tiles][64 lanes] x half8 : A operand of the g GEMM for the tokens of
 //         a page (0) and for the tokens of the page after it seen from the same page start (1)
 //   rot   [2][N] float2 : (cos, sin)(2 pi f 32 / T) and (cos, sin)(2 pi f 64 / T), the frame rotation of one
 //         page step and of two
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ tabE, half8* __restrict__ tabET,
-                                                            float2v* __restrict__ rot, int KS, int T, int N) {
+                                                            float2v* __restrict__ rot, int KS, int T, int N, int NSL) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  const int nE = kFreqWaves * 2 * KS * 64, nET = 2 * kFreqWaves * 2 * KS * 64;
+  const int nE = NSL * 2 * KS * 64, nET = 2 * NSL * 2 * KS * 64;
   if (idx < nE) {
     const int lane = idx & 63, s = (idx >> 6) % KS, rb = ((idx >> 6) / KS) & 1, w = (idx >> 6) / (2 * KS);
     const int lg = lane >> 4, lc = lane & 15;
@@ -60,8 +60,8 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
     tabE[idx] = out;
   } else if (idx < nE + nET) {
     const int k = idx - nE;
-    const int lane = k & 63, rt = (k >> 6) % (2 * KS), w = ((k >> 6) / (2 * KS)) % kFreqWaves;
-    const int page = (k >> 6) / (2 * KS * kFreqWaves);
+    const int lane = k & 63, rt = (k >> 6) % (2 * KS), w = ((k >> 6) / (2 * KS)) % NSL;
+    const int page = (k >> 6) / (2 * KS * NSL);
     const int lg = lane >> 4, rho = lane & 15;
     const int f = w * 16 * KS + freq_of(rt, rho >> 2, (rho & 3) >> 1);
     const int cs = rho & 1;
@@ -81,9 +81,12 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
   }
 }
 
+// frequency slices: four (one per SIMD, score and value wave of a slice side by side) up to N = 512; eight for
+// N = 1024, whose per-wave state only fits when a pass runs one role on all eight waves
+static inline int table_slices(int N) { return N > 512 ? 8 : 4; }
 static inline size_t tables_bytes(int N) {
-  const int KS = N / 64;
-  return (size_t)(3 * kFreqWaves * 2 * KS * 64) * 16 + (size_t)2 * N * 8;
+  const int NSL = table_slices(N), KS = N / (16 * NSL);
+  return (size_t)(3 * NSL * 2 * KS * 64) * 16 + (size_t)2 * N * 8;
 }
 
 
@@ -112,6 +115,18 @@ __device__ __forceinline__ void rot_pair(float c, float s, float& x, float& y) {
   const float sy = s * y, sx = s * x;
   x = __builtin_fmaf(c, x, sy);
   y = __builtin_fmaf(c, y, -sx);
+}
+// The same with the results in the registers of the operands.  State that lives across loop iterations in plain
+// registers (not in accumulators of the matrix unit) is otherwise left wherever the last instruction of a rotation
+// put it, and every iteration ends with one move per value to bring the registers back in order.
+__device__ __forceinline__ void rot_pair_in_place(float c, float s, float& x, float& y) {
+  float sy, sx;
+  asm("v_mul_f32 %0, %4, %3\n\t"
+      "v_mul_f32 %1, %4, %2\n\t"
+      "v_fma_f32 %2, %5, %2, %0\n\t"
+      "v_fma_f32 %3, %5, %3, -%1"
+      : "=&v"(sy), "=&v"(sx), "+v"(x), "+v"(y)
+      : "v"(s), "v"(c));
 }
 // pair(rt, f2, c, s) applies one rotation and returns one of its results; pin(b) passes the results of
 // batch b (row tiles 4b .. 4b+3) through an empty asm volatile, which keeps their arithmetic above the
@@ -180,6 +195,7 @@ struct MidParams {
   float* pd;
   float* pg;
   float* pon;
+  float* scores;   // two-pass mode: [groups][Hkv][pages][16 columns][32 tokens] fp32
   int B, Hq, Hkv, D, G, nbpg, N, L_m, T, n_split, tiles_per_split;
   float sm_log2e;
 };
@@ -194,25 +210,34 @@ struct MidParams {
 // (dp_k / 32).  VMAX: V dim groups of 16 (dp_v / 16).
 // NST: page stages per wave in LDS; the K / V pages travel HBM -> LDS with global_load_lds (no registers
 // held while in flight), NST - 1 pages ahead of their use.
-template <typename E, int KS, int KMAX, int VMAX, int NST>
+// MODE 0: the fused pipeline above (N <= 512).  For N = 1024 a wave cannot hold twice the state, so the work is cut
+// into two passes over the same pages, each running ONE role on all eight waves (eight frequency slices):
+// MODE 1, scores: eight partials per page meet in LDS, their sum (the complete score of the page) goes to
+//         memory (2 KiB per page and workgroup, against 16 KiB of K/V);
+// MODE 2, values: every wave reads the page's scores back, runs the softmax and keeps its slice of the g
+//         history; waves 0-3 stream V.  No exchange between the waves at all.
+template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
+  constexpr int NSL = MODE == 0 ? kFreqWaves : 2 * kFreqWaves;   // frequency slices
   using M = Mma<E>;
   using vec8 = typename M::vec8;
   constexpr int kFragsMax = (2 * KMAX > VMAX ? 2 * KMAX : VMAX);   // fragments (1 KiB) of one page of one wave
-  __shared__ __attribute__((aligned(16))) unsigned char s_stage[8][NST][kFragsMax * 1024];
-  __shared__ float s_part[2][kFreqWaves][16 * kPart];
-  __shared__ float4v s_rot[kFreqWaves * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
+  static_assert(MODE == 0 || NST == 2, "the passes wait for every outstanding load at the top of a page");
+  // in the two-pass modes only waves 0-3 stream pages
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[MODE == 0 ? 8 : 4][NST][kFragsMax * 1024];
+  __shared__ float s_part[MODE == 2 ? 1 : 2][MODE == 2 ? 1 : NSL][16 * kPart];
+  __shared__ float4v s_rot[NSL * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
   // Narrow pages leave LDS for a second g operand: the value waves then accumulate two pages per frame (the second
   // through E^T of the token offsets 32..63, read from LDS) and rotate their history every other page only.
-  constexpr bool TWO = kFragsMax <= 4;
+  constexpr bool TWO = MODE == 0 && kFragsMax <= 4;
   __shared__ float4v s_rot2[TWO ? kFreqWaves * 2 * KS * 4 : 1];   // the same for a step of two pages
   __shared__ uint4v s_et1[TWO ? kFreqWaves * 2 * KS * 64 : 1];    // [slice][row tile][lane]
 
   const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
-  const bool score_wave = w < kFreqWaves;
-  const int sl = w & 3;  // frequency slice and batch element of the group
+  const bool score_wave = MODE == 0 ? w < kFreqWaves : MODE == 1;
+  const int sl = MODE == 0 ? (w & 3) : w;  // frequency slice; below 4 also the batch element of the group
   const int split = blockIdx.x, h = blockIdx.y, grp = blockIdx.z;
   const int G = p.G, N = p.N;
   const int b0 = grp * p.nbpg;
@@ -222,15 +247,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int bb_r = lc / G, g_r = lc - bb_r * G;
   const int64_t qrow = valid_r ? ((int64_t)(b0 + bb_r) * p.Hq + h * G + g_r) : 0;
   const int fbase = sl * 16 * KS;
-  const bool has_mn = sl < nb;
-  const int my_b = b0 + (sl < nb ? sl : 0);
+  const bool has_mn = sl < nb && sl < kFreqWaves;
+  const int my_b = b0 + (has_mn ? sl : 0);
+  const int stw = has_mn ? w & 3 : 0;   // page stage of this wave
 
   const int n_tiles = (p.L_m + 31) >> 5;
   const int t_beg = split * p.tiles_per_split;
   const int t_end = min(n_tiles, t_beg + p.tiles_per_split);
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
 
-  if (score_wave && lc == 0) {
+  if ((MODE != 0 || score_wave) && lc == 0) {
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) {
       const float2v a = p.rot[fbase + freq_of(rt, lg, 0)];
@@ -256,7 +282,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // a page moves the fragments the head really has (two stages: the page wait below is always "all landed")
     auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* kp = kbase + (int64_t)t * dpk * 32;
-      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
+      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
@@ -351,24 +377,40 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
     __syncthreads();   // the rotation constants in LDS are complete
     const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
+    // score pass: the complete scores of page pg of the split (sum of the eight partials; thread = (column,
+    // token)) go to memory.  Called one page late, behind that page's barrier.
+    auto flush_scores = [&](int pg) {
+      if constexpr (MODE == 1) {
+        constexpr int kW = 16 * kPart * 4;   // bytes between the partials of two waves
+        const float sum = lds_sum8_b32<kW>(lds_addr_of(&s_part[pg & 1][0][(tid >> 5) * kPart + (tid & 31)]));
+        p.scores[((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pg) * 512 + tid] = sum;
+      }
+    };
 
     for (int it = 0; it <= n_it; ++it) {
       if (it < n_it) {
         const int t = t_beg + it;
         uint4v kraw[4];   // two ksteps of both token blocks at a time
-        const unsigned kst = lds_addr_of(&s_stage[w][it % NST][0]) + lane * 16;
+        const unsigned kst = lds_addr_of(&s_stage[MODE == 0 ? w : stw][it % NST][0]) + lane * 16;
         uint4v rc[2][4];
         if (has_k) {
           // pages t+1 .. t+NST-2 may still be in flight; page t has landed: start its LDS reads now
           if (it + NST - 2 < n_it) wait_vmcnt<(NST - 2) * 2 * KMAX>();
           else wait_vmcnt<0>();
           if (it + NST - 1 < n_it) issue_k(t + NST - 1);   // refills the stage read one page ago
+        }
+        // The results of these reads arrive later (the wait is tied to them further down); until then no
+        // instruction may touch their registers.  A read under a condition makes the compiler merge its result
+        // with the other path, which it may do by copying the registers at once: where that happened the reads
+        // are issued by every wave (a wave without pages reads its idle stage and drops the result).
+        if (MODE != 0 || has_k) {
           // ksteps 0, 1: issued early, consumed after the coefficient-domain product
           kraw[0] = lds_read_b128_async_at<0>(kst);
           kraw[1] = lds_read_b128_async_at<1024>(kst);
           kraw[2] = lds_read_b128_async_at<KMAX * 1024>(kst);
           kraw[3] = lds_read_b128_async_at<(KMAX + 1) * 1024>(kst);
         }
+        if (it > 0) flush_scores(it - 1);   // behind the page wait: the store has a whole page to complete
         rot_issue<0>(rot_lane, rc[0]);
         if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
         float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
@@ -385,7 +427,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         // advance W' by one page step
         rot_apply<2 * KS, 2>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
-          rot_pair(c, sn, Wc[rt][f2], Ws[rt][f2]);
+          rot_pair_in_place(c, sn, Wc[rt][f2], Ws[rt][f2]);
           return Ws[rt][f2];
         }, [&](int b) {
 #pragma unroll
@@ -419,8 +461,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int v = 0; v < 4; ++v) o[v] = accf[rb][v] * colscale + accm[rb][v] * p.sm_log2e + c0col;
           *(float4v*)&s_part[it & 1][sl][lc * kPart + rb * 16 + 4 * lg] = o;
         }
+      } else if (it > 0) {
+        flush_scores(it - 1);
       }
-      barrier_lds_only();
+      if (MODE == 0 || it < n_it) barrier_lds_only();
     }
   } else {
     // =============================== value waves ===============================
@@ -430,7 +474,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool has_v = has_mn && ndg > 0;
     auto issue_v = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* vp = vbase + (int64_t)t * dpv * 32;
-      unsigned char* st = &s_stage[w][(t - t_beg) % NST][0];
+      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
 #pragma unroll
       for (int f = 0; f < VMAX; ++f)
         if (f < ndg) load_frag_to_lds<2>(vp + f * 512 + lane * 8, st + f * 1024);
@@ -461,6 +505,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();   // the rotation constants in LDS are complete
     const unsigned rot_lane = lds_addr_of(TWO ? &s_rot2[(sl * 2 * KS) * 4 + lg] : &s_rot[(sl * 2 * KS) * 4 + lg]);
     const unsigned et1_lane = lds_addr_of(&s_et1[TWO ? (sl * 2 * KS) * 64 + lane : 0]);
+    // value pass: the scores of a page (column lc, tokens 8*lg .. 8*lg+7) are fetched one page ahead
+    float4v sc_next[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
+    const float* sc_src = nullptr;
+    if constexpr (MODE == 2) {
+      sc_src = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg) * 512 + lc * 32 + 8 * lg;
+      if (n_it > 0) {
+        sc_next[0] = *(const float4v*)sc_src;
+        sc_next[1] = *(const float4v*)(sc_src + 4);
+      }
+    }
 
     // one page of the value stage (page it - 1 of the split)
     auto value_page = [&](int it, auto first_tag) {
@@ -473,10 +527,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           rot_issue<0>(rot_lane, rc[0]);
           if (RCB == 2 && 2 * KS > 4) rot_issue<1>(rot_lane, rc[RCB - 1]);
         }
+        float sc[8];
+        if constexpr (MODE == 2) {
+          // taken before the next page is requested: a wait placed here by the compiler then covers loads that
+          // have had a whole page to land, and nothing that was issued a moment ago
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            sc[e] = sc_next[e >> 2][e & 3];
+            asm volatile("" : "+v"(sc[e]));
+          }
+        }
         if (has_v) {
           if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
           else wait_vmcnt<0>();
           if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
+        }
+        if constexpr (MODE == 2) {
+          const float* nx = sc_src + (int64_t)min(pg + 1, n_it - 1) * 512;   // clamped: the load is unconditional
+          sc_next[0] = *(const float4v*)nx;
+          sc_next[1] = *(const float4v*)(nx + 4);
         }
         // the g history moves into the frame of this page (of this pair of pages)
         if constexpr (first_of_frame)
@@ -490,8 +559,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           asm volatile("" : "+v"(hacc[4 * b]), "+v"(hacc[4 * b + 1]), "+v"(hacc[4 * b + 2]), "+v"(hacc[4 * b + 3]));
         });
         // scores of the page in B-operand layout (column lc, tokens 8*lg + e): four partials to sum
-        float sc[8];
-        {
+        if constexpr (MODE == 0) {
           uint4v part[kFreqWaves][2];
           const unsigned pst = lds_addr_of(&s_part[buf][0][lc * kPart + 8 * lg]);
           constexpr int kW = 16 * kPart * 4;   // bytes between the partials of two score waves
@@ -517,7 +585,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           }
         }
         uint4v vraw[4];   // four dim groups at a time
-        const unsigned vst = lds_addr_of(&s_stage[w][pg % NST][0]) + lane * 16;
+        const unsigned vst = lds_addr_of(&s_stage[MODE == 0 ? w : stw][pg % NST][0]) + lane * 16;
         if (has_v) {
           vraw[0] = lds_read_b128_async_at<0>(vst);
           vraw[1] = lds_read_b128_async_at<1024>(vst);
@@ -577,8 +645,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           }
         }
     };
-    barrier_lds_only();   // iteration 0: the score waves are one page ahead
-    if constexpr (TWO) {
+    if constexpr (MODE == 2) {
+      for (int it = 1; it <= n_it; ++it) value_page(it, std::true_type{});
+    } else if constexpr (TWO) {
+      barrier_lds_only();   // iteration 0: the score waves are one page ahead
       for (int it = 1; it <= n_it; it += 2) {
         value_page(it, std::true_type{});
         barrier_lds_only();
@@ -588,6 +658,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
       }
     } else {
+      barrier_lds_only();   // iteration 0: the score waves are one page ahead
       for (int it = 1; it <= n_it; ++it) {
         value_page(it, std::true_type{});
         barrier_lds_only();

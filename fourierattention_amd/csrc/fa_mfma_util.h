@@ -72,6 +72,20 @@ template <int AFTER>
 __device__ __forceinline__ void lds_wait_for4(uint4v (&r)[4]) {
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(AFTER) : "memory");
 }
+// sum of eight floats STEP bytes apart, read like the accesses above and complete on return
+template <int STEP>
+__device__ __forceinline__ float lds_sum8_b32(unsigned lds_addr) {
+  static_assert(STEP % 4 == 0 && 7 * STEP < 65536, "immediate offsets of ds_read_b32");
+  float v0, v1, v2, v3, v4, v5, v6, v7;
+  asm volatile(
+      "ds_read_b32 %0, %8\n\tds_read_b32 %1, %8 offset:%9\n\tds_read_b32 %2, %8 offset:%10\n\t"
+      "ds_read_b32 %3, %8 offset:%11\n\tds_read_b32 %4, %8 offset:%12\n\tds_read_b32 %5, %8 offset:%13\n\t"
+      "ds_read_b32 %6, %8 offset:%14\n\tds_read_b32 %7, %8 offset:%15\n\ts_waitcnt lgkmcnt(0)"
+      : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4), "=&v"(v5), "=&v"(v6), "=&v"(v7)
+      : "v"(lds_addr), "n"(STEP), "n"(2 * STEP), "n"(3 * STEP), "n"(4 * STEP), "n"(5 * STEP), "n"(6 * STEP), "n"(7 * STEP)
+      : "memory");
+  return ((v0 + v1) + (v2 + v3)) + ((v4 + v5) + (v6 + v7));
+}
 // workgroup barrier that orders LDS traffic only (global loads stay in flight)
 __device__ __forceinline__ void barrier_lds_only() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 

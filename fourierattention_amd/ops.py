@@ -245,7 +245,7 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
     does not cover ``N`` (the call then takes the generic kernels)."""
     lib = _lib.load()
     nbytes = lib.fa_decode_tables_bytes(int(n_f))
-    if nbytes == 0 or n_f not in (128, 256, 512):
+    if nbytes == 0 or n_f not in (128, 256, 512, 1024):
         return None
     buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
     check(lib.fa_decode_tables_build(buf.data_ptr(), nbytes, int(n_f), int(period), _stream(torch.device(device))))

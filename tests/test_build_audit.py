@@ -1,0 +1,59 @@
+"""The build's check of the generated assembly: an inline-asm LDS read whose registers are touched before the
+wait that covers it must be reported (the compiler may copy such registers when a conditional read is merged
+with the other path; nothing else would notice)."""
+from fourierattention_amd.build import audit_async_lds_reads
+
+GOOD = """
+_Zkernel_a:
+\t;;#ASMSTART
+\tds_read_b128 v[10:13], v1 offset:0
+\t;;#ASMEND
+\tv_add_f32_e32 v20, v21, v22
+\t;;#ASMSTART
+\ts_waitcnt lgkmcnt(0)
+\t;;#ASMEND
+\tv_mov_b32_e32 v30, v12
+"""
+
+# the copy the compiler makes when the read sits in one arm of a branch
+BAD_COPY = """
+_Zkernel_b:
+\t;;#ASMSTART
+\tds_read_b128 v[82:85], v1 offset:0xc00
+\t;;#ASMEND
+\ts_nop 0
+\tv_mov_b32_e32 v93, v85
+\t;;#ASMSTART
+\ts_waitcnt lgkmcnt(0)
+\t;;#ASMEND
+"""
+
+# a counted wait leaves the youngest reads in flight
+PARTIAL = """
+_Zkernel_c:
+\t;;#ASMSTART
+\tds_read_b128 v[10:13], v1
+\t;;#ASMEND
+\t;;#ASMSTART
+\tds_read_b128 v[14:17], v1 offset:64
+\t;;#ASMEND
+\t;;#ASMSTART
+\ts_waitcnt lgkmcnt(1)
+\t;;#ASMEND
+\tv_mul_f32_e32 v40, v10, v11
+\tv_mul_f32_e32 v41, v14, v15
+"""
+
+
+def test_clean_sequence_passes():
+    assert audit_async_lds_reads(GOOD) == []
+
+
+def test_copy_before_wait_is_reported():
+    found = audit_async_lds_reads(BAD_COPY)
+    assert len(found) == 1 and "_Zkernel_b" in found[0] and "v_mov_b32_e32 v93, v85" in found[0]
+
+
+def test_counted_wait_releases_only_the_older_reads():
+    found = audit_async_lds_reads(PARTIAL)
+    assert len(found) == 1 and "v41" in found[0] and "v40" not in found[0]

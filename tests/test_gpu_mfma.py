@@ -42,6 +42,9 @@ MFMA_CASES = [
     (torch.float16, 3, 4, 4, 64, 2, 16, 256, 420, 2, [10, 30, 64, 1], [3, 64, 33, 17]),  # MHA, head_dim 64, fp16
     (torch.bfloat16, 2, 32, 8, 128, 4, 64, 1024, 2200, 2, [64] * 8, [64] * 8),       # the benchmark's geometry, short
     (torch.bfloat16, 3, 16, 2, 128, 4, 200, 256, 900, 3, [64, 40], [64, 96]),        # 8:1 grouping, window of several tiles
+    # 1024 frequencies: the mid rows run as a score pass and a value pass
+    (torch.bfloat16, 5, 16, 4, 128, 4, 32, 2048, 4500, 2, [64] * 4, [64] * 4),
+    (torch.float16, 2, 8, 2, 128, 4, 32, 2048, 4200, 2, [0, 128], [120, 7]),
 ]
 
 
