@@ -25,6 +25,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 WORKLOADS = {
     # name: B, ctx, Hq, Hkv, D, I, W, M, compressed dims per head, max_new_tokens
     "config3_decode_attn_8b_32k": dict(B=8, ctx=32768, Hq=32, Hkv=8, D=128, I=4, W=1024, M=1024, cper=64, max_new=128),
+    # the per-layer attention of BASELINE configs 4 and 5 (their end-to-end runs are under --e2e)
+    "config4_decode_attn_8b_64k": dict(B=16, ctx=65536, Hq=32, Hkv=8, D=128, I=4, W=1024, M=1024, cper=64, max_new=128),
+    "config5_decode_attn_3b_128k": dict(B=4, ctx=131072, Hq=24, Hkv=8, D=128, I=4, W=1024, M=2048, cper=64, max_new=512),
     "config1_cpu_geometry_3b_2k": dict(B=1, ctx=2048, Hq=24, Hkv=8, D=128, I=4, W=512, M=256, cper=64, max_new=64),
 }
 
@@ -159,6 +162,68 @@ def compress_bench(device, reps=20):
             "operand_dtype": "f16 (basis and data), fp32 accumulation"}
 
 
+E2E = {
+    # BASELINE configs 4 and 5: a random-init decoder with the Fourier cache on every layer
+    "config4_e2e_8b_64k": dict(preset="llama-3.1-8b", B=16, prompt=65536, new=128, I=4, W=1024, M=1024, cper=64),
+    "config5_e2e_3b_128k": dict(preset="llama-3.2-3b", B=4, prompt=131072, new=512, I=4, W=1024, M=2048, cper=64),
+}
+
+
+def e2e_bench(name, device, steps=None, warmup=3):
+    """Greedy decode of a random-init LLaMA with the Fourier cache on every layer.  The prompt's K/V are
+    synthetic (random rows pushed through the cache's own prefill, layer by layer): the quadratic prompt pass
+    of a random model is not what this figure is about.  Every timed step is a full model step: embedding,
+    all layers (projections, rotary embedding, cache update, Fourier attention, MLP), final norm, LM head,
+    argmax."""
+    from fourierattention_amd import DynamicCache, ExtraConfig, masks
+    from fourierattention_amd.llama import PRESETS, LlamaConfig, random_init, synthetic_prefill
+    e = E2E[name]
+    cfg = LlamaConfig(**PRESETS[e["preset"]])
+    steps = steps or e["new"]
+    m = masks.synthetic_masks(cfg.num_hidden_layers, cfg.num_key_value_heads, cfg.head_dim, e["cper"], seed=0)
+    ec = ExtraConfig(numinittokens=e["I"], maxlocallen=e["W"], maxmidstates=e["M"], non_critical_dims=m,
+                     non_critical_dims_path=None, max_position_embeddings=1 << 20,
+                     num_key_value_heads=cfg.num_key_value_heads, max_new_tokens=e["new"] + warmup + 8, model_type="llama")
+    model = random_init(cfg, torch.bfloat16, device, seed=0)
+    cache = DynamicCache(ec, device=device)
+    t0 = time.perf_counter()
+    synthetic_prefill(cache, cfg, e["B"], e["prompt"], torch.bfloat16, device, seed=0)
+    torch.cuda.synchronize()
+    fill_s = time.perf_counter() - t0
+    g = torch.Generator(device=device).manual_seed(1)
+    ids = torch.randint(0, cfg.vocab_size, (e["B"], 1), generator=g, device=device)
+    with torch.no_grad():
+        for _ in range(warmup):
+            ids = model(input_ids=ids, past_key_values=cache, num_logits_to_keep=1).logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ids = model(input_ids=ids, past_key_values=cache, num_logits_to_keep=1).logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    assert cache.get_seq_length() == e["prompt"] + warmup + steps
+    hd = cfg.num_key_value_heads * cfg.head_dim
+    held = 0
+    for layer in cache._layers:
+        for t in (layer.k, layer.v):
+            held += t.il.numel() * t.il.element_size() + t.coef.numel() * 4 + t.mid.data.numel() * t.mid.data.element_size()
+    ctx = e["prompt"] + warmup + steps
+    full = 2 * ctx * hd * 2 * cfg.num_hidden_layers * e["B"]
+    L = ctx - e["I"] - e["W"]
+    ck = e["cper"] * cfg.num_key_value_heads
+    used = (2 * (e["I"] + e["W"]) * hd * 2 + 2 * L * (hd - ck) * 2 + 2 * e["M"] * ck * 4) * cfg.num_hidden_layers * e["B"]
+    return {"metric": "end-to-end greedy decode tokens/s, random-init model, Fourier cache on every layer",
+            "value": round(e["B"] * steps / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(dt / steps * 1e3, 3), "higher_is_better": True, "dtype": "bf16",
+            "data": "synthetic (random weights, random prompt K/V through the cache's prefill)",
+            "config": {"workload": name, "model": e["preset"], "batch": e["B"], "prompt": e["prompt"],
+                       "new_tokens": steps, "sink": e["I"], "window": e["W"], "coeff_rows": e["M"],
+                       "compressed_dims_per_head": e["cper"], "T_x": cache.period_reconstruct},
+            "kv_cache_bytes": {"full_bf16": full, "fourier_in_use": used, "fourier_allocated": held,
+                               "reduction_in_use": round(full / used, 3)},
+            "synthetic_prefill_s": round(fill_s, 2)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -167,6 +232,9 @@ def main():
     ap.add_argument("--workload", default="config3_decode_attn_8b_32k", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
+    ap.add_argument("--e2e", choices=list(E2E), default=None,
+                    help="run the end-to-end decode of a random-init model instead (its own JSON line); --steps caps the "
+                         "number of timed tokens per sequence")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run ten 1 GiB device-to-device copies (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -181,6 +249,10 @@ def main():
     torch.cuda.set_device(device)
     from fourierattention_amd import _lib
     _lib.load()
+    if args.e2e:
+        explicit = any(x == "--steps" or x.startswith("--steps=") for x in sys.argv[1:])
+        print(json.dumps(e2e_bench(args.e2e, device, steps=args.steps if explicit else None)))
+        return
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)

@@ -1,0 +1,205 @@
+"""Minimal LLaMA decoder around the Fourier cache: what runs either side of the attention path in one
+decode step (fourier_attn_triton/modeling_llama_fourier.py:78-98 RMSNorm, 100-190 rotary embedding,
+246-283 SwiGLU MLP, 677-754 decoder layer, 912-1033 model forward, 1090-1200 LM head) and the greedy loop
+of models/fourier.py:155-203.
+
+Stock math only: the projections and the MLP are ``torch`` GEMMs, the attention module is
+``fourierattention_amd.attention.LlamaSdpaAttention``.  Weights are random (no checkpoint can be fetched
+here); ``synthetic_prefill`` fills the cache of every layer with a random prompt of the requested length
+through the cache's own prefill branch, so a decode benchmark at a long context does not have to run the
+quadratic prompt pass of a random model first.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from types import SimpleNamespace
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import synth
+from .attention import LlamaSdpaAttention
+from .cache import DynamicCache
+
+
+@dataclass
+class LlamaConfig:
+    hidden_size: int = 4096
+    intermediate_size: int = 14336
+    num_hidden_layers: int = 32
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    head_dim: Optional[int] = None
+    vocab_size: int = 128256
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    attention_bias: bool = False
+    mlp_bias: bool = False
+    tie_word_embeddings: bool = False
+
+    def __post_init__(self):
+        if self.head_dim is None:
+            self.head_dim = self.hidden_size // self.num_attention_heads
+
+
+PRESETS = {
+    "llama-3.1-8b": dict(hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+                         num_key_value_heads=8, head_dim=128),
+    "llama-3.2-3b": dict(hidden_size=3072, intermediate_size=8192, num_hidden_layers=28, num_attention_heads=24,
+                         num_key_value_heads=8, head_dim=128, tie_word_embeddings=True),
+}
+
+
+class LlamaRMSNorm(nn.Module):
+    """Variance in fp32, scale in the input dtype (modeling_llama_fourier.py:78-95)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def forward(self, x):
+        dt = x.dtype
+        x = x.float()
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * x.to(dt)
+
+
+class LlamaRotaryEmbedding(nn.Module):
+    """Plain ("default") rotary tables: ``inv_freq = theta^(-2i/D)``, angles in fp32, tables in the
+    activation dtype (modeling_llama_fourier.py:165-187)."""
+
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        d = config.head_dim
+        inv_freq = 1.0 / (config.rope_theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    @torch.no_grad()
+    def forward(self, x, position_ids):
+        freqs = position_ids[:, :, None].float() * self.inv_freq[None, None, :].float().to(position_ids.device)
+        emb = torch.cat((freqs, freqs), dim=-1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
+class LlamaMLP(nn.Module):
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=config.mlp_bias)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=config.mlp_bias)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=config.mlp_bias)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class LlamaDecoderLayer(nn.Module):
+    def __init__(self, config: LlamaConfig, layer_idx: int):
+        super().__init__()
+        self.self_attn = LlamaSdpaAttention(config, layer_idx)
+        self.mlp = LlamaMLP(config)
+        self.input_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, hidden_states, position_embeddings, past_key_value, cache_position=None):
+        h, _, _ = self.self_attn(self.input_layernorm(hidden_states), past_key_value=past_key_value, use_cache=True,
+                                 cache_position=cache_position, position_embeddings=position_embeddings)
+        hidden_states = hidden_states + h
+        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+
+
+class LlamaModel(nn.Module):
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList([LlamaDecoderLayer(config, i) for i in range(config.num_hidden_layers)])
+        self.norm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.rotary_emb = LlamaRotaryEmbedding(config)
+
+    def forward(self, input_ids, past_key_values: DynamicCache, position_ids=None):
+        """A cache object is required (modeling_llama_fourier.py:946-949 would otherwise build one without
+        its configuration and fail); positions continue from ``past_key_values.get_seq_length()``
+        (modeling_llama_fourier.py:959-963)."""
+        if past_key_values is None:
+            raise ValueError("a Fourier DynamicCache must be passed as past_key_values")
+        x = self.embed_tokens(input_ids)
+        seen = past_key_values.get_seq_length()
+        cache_position = torch.arange(seen, seen + x.shape[1], device=x.device)
+        if position_ids is None:
+            position_ids = cache_position.unsqueeze(0)
+        pe = self.rotary_emb(x, position_ids)
+        for layer in self.layers:
+            x = layer(x, pe, past_key_values, cache_position)
+        return self.norm(x)
+
+
+class LlamaForCausalLM(nn.Module):
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.config = config
+        self.model = LlamaModel(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.model.embed_tokens.weight
+
+    def forward(self, input_ids, past_key_values: DynamicCache, use_cache: bool = True, position_ids=None,
+                num_logits_to_keep: int = 0):
+        h = self.model(input_ids, past_key_values, position_ids)
+        if num_logits_to_keep:
+            h = h[:, -num_logits_to_keep:, :]
+        return SimpleNamespace(logits=self.lm_head(h).float(), past_key_values=past_key_values)
+
+
+def random_init(config: LlamaConfig, dtype=torch.bfloat16, device="cuda:0", seed: int = 0, std: float = 0.02):
+    """A model of the given architecture with seeded normal weights (norm scales stay 1)."""
+    with torch.device(device):
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(dtype)
+        try:
+            model = LlamaForCausalLM(config)
+        finally:
+            torch.set_default_dtype(prev)
+    g = torch.Generator(device=device).manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() > 1:
+                p.normal_(0.0, std, generator=g)
+    return model.eval()
+
+
+@torch.no_grad()
+def greedy_generate(model: LlamaForCausalLM, input_ids: torch.Tensor, cache: DynamicCache, max_new_tokens: int,
+                    eos_token_id: Optional[int] = None):
+    """The loop of models/fourier.py:175-190: feed the prompt, then one argmax token per step with the cache
+    threaded through.  Returns ``(B, prompt + generated)`` ids.  With ``eos_token_id`` the loop stops once
+    every sequence of the batch has produced it (the reference handles batch 1 only)."""
+    seq = input_ids
+    done = torch.zeros(input_ids.shape[0], dtype=torch.bool, device=input_ids.device)
+    for _ in range(max_new_tokens):
+        out = model(input_ids=input_ids, past_key_values=cache, use_cache=True, num_logits_to_keep=1)
+        input_ids = torch.argmax(out.logits[:, -1, :], dim=-1, keepdim=True)
+        seq = torch.cat([seq, input_ids], dim=-1)
+        if eos_token_id is not None:
+            done |= input_ids[:, 0] == eos_token_id
+            if bool(done.all()):
+                break
+    return seq
+
+
+@torch.no_grad()
+def synthetic_prefill(cache: DynamicCache, config: LlamaConfig, batch: int, prompt_len: int, dtype=torch.bfloat16,
+                      device="cuda:0", seed: int = 0):
+    """Fill every layer of ``cache`` with a random prompt: K, V ~ N(0, 1), rotary embedding on K, pushed
+    through ``cache.update`` layer by layer in ascending order exactly as a prompt pass does."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    cos, sin = synth.rope_tables(torch.arange(prompt_len), config.head_dim, config.rope_theta)
+    cos, sin = cos.to(device), sin.to(device)
+    shape = (batch, config.num_key_value_heads, prompt_len, config.head_dim)
+    for layer in range(config.num_hidden_layers):
+        k = synth.apply_rope(torch.randn(shape, generator=g, device=device, dtype=torch.float32), cos, sin).to(dtype)
+        v = torch.randn(shape, generator=g, device=device, dtype=torch.float32).to(dtype)
+        cache.update(k, v, layer)
+        del k, v

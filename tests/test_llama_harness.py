@@ -1,0 +1,132 @@
+"""The minimal LLaMA decoder and greedy loop around the cache (fourierattention_amd/llama.py).
+
+CPU: with a window larger than the sequence nothing is compressed, so the cached decode must reproduce a full
+recomputation of the sequence with the same weights (exact attention either way) — this pins positions, the
+prefill / decode dispatch and the threading of the cache through the loop.
+GPU: with a compressed cache, every decode step's logits are compared with the same weights run layer by layer
+on the CPU through the oracle cache and the oracle attention.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.test_gpu_cache import _cfg, _masks
+
+
+def _tiny(layers=2, hidden=64, heads=4, kv=2, hd=16, vocab=97):
+    from fourierattention_amd.llama import LlamaConfig
+    return LlamaConfig(hidden_size=hidden, intermediate_size=2 * hidden, num_hidden_layers=layers, num_attention_heads=heads,
+                       num_key_value_heads=kv, head_dim=hd, vocab_size=vocab)
+
+
+def test_greedy_loop_matches_full_recompute_cpu():
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import greedy_generate, random_init
+    cfg = _tiny()
+    model = random_init(cfg, dtype=torch.float32, device="cpu", seed=3, std=0.3)
+    masks = _masks(cfg.num_hidden_layers, cfg.num_key_value_heads, cfg.head_dim, [8, 8], [8, 8])
+    ec = lambda: _cfg(masks, numinittokens=2, maxlocallen=64, maxmidstates=8, num_key_value_heads=cfg.num_key_value_heads,
+                      max_new_tokens=16, max_position_embeddings=256)
+    g = torch.Generator().manual_seed(0)
+    prompt = torch.randint(0, cfg.vocab_size, (2, 11), generator=g)
+    seq = greedy_generate(model, prompt, DynamicCache(ec(), device="cpu"), max_new_tokens=6)
+    assert seq.shape == (2, 17) and torch.equal(seq[:, :11], prompt)
+    # the same tokens one by one from scratch: a fresh cache and a prompt pass over everything so far
+    cur = prompt
+    for step in range(6):
+        out = model(input_ids=cur, past_key_values=DynamicCache(ec(), device="cpu"), num_logits_to_keep=1)
+        nxt = out.logits[:, -1, :].argmax(-1, keepdim=True)
+        assert torch.equal(nxt, seq[:, 11 + step: 12 + step]), step
+        cur = torch.cat([cur, nxt], dim=-1)
+    # and the logits of a cached step agree with the recomputation
+    cache = DynamicCache(ec(), device="cpu")
+    model(input_ids=seq[:, :14], past_key_values=cache)
+    a = model(input_ids=seq[:, 14:15], past_key_values=cache).logits[:, -1]
+    b = model(input_ids=seq[:, :15], past_key_values=DynamicCache(ec(), device="cpu")).logits[:, -1]
+    assert cache.get_seq_length() == 15
+    torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4)
+
+
+def test_model_requires_a_cache():
+    from fourierattention_amd.llama import random_init
+    model = random_init(_tiny(layers=1), dtype=torch.float32, device="cpu")
+    with pytest.raises(ValueError):
+        model(input_ids=torch.zeros((1, 3), dtype=torch.long), past_key_values=None)
+
+
+def test_eos_stops_the_loop():
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import greedy_generate, random_init
+    cfg = _tiny(layers=1)
+    model = random_init(cfg, dtype=torch.float32, device="cpu", seed=1, std=0.3)
+    masks = _masks(1, cfg.num_key_value_heads, cfg.head_dim, [8, 8], [8, 8])
+    ec = lambda: _cfg(masks, numinittokens=2, maxlocallen=64, maxmidstates=8, num_key_value_heads=cfg.num_key_value_heads,
+                      max_new_tokens=16, max_position_embeddings=256)
+    prompt = torch.tensor([[5, 6, 7, 8]])
+    free = greedy_generate(model, prompt, DynamicCache(ec(), device="cpu"), max_new_tokens=5)
+    stop = greedy_generate(model, prompt, DynamicCache(ec(), device="cpu"), max_new_tokens=5, eos_token_id=int(free[0, 5]))
+    assert stop.shape[1] == 6 and torch.equal(stop, free[:, :6])
+
+
+def _oracle_forward(model, cfg, cache, ids, pos0, gpu_cache):
+    """The model's forward on the CPU in float64 with the oracle cache and the oracle attention."""
+    from oracle import fourier_oracle as fo
+    f64 = lambda t: t.detach().double().cpu().numpy()
+    x = f64(model.model.embed_tokens.weight)[ids.cpu().numpy()]                 # (B, q, hidden)
+    B, q_len, _ = x.shape
+    Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    cos, sin = fo.rope_tables(np.arange(pos0, pos0 + q_len), D, cfg.rope_theta)
+    rms = lambda v, w: v / np.sqrt((v * v).mean(-1, keepdims=True) + cfg.rms_norm_eps) * f64(w)
+    for li, layer in enumerate(model.model.layers):
+        at = layer.self_attn
+        h = rms(x, layer.input_layernorm.weight)
+        proj = lambda lin, n: (h @ f64(lin.weight).T).reshape(B, q_len, n, D).transpose(0, 2, 1, 3)
+        qh, kh, vh = proj(at.q_proj, Hq), proj(at.k_proj, Hkv), proj(at.v_proj, Hkv)
+        qh, kh = fo.apply_rope(qh, cos, sin), fo.apply_rope(kh, cos, sin)
+        kw, vw = cache.update(kh, vh, li)
+        if kw["k_init"] is None and kw["k_compressed"] is None and kw["k_uncompressed"] is None:
+            S = kw["k_local"].shape[1]
+            k = kw["k_local"].reshape(B, S, Hkv, D).transpose(0, 2, 1, 3).repeat(Hq // Hkv, axis=1)
+            v = vw["v_local"].reshape(B, S, Hkv, D).transpose(0, 2, 1, 3).repeat(Hq // Hkv, axis=1)
+            s = np.einsum("bhqd,bhkd->bhqk", qh, k) / np.sqrt(D)
+            s = np.where(np.arange(S)[None, :] <= np.arange(q_len)[:, None] + (S - q_len), s, -np.inf)
+            p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
+            o = np.einsum("bhqk,bhkd->bhqd", p, v)
+        else:
+            for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average"):
+                getattr(cache, n)[li] = getattr(gpu_cache, n)[li].float().cpu().numpy()   # isolate the attention from the stats
+            o = cache.attend(qh, kw, vw, li, Hq, Hkv)
+        o = o.transpose(0, 2, 1, 3).reshape(B, q_len, Hq * D)
+        x = x + o @ f64(at.o_proj.weight).T
+        h2 = rms(x, layer.post_attention_layernorm.weight)
+        gate = h2 @ f64(layer.mlp.gate_proj.weight).T
+        x = x + ((gate / (1 + np.exp(-gate))) * (h2 @ f64(layer.mlp.up_proj.weight).T)) @ f64(layer.mlp.down_proj.weight).T
+    return rms(x, model.model.norm.weight)[:, -1] @ f64(model.lm_head.weight).T
+
+
+@pytest.mark.gpu
+def test_compressed_decode_steps_match_the_oracle_model():
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import LlamaConfig, random_init
+    from oracle.cache_oracle import OracleCache
+    cfg = LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=64, vocab_size=211)
+    model = random_init(cfg, dtype=torch.float32, device="cuda:0", seed=5, std=0.15)
+    masks = _masks(2, 2, 64, [32, 20], [32, 40], seed=2)
+    ec = _cfg(masks, numinittokens=4, maxlocallen=32, maxmidstates=64, num_key_value_heads=2, max_new_tokens=8,
+              max_position_embeddings=1024)
+    gpu, cpu = DynamicCache(ec), OracleCache(ec, masks=masks, model_dtype="fp32")
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, cfg.vocab_size, (2, 300), generator=g)
+    with torch.no_grad():
+        got = model(input_ids=ids.cuda(), past_key_values=gpu, num_logits_to_keep=1).logits[:, -1].cpu().numpy()
+        want = _oracle_forward(model, cfg, cpu, ids, 0, gpu)
+        np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)     # prompt pass: exact attention on both sides
+        nxt = torch.from_numpy(want.argmax(-1))[:, None]
+        for step in range(4):
+            assert gpu.get_seq_length() == 300 + step == cpu.get_seq_length()
+            got = model(input_ids=nxt.cuda(), past_key_values=gpu, num_logits_to_keep=1).logits[:, -1].cpu().numpy()
+            want = _oracle_forward(model, cfg, cpu, nxt, 300 + step, gpu)
+            # fp32 storage: the kernels' fp32 arithmetic against float64; logits are O(1)
+            np.testing.assert_allclose(got, want, rtol=5e-3, atol=5e-3)
+            nxt = torch.from_numpy(want.argmax(-1))[:, None]
