@@ -49,6 +49,11 @@ struct PrepArgs {
   float* c0;
   int Hq, Hkv, D, N, Ck;
   float sm_log2e;
+  // matrix-core mid rows: W goes out in the register layout of that kernel's score waves instead,
+  // [batch group][KV head][frequency slice][row tile][cos | sin][column][pair of frequencies] x 2 frequencies, so
+  // that each of its loads is one contiguous 512-byte line
+  float* W_lane;
+  int nbpg, n_slices, ks;
 };
 
 // bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx
@@ -109,7 +114,18 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx) 
 #pragma unroll
     for (int i = 0; i < 32; ++i) a = fmaf(v[i], s_qs[g][jq + 4 * i], a);
     a = fa_group_sum<4>(a);
-    if (jq == 0) W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = a * mul;
+    if (jq == 0) {
+      if (pa.W_lane) {
+        const int cs = n >= N, nn = n - cs * N;
+        const int per = 16 * pa.ks, sl = nn / per, r = nn - sl * per;
+        const int grp = b / pa.nbpg, lc = (b - grp * pa.nbpg) * G + g;
+        const int lane = lc * 4 + ((r & 7) >> 1);
+        const int64_t tile = ((int64_t)(grp * Hkv + h) * pa.n_slices + sl) * 2 * pa.ks + (r >> 3);
+        pa.W_lane[((tile * 2 + cs) * 64 + lane) * 2 + (r & 1)] = a * mul;
+      } else {
+        W[((int64_t)b * Hq + h * G + g) * 2 * N + n] = a * mul;
+      }
+    }
   }
 }
 
@@ -480,7 +496,11 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ md_on, int n_mid_split, const float* __restrict__ v_mc,
     const float* __restrict__ avg_u, const float* __restrict__ avg_d, const float* __restrict__ scale,
     const int32_t* __restrict__ vc_list, const int32_t* __restrict__ vc_h, const int32_t* __restrict__ vn_list,
-    const int32_t* __restrict__ vn_h, float* __restrict__ out, int Hq, int Hkv, int D, int N, int Cv) {
+    const int32_t* __restrict__ vn_h, float* __restrict__ out, int Hq, int Hkv, int D, int N, int Cv, int g_nbpg) {
+  // g_nbpg > 0: the g partials come from the matrix-core kernel in its own layout, per (batch group of g_nbpg,
+  // KV head, split) N/8 tiles of [column][pair of frequencies] x {cos f, sin f, cos f+1, sin f+1},
+  // column = (batch element within the group) * G + query head within the KV head; otherwise one row of 2N per
+  // (query head, split)
   extern __shared__ float smem[];
   const int G = Hq / Hkv;
   const int n_all = n_il_split + n_mid_split;
@@ -520,12 +540,25 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   constexpr int kGPre = kMergePre / 2;
   const int g_items = G * 2 * N / 4;                 // 2N is a multiple of 4
   const int g_item = tid >> 1, g_half = tid & 1;
+  const int64_t g_split_stride = g_nbpg > 0 ? (int64_t)16 * 2 * N : (int64_t)2 * N;
+  // item -> (query head g, group of four values n4) and the address of its values in split 0
+  auto g_locate = [&](int item, int& g, int& n4) -> const float* {
+    if (g_nbpg > 0) {   // consecutive items walk through the 64 * G contiguous bytes this block owns in a tile
+      g = (item >> 2) % G;
+      n4 = (item / (4 * G)) * 4 + (item & 3);
+      const int grp = b / g_nbpg, lc = (b - grp * g_nbpg) * G + g;
+      return md_g + (int64_t)(grp * Hkv + h) * n_mid_split * g_split_stride + (int64_t)(n4 >> 2) * 256 + (lc * 4 + (n4 & 3)) * 4;
+    }
+    g = item / (2 * N / 4);
+    n4 = item - g * (2 * N / 4);
+    return md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
+  };
   float4 g_pre[kGPre];
   if (has_coef && g_item < g_items) {
-    const int g = g_item / (2 * N / 4), n4 = g_item - g * (2 * N / 4);
-    const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
+    int g, n4;
+    const float* gp = g_locate(g_item, g, n4);
 #pragma unroll
-    for (int u = 0; u < kGPre; ++u) g_pre[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * u, n_mid_split - 1) * 2 * N);
+    for (int u = 0; u < kGPre; ++u) g_pre[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * u, n_mid_split - 1) * g_split_stride);
   }
   // V coefficients: rows part, part + parts, ... of dim c_lo + j
   const int j = tid & (cwp - 1), part = tid / cwp;
@@ -604,8 +637,8 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
         }
       };
       for (int item = g_item; item < g_items; item += 512) {   // same trip count for both threads of a pair
-        const int g = item / (2 * N / 4), n4 = item - g * (2 * N / 4);
-        const float* gp = md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
+        int g, n4;
+        const float* gp = g_locate(item, g, n4);
         const float* wg = s_w + g * n_all + n_il_split;
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
         int u0 = 0;
@@ -618,13 +651,20 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
           float4 v[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u)
-            v[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * (u0 + u), n_mid_split - 1) * 2 * N);
+            v[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * (u0 + u), n_mid_split - 1) * g_split_stride);
 #pragma unroll
           for (int u = 0; u < 4; ++u) fold1(v[u], g_half + 2 * (u0 + u), wg, a);
         }
         a.x += fa_dpp<FA_DPP_XOR1>(a.x); a.y += fa_dpp<FA_DPP_XOR1>(a.y);
         a.z += fa_dpp<FA_DPP_XOR1>(a.z); a.w += fa_dpp<FA_DPP_XOR1>(a.w);
-        if (g_half == 0) *(float4*)(s_g + g * 2 * N + 4 * n4) = a;
+        if (g_half == 0) {
+          if (g_nbpg > 0) {   // {cos f, sin f, cos f+1, sin f+1} with f = 2 * n4
+            *(float2*)(s_g + g * 2 * N + 2 * n4) = make_float2(a.x, a.z);
+            *(float2*)(s_g + g * 2 * N + N + 2 * n4) = make_float2(a.y, a.w);
+          } else {
+            *(float4*)(s_g + g * 2 * N + 4 * n4) = a;
+          }
+        }
       }
       __syncthreads();
       // g . V_coef
@@ -943,14 +983,16 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     o += fa_align_up(bytes, 256);
     return at;
   };
-  p.off_W = take(rows * 2 * N * 4);
+  // W: one row of 2N per query head; the matrix-core path keeps 16 columns per (batch group, KV head) instead
+  p.off_W = take(mfma ? (size_t)p.n_groups * Hkv * 16 * 2 * N * 4 : rows * 2 * N * 4);
   p.off_c0 = take(rows * 4);
   p.off_ilm = take(rows * p.n_il_split * 4);
   p.off_ild = take(rows * p.n_il_split * 4);
   p.off_ilo = take(rows * p.n_il_split * D * 4);
   p.off_mm = take(rows * p.n_mid_split * 4);
   p.off_md = take(rows * p.n_mid_split * 4);
-  p.off_mg = take(rows * p.n_mid_split * 2 * N * 4);
+  // g partials: a row of 2N per (query head, split); the matrix-core path stores 16 columns per (batch group, KV head, split)
+  p.off_mg = take((mfma ? (size_t)p.n_groups * Hkv * 16 : rows) * p.n_mid_split * 2 * N * 4);
   p.off_mon = take(rows * p.n_mid_split * D * 4);
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
   p.n_merge_chunks = 1;
@@ -1029,7 +1071,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   const bool fuse_il = sizeof(E) == 2 && p_il_fast && p.n_il_split > 0 && p.n_mid_split > 0;
   if (p.n_mid_split > 0) {
     PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
-                   a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e};
+                   a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e,
+                   p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks};
     const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
@@ -1124,7 +1167,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     }
     decode_merge_kernel<<<dim3(a.Hkv, a.B, kMergeChunks), 1024, lds, st>>>(
         ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
-        a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv);
+        a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv,
+        p.path == Path::Mfma ? p.nbpg : 0);
   }
   if (ev) hipEventRecord(ev[4], st);
   return fa_check_launch("fa_decode_attn");

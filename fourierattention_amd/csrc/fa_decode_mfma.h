@@ -177,7 +177,8 @@ __device__ __forceinline__ void et1_accumulate(unsigned lane_base, half8 pf, flo
 template <typename E>
 struct MidParams {
   const E* q;
-  const float* W;       // [B][Hq][2N] fp32, already carrying sm_scale*log2e/N
+  const float* W;       // fp32, already carrying sm_scale*log2e/N, in the lane layout of the score waves:
+                        // [batch group][KV head][slice][row tile][cos | sin][column][pair of frequencies] x float2
   const float* c0;      // [B][Hq]
   const E* k_mid;
   const E* v_mid;
@@ -256,19 +257,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int t_end = min(n_tiles, t_beg + p.tiles_per_split);
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
 
-  if ((MODE != 0 || score_wave) && lc == 0) {
-#pragma unroll
-    for (int rt = 0; rt < 2 * KS; ++rt) {
-      const float2v a = p.rot[fbase + freq_of(rt, lg, 0)];
-      const float2v b = p.rot[fbase + freq_of(rt, lg, 1)];
-      s_rot[(sl * 2 * KS + rt) * 4 + lg] = float4v{a[0], a[1], b[0], b[1]};
-      if (TWO) {
-        const float2v a2 = p.rot[N + fbase + freq_of(rt, lg, 0)];
-        const float2v b2 = p.rot[N + fbase + freq_of(rt, lg, 1)];
-        s_rot2[(sl * 2 * KS + rt) * 4 + lg] = float4v{a2[0], a2[1], b2[0], b2[1]};
-      }
+  // Rotation constants of slice sl into LDS: one entry (row tile, pair of frequencies) per lane, requested early and
+  // stored once the other loads of the prologue are on their way.  Where both roles run, the value waves do it (they
+  // have time to spare before the first page).
+  float4v rot_one = float4v{0.f, 0.f, 0.f, 0.f}, rot_two = float4v{0.f, 0.f, 0.f, 0.f};
+  const bool rot_lane_ok = lane < 2 * KS * 4;
+  auto rot_fetch = [&]() {
+    if (rot_lane_ok) {
+      const int f = fbase + freq_of(lane >> 2, lane & 3, 0);   // even: (c, s)(f), (c, s)(f + 1) are 16 aligned bytes
+      rot_one = *(const float4v*)&p.rot[f];
+      if (TWO) rot_two = *(const float4v*)&p.rot[N + f];
     }
-  }
+  };
+  auto rot_store = [&]() {
+    if (rot_lane_ok) {
+      s_rot[(sl * 2 * KS) * 4 + lane] = rot_one;
+      if (TWO) s_rot2[(sl * 2 * KS) * 4 + lane] = rot_two;
+    }
+  };
 
   if (score_wave) {
     // =============================== score waves ===============================
@@ -294,24 +300,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = 0; i < NST - 1; ++i)
         if (i < n_it) issue_k(t_beg + i);
     }
+    if (MODE == 1) rot_fetch();
+    // the index list of the gathered query dims is requested now: the query loads that depend on it then go out
+    // while the tables and the weights are still on their way, instead of starting a round trip of their own later
+    int dim[KMAX][8];
+    if (kn_len > 0) {
+      const int32_t* kl = p.kn_list + kn0;
+#pragma unroll
+      for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dim[s][e] = kl[min(s * 32 + 8 * lg + e, kn_len - 1)];
+    }
     half8 Ea[2][KS];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int s = 0; s < KS; ++s) Ea[rb][s] = p.tabE[((sl * 2 + rb) * KS + s) * 64 + lane];
 
     // coefficient-domain query: Wc/Ws[rt][f2] = (cos-row, sin-row) weights of frequency
     // freq_of(rt, lg, f2) for column lc; normalised per column, rotated to the first page
     float Wc[2 * KS][2], Ws[2 * KS][2];
     float wmax = 0.f;
+    // the gathered query values: requested behind the weights, needed only once those have been processed
+    E qv[KMAX][8];
     {
-      const float* wr = p.W + qrow * 2 * N;
+      const float2v* wl = (const float2v*)p.W + ((int64_t)((grp * p.Hkv + h) * NSL + sl) * 2 * KS * 2) * 64 + (lc * 4 + lg);
+      float2v wc2[2 * KS], ws2[2 * KS];
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) {
-        const int f = fbase + freq_of(rt, lg, 0);
-        float2v c2 = *(const float2v*)(wr + f);      // row 0 stands in for columns past the group
-        float2v s2 = *(const float2v*)(wr + N + f);
-        if (!valid_r) c2 = s2 = float2v{0.f, 0.f};
+        wc2[rt] = wl[(rt * 2 + 0) * 64];
+        ws2[rt] = wl[(rt * 2 + 1) * 64];
+      }
+      // the table operand goes out behind the weights: loads return in order, so the arithmetic on the weights
+      // below runs while the (four times larger) table is still arriving
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) Ea[rb][s] = p.tabE[((sl * 2 + rb) * KS + s) * 64 + lane];
+      if (kn_len > 0) {
+        const E* qr = p.q + qrow * p.D - h * p.D;
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) qv[s][e] = qr[dim[s][e]];
+      }
+#pragma unroll
+      for (int rt = 0; rt < 2 * KS; ++rt) {
+        float2v c2 = wc2[rt], s2 = ws2[rt];
+        if (!valid_r) c2 = s2 = float2v{0.f, 0.f};   // lanes of columns past the group hold nothing
         Wc[rt][0] = c2[0]; Wc[rt][1] = c2[1];
         Ws[rt][0] = s2[0]; Ws[rt][1] = s2[1];
         wmax = fmaxf(wmax, fmaxf(fmaxf(fabsf(c2[0]), fabsf(c2[1])), fmaxf(fabsf(s2[0]), fabsf(s2[1]))));
@@ -349,20 +381,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int s = 0; s < KMAX; ++s)
 #pragma unroll
       for (int e = 0; e < 8; ++e) Qb[s][e] = (typename M::elem)0.f;
-    if (kn_len > 0) {   // one branch around the whole gather; nothing inside is conditional
+    if (kn_len > 0) {   // nothing inside these branches is conditional
       const bool mine = has_mn && valid_r && bb_r == sl;
-      const int32_t* kl = p.kn_list + kn0;
-      const E* qr = p.q + qrow * p.D - h * p.D;
-      int dim[KMAX][8];
-#pragma unroll
-      for (int s = 0; s < KMAX; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dim[s][e] = kl[min(s * 32 + 8 * lg + e, kn_len - 1)];
-      E qv[KMAX][8];
-#pragma unroll
-      for (int s = 0; s < KMAX; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qv[s][e] = qr[dim[s][e]];
 #pragma unroll
       for (int s = 0; s < KMAX; ++s)
 #pragma unroll
@@ -375,6 +395,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
+    if (MODE == 1) rot_store();
     __syncthreads();   // the rotation constants in LDS are complete
     const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
     // score pass: the complete scores of page pg of the split (sum of the eight partials; thread = (column,
@@ -484,14 +505,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = 0; i < NST - 1; ++i)
         if (i < n_it) issue_v(t_beg + i);
     }
+    rot_fetch();
+    uint4v et1v[TWO ? 2 * KS : 1];   // E^T of the second page of a frame, on its way to LDS
     half8 ETa[2 * KS];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
     if (TWO) {
       const uint4v* src = (const uint4v*)(p.tabET + (kFreqWaves + sl) * 2 * KS * 64) + lane;
 #pragma unroll
-      for (int rt = 0; rt < 2 * KS; ++rt) s_et1[(sl * 2 * KS + rt) * 64 + lane] = src[rt * 64];
+      for (int rt = 0; rt < 2 * KS; ++rt) et1v[rt] = src[rt * 64];
     }
+    rot_store();
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -499,10 +523,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int f = 0; f < VMAX; ++f) oacc[f] = float4v{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, d_run = 0.f;
     const bool ragged_tail = (p.L_m & 31) != 0;
-    // the table loads must have landed before the loop starts (see the score waves)
+    __syncthreads();   // the rotation constants in LDS are complete
+    // Only the rotation constants had to be there for the meeting above (the score waves need them for their first
+    // page); this wave's own operands may arrive while the score waves work on that page.  They must have landed
+    // before the loop starts: inside it the only waits on vector memory are the explicit page waits.
+    if (TWO) {
+#pragma unroll
+      for (int rt = 0; rt < 2 * KS; ++rt) s_et1[(sl * 2 * KS + rt) * 64 + lane] = et1v[rt];
+    }
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
-    __syncthreads();   // the rotation constants in LDS are complete
     const unsigned rot_lane = lds_addr_of(TWO ? &s_rot2[(sl * 2 * KS) * 4 + lg] : &s_rot[(sl * 2 * KS) * 4 + lg]);
     const unsigned et1_lane = lds_addr_of(&s_et1[TWO ? (sl * 2 * KS) * 64 + lane : 0]);
     // value pass: the scores of a page (column lc, tokens 8*lg .. 8*lg+7) are fetched one page ahead
@@ -673,34 +703,41 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         p.pm[base] = m_run;
         p.pd[base] = dsum;
       }
-      float* g = p.pg + base * 2 * N;
+    }
+    {
+      // g of this split, back from the page frame (rotation by +phi), in the layout it is held in:
+      // [batch group][KV head][split][slice][row tile][column][pair of frequencies] x {cos f, sin f, cos f+1,
+      // sin f+1}: every store is one contiguous KiB (the columns of one batch element lie side by side for the
+      // merge); lanes of columns past the group store values that nobody reads
+      float4v* gl = (float4v*)p.pg + ((((int64_t)(grp * p.Hkv + h) * p.n_split + split) * NSL + sl) * 2 * KS) * 64 + (lc * 4 + lg);
       const int64_t last = (int64_t)32 * (t_end > t_beg ? t_beg + (TWO ? ((n_it - 1) & ~1) : n_it - 1) : t_beg);
       float sn[2], co[2], s8, c8;   // stepped phases, as for the first page
       fast_sincos_phase(8, last, p.T, &s8, &c8);
 #pragma unroll
       for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), last, p.T, &sn[f2], &co[f2]);
 #pragma unroll
-      for (int rt = 0; rt < 2 * KS; ++rt)
+      for (int rt = 0; rt < 2 * KS; ++rt) {
+        float4v o;
 #pragma unroll
         for (int f2 = 0; f2 < 2; ++f2) {
-          const int f = fbase + freq_of(rt, lg, f2);
           const float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
-          g[f] = co[f2] * x - sn[f2] * y;       // back from the page frame: rotation by +phi
-          g[N + f] = sn[f2] * x + co[f2] * y;
+          o[2 * f2] = co[f2] * x - sn[f2] * y;
+          o[2 * f2 + 1] = sn[f2] * x + co[f2] * y;
           const float cn = co[f2] * c8 - sn[f2] * s8;
           sn[f2] = sn[f2] * c8 + co[f2] * s8;
           co[f2] = cn;
         }
+        gl[rt * 64] = o;
+      }
+    }
+    if (valid_r) {
+      const int64_t base = qrow * p.n_split + split;
       if (has_mn && bb_r == sl) {
-        const int vn_len = p.vn_h[h + 1] - p.vn_h[h];
+        // rows of D floats: dims past the head's stored count are written too (zeros, never read)
         float* on = p.pon + base * p.D;
 #pragma unroll
         for (int f = 0; f < VMAX; ++f)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const int j = f * 16 + 4 * lg + v;
-            if (f < ndg && j < vn_len) on[j] = oacc[f][v];
-          }
+          if (f < ndg) *(float4v*)&on[f * 16 + 4 * lg] = oacc[f];
       }
     }
   }
