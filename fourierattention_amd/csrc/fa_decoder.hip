@@ -1,0 +1,166 @@
+// The elementwise steps of one decoder layer around the attention path, each as one launch: residual add +
+// RMSNorm (modeling_llama_fourier.py:87-92, 735-750), rotary embedding of q and k (213-244), SwiGLU gate
+// (277).  Every value is rounded where the reference's chain of tensor operations rounds it (each tensor op
+// of a 16-bit model rounds its result to that type), so the results agree with that chain to the last bit
+// except where a reduction order or an exponential differs in the last place.
+#include "fa_common.h"
+
+namespace {
+
+template <typename E> struct Rounder;
+template <> struct Rounder<bf16_t> {
+  static __device__ __forceinline__ bf16_t put(float v) { return bf16_t{fa_f32_to_bf16_bits(v)}; }
+};
+template <> struct Rounder<f16_t> {
+  static __device__ __forceinline__ f16_t put(float v) { return f16_t{(_Float16)v}; }
+};
+template <> struct Rounder<float> {
+  static __device__ __forceinline__ float put(float v) { return v; }
+};
+// through the storage type and back: what a tensor op leaves for the next one.  The value passes through an empty
+// asm: the compiler otherwise contracts a product and the sum that follows into one multiply-add (fp32), or folds
+// a conversion to half and back into a mixed-precision multiply-add (fp16) -- both skip exactly the rounding this
+// function is for.
+template <typename E>
+__device__ __forceinline__ float rnd(float v) {
+  float r = fa_to_float(Rounder<E>::put(v));
+  asm("" : "+v"(r));
+  return r;
+}
+template <>
+__device__ __forceinline__ float rnd<f16_t>(float v) {
+  _Float16 h = (_Float16)v;
+  asm("" : "+v"(h));
+  return (float)h;
+}
+
+// one block per row: h += delta (optional), y = weight * (h * rsqrt(mean(h^2) + eps)).to(dtype)
+// W = elements per access: 16 bytes when the row length allows (rows then start 16-byte aligned), else one element
+template <typename E, int W>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(E* __restrict__ h, const E* __restrict__ delta,
+                                                           const E* __restrict__ weight, E* __restrict__ y, int hidden,
+                                                           float eps) {
+  struct alignas(sizeof(E) * W) Pack { E e[W]; };
+  __shared__ float s_red[4];
+  const int64_t row = blockIdx.x;
+  Pack* hr = reinterpret_cast<Pack*>(h + row * hidden);
+  const Pack* dr = delta ? reinterpret_cast<const Pack*>(delta + row * hidden) : nullptr;
+  const Pack* wr = reinterpret_cast<const Pack*>(weight);
+  Pack* yr = reinterpret_cast<Pack*>(y + row * hidden);
+  constexpr int kIter = 8192 / (256 * W);   // hidden <= 8192; all indexing below is static (registers, no scratch)
+  const int packs = hidden / W;
+  float v[kIter][W];
+  float ss = 0.f;
+#pragma unroll
+  for (int n = 0; n < kIter; ++n) {
+    const int i = n * 256 + threadIdx.x;
+    if (i < packs) {
+      Pack a = hr[i];
+      if (dr) {
+        const Pack d = dr[i];
+#pragma unroll
+        for (int e = 0; e < W; ++e) a.e[e] = Rounder<E>::put(fa_to_float(a.e[e]) + fa_to_float(d.e[e]));
+        hr[i] = a;
+      }
+#pragma unroll
+      for (int e = 0; e < W; ++e) {
+        v[n][e] = fa_to_float(a.e[e]);
+        ss += v[n][e] * v[n][e];
+      }
+    }
+  }
+  ss = fa_wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float inv = rsqrtf((s_red[0] + s_red[1] + s_red[2] + s_red[3]) / (float)hidden + eps);
+#pragma unroll
+  for (int n = 0; n < kIter; ++n) {
+    const int i = n * 256 + threadIdx.x;
+    if (i < packs) {
+      const Pack wv = wr[i];
+      Pack o;
+#pragma unroll
+      for (int e = 0; e < W; ++e) o.e[e] = Rounder<E>::put(fa_to_float(wv.e[e]) * rnd<E>(v[n][e] * inv));
+      yr[i] = o;
+    }
+  }
+}
+
+// grid (rows, Hq + Hkv), block D / 2: x <- x * cos + rotate_half(x) * sin on one head of q or k
+template <typename E>
+__global__ void rope_qk_kernel(E* __restrict__ q, E* __restrict__ k, const E* __restrict__ cs, const E* __restrict__ sn,
+                               int Hq, int Hkv, int D) {
+  const int64_t row = blockIdx.x;
+  const int head = blockIdx.y, i = threadIdx.x, half = D >> 1;
+  E* x = head < Hq ? q + (row * Hq + head) * D : k + (row * Hkv + (head - Hq)) * D;
+  const float x1 = fa_to_float(x[i]), x2 = fa_to_float(x[i + half]);
+  const float c1 = fa_to_float(cs[row * D + i]), c2 = fa_to_float(cs[row * D + i + half]);
+  const float s1 = fa_to_float(sn[row * D + i]), s2 = fa_to_float(sn[row * D + i + half]);
+  // rotate_half(x) = (-x2, x1)
+  x[i] = Rounder<E>::put(rnd<E>(x1 * c1) + rnd<E>(-x2 * s1));
+  x[i + half] = Rounder<E>::put(rnd<E>(x2 * c2) + rnd<E>(x1 * s2));
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const E* __restrict__ gate, const E* __restrict__ up,
+                                                        E* __restrict__ out, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float g = fa_to_float(gate[i]);
+  out[i] = Rounder<E>::put(rnd<E>(g / (1.0f + expf(-g))) * fa_to_float(up[i]));
+}
+
+template <typename F>
+int by_dtype(int dtype, const char* what, F&& f) {
+  switch (dtype) {
+    case FA_BF16: f(bf16_t{}); return FA_OK;
+    case FA_FP16: f(f16_t{}); return FA_OK;
+    case FA_FP32: f(float{}); return FA_OK;
+    default: fa_set_error("%s: dtype %d", what, dtype); return FA_ERR_BAD_DTYPE;
+  }
+}
+
+}  // namespace
+
+extern "C" int fa_add_rmsnorm(void* h, const void* delta, const void* weight, void* y, int rows, int hidden, float eps,
+                              int dtype, fa_stream_t stream) {
+  FA_REQUIRE(h && weight && y, FA_ERR_NULL_POINTER, "fa_add_rmsnorm: null pointer");
+  FA_REQUIRE(rows >= 0 && hidden > 0 && hidden <= 8192, FA_ERR_BAD_SHAPE, "fa_add_rmsnorm: rows=%d hidden=%d (at most 8192)",
+             rows, hidden);
+  if (rows == 0) return FA_OK;
+  hipStream_t st = fa_hip_stream(stream);
+  int rc = by_dtype(dtype, "fa_add_rmsnorm", [&](auto tag) {
+    using E = decltype(tag);
+    constexpr int kVec = 16 / (int)sizeof(E);
+    const bool vec = hidden % kVec == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)y) & 15) == 0;
+    if (vec) add_rmsnorm_kernel<E, kVec><<<rows, 256, 0, st>>>((E*)h, (const E*)delta, (const E*)weight, (E*)y, hidden, eps);
+    else add_rmsnorm_kernel<E, 1><<<rows, 256, 0, st>>>((E*)h, (const E*)delta, (const E*)weight, (E*)y, hidden, eps);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_add_rmsnorm");
+}
+
+extern "C" int fa_rope_qk(void* q, void* k, const void* cos, const void* sin, int rows, int Hq, int Hkv, int D, int dtype,
+                          fa_stream_t stream) {
+  FA_REQUIRE(q && k && cos && sin, FA_ERR_NULL_POINTER, "fa_rope_qk: null pointer");
+  FA_REQUIRE(rows >= 0 && Hq > 0 && Hkv > 0 && D > 0 && D % 2 == 0 && D <= 2048, FA_ERR_BAD_SHAPE,
+             "fa_rope_qk: rows=%d Hq=%d Hkv=%d D=%d", rows, Hq, Hkv, D);
+  if (rows == 0) return FA_OK;
+  hipStream_t st = fa_hip_stream(stream);
+  int rc = by_dtype(dtype, "fa_rope_qk", [&](auto tag) {
+    using E = decltype(tag);
+    rope_qk_kernel<E><<<dim3(rows, Hq + Hkv), D / 2, 0, st>>>((E*)q, (E*)k, (const E*)cos, (const E*)sin, Hq, Hkv, D);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_rope_qk");
+}
+
+extern "C" int fa_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, fa_stream_t stream) {
+  FA_REQUIRE(gate && up && out, FA_ERR_NULL_POINTER, "fa_silu_mul: null pointer");
+  FA_REQUIRE(n >= 0, FA_ERR_BAD_SHAPE, "fa_silu_mul: n=%lld", (long long)n);
+  if (n == 0) return FA_OK;
+  hipStream_t st = fa_hip_stream(stream);
+  int rc = by_dtype(dtype, "fa_silu_mul", [&](auto tag) {
+    using E = decltype(tag);
+    silu_mul_kernel<E><<<fa_cdiv(n, 256), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out, n);
+  });
+  return rc != FA_OK ? rc : fa_check_launch("fa_silu_mul");
+}

@@ -19,8 +19,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import synth
-from .attention import LlamaSdpaAttention
+from . import ops, synth
+from .attention import LlamaSdpaAttention, fourier_attention
 from .cache import DynamicCache
 
 
@@ -109,6 +109,24 @@ class LlamaDecoderLayer(nn.Module):
         hidden_states = hidden_states + h
         return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
 
+    def forward_fused(self, h, delta, position_embeddings, past_key_value, cache_position=None):
+        """The same layer on the GPU with its elementwise chains in single launches.  ``h`` is the residual
+        stream, updated in place; ``delta`` the branch output not yet added to it (``None`` for the first layer).
+        Returns this layer's MLP output, to be added by whoever normalises next."""
+        at = self.self_attn
+        y = ops.add_rmsnorm(h, delta, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
+        bsz, q_len, _ = y.shape
+        q, k, v = at.q_proj(y), at.k_proj(y), at.v_proj(y)
+        cos, sin = position_embeddings
+        ops.rope_qk_(q, k, cos, sin, at.head_dim)
+        split = lambda t, n: t.view(bsz, q_len, n, at.head_dim).transpose(1, 2)
+        o = fourier_attention(split(q, at.num_heads), split(k, at.num_key_value_heads), split(v, at.num_key_value_heads),
+                              past_key_value, at.layer_idx, at.num_heads, at.num_key_value_heads,
+                              {"sin": sin, "cos": cos, "cache_position": cache_position})
+        y = ops.add_rmsnorm(h, at.o_proj(o), self.post_attention_layernorm.weight,
+                            self.post_attention_layernorm.variance_epsilon)
+        return self.mlp.down_proj(ops.silu_mul(self.mlp.gate_proj(y), self.mlp.up_proj(y)))
+
 
 class LlamaModel(nn.Module):
     def __init__(self, config: LlamaConfig):
@@ -118,6 +136,9 @@ class LlamaModel(nn.Module):
         self.layers = nn.ModuleList([LlamaDecoderLayer(config, i) for i in range(config.num_hidden_layers)])
         self.norm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self.rotary_emb = LlamaRotaryEmbedding(config)
+        # on the GPU: residual add + RMSNorm, rotary embedding and the SwiGLU gate as one launch each (same
+        # arithmetic and rounding points as the module chain below); False keeps the chain of tensor ops
+        self.fused_elementwise = True
 
     def forward(self, input_ids, past_key_values: DynamicCache, position_ids=None):
         """A cache object is required (modeling_llama_fourier.py:946-949 would otherwise build one without
@@ -131,6 +152,12 @@ class LlamaModel(nn.Module):
         if position_ids is None:
             position_ids = cache_position.unsqueeze(0)
         pe = self.rotary_emb(x, position_ids)
+        if x.is_cuda and self.fused_elementwise and not self.config.attention_bias and x.shape[-1] <= 8192:
+            x, delta = x.contiguous(), None
+            pe = tuple(t.expand(x.shape[0], -1, -1).contiguous() for t in pe)   # one table row per token, made once
+            for layer in self.layers:
+                delta = layer.forward_fused(x, delta, pe, past_key_values, cache_position)
+            return ops.add_rmsnorm(x, delta, self.norm.weight, self.norm.variance_epsilon)
         for layer in self.layers:
             x = layer(x, pe, past_key_values, cache_position)
         return self.norm(x)

@@ -219,6 +219,42 @@ def stream_update(k_new: torch.Tensor, v_new: torch.Tensor, k_ring: torch.Tensor
     check(_lib.load().fa_stream_update(ctypes.byref(a), _stream(k_ring.device)))
 
 
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``h += delta`` (when given, in place) and ``LlamaRMSNorm`` of the result in one launch
+    (modeling_llama_fourier.py:735-750, 87-92).  ``h, delta (..., hidden)`` contiguous."""
+    _require_gpu(h, "h")
+    assert h.is_contiguous() and weight.is_contiguous() and weight.dtype == h.dtype
+    assert delta is None or (delta.is_contiguous() and delta.shape == h.shape and delta.dtype == h.dtype)
+    y = torch.empty_like(h)
+    hidden = h.shape[-1]
+    check(_lib.load().fa_add_rmsnorm(h.data_ptr(), _ptr(delta), weight.data_ptr(), y.data_ptr(), h.numel() // hidden, hidden,
+                                     float(eps), dtype_code(h.dtype), _stream(h.device)))
+    return y
+
+
+def rope_qk_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, head_dim: int) -> None:
+    """Rotary embedding in place on ``q (B, q_len, Hq*D)`` and ``k (B, q_len, Hkv*D)`` (the projection outputs);
+    ``cos, sin (B or 1, q_len, D)`` (modeling_llama_fourier.py:213-244)."""
+    _require_gpu(q, "q")
+    assert q.is_contiguous() and k.is_contiguous() and q.dtype == k.dtype
+    rows = q.shape[0] * q.shape[1]
+    if cos.shape[0] != q.shape[0]:
+        cos, sin = cos.expand(q.shape[0], -1, -1), sin.expand(q.shape[0], -1, -1)
+    cos, sin = cos.to(q.dtype).contiguous(), sin.to(q.dtype).contiguous()
+    check(_lib.load().fa_rope_qk(q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, q.shape[2] // head_dim,
+                                 k.shape[2] // head_dim, head_dim, dtype_code(q.dtype), _stream(q.device)))
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` in one launch (modeling_llama_fourier.py:277)."""
+    _require_gpu(gate, "gate")
+    assert gate.is_contiguous() and up.is_contiguous() and gate.shape == up.shape and gate.dtype == up.dtype
+    out = torch.empty_like(gate)
+    check(_lib.load().fa_silu_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), dtype_code(gate.dtype),
+                                  _stream(gate.device)))
+    return out
+
+
 class MultiDimHiPPO2(torch.nn.Module):
     """Same call contract as the reference class (TRI:840-865): without ``slice_input`` the
     whole ``base_input (B, L, C)`` is projected (period and length ``int(1/dt)``: longer inputs

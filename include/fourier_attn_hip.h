@@ -270,6 +270,27 @@ int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
  * (3) the merge kernel.  A measurement aid for benchmarks (the reference has no timers). */
 int fa_decode_attn_timed(const fa_decode_args* args, fa_stream_t stream, float* ms_out);
 
+/* ---------------------------------------------------------------------------
+ * Elementwise steps of the decoder layer around the attention (one launch each)
+ * ------------------------------------------------------------------------- */
+
+/* The residual add of LlamaDecoderLayer.forward followed by LlamaRMSNorm.forward
+ * (MODEL:735-750, 87-92): if delta is non-NULL, h <- h + delta (rounded to
+ * `dtype`, in place); y = weight * (h * rsqrt(mean(h^2) + eps)).to(dtype).
+ * h, delta, y: (rows, hidden) contiguous; weight: (hidden); hidden <= 8192. */
+int fa_add_rmsnorm(void* h, const void* delta, const void* weight, void* y, int rows, int hidden,
+                   float eps, int dtype, fa_stream_t stream);
+
+/* apply_rotary_pos_emb (MODEL:213-244) in place: x <- x * cos + rotate_half(x) * sin
+ * on every head of q (rows, Hq * D) and k (rows, Hkv * D); cos, sin: (rows, D) in
+ * `dtype`.  Products and sum are rounded to `dtype` one by one like the tensor ops. */
+int fa_rope_qk(void* q, void* k, const void* cos, const void* sin, int rows, int Hq, int Hkv, int D,
+               int dtype, fa_stream_t stream);
+
+/* act_fn(gate_proj(x)) * up_proj(x) of LlamaMLP.forward (MODEL:277) with
+ * act_fn = silu: out[i] = silu(gate[i]).to(dtype) * up[i], n elements. */
+int fa_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, fa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

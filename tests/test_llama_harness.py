@@ -130,3 +130,70 @@ def test_compressed_decode_steps_match_the_oracle_model():
             # fp32 storage: the kernels' fp32 arithmetic against float64; logits are O(1)
             np.testing.assert_allclose(got, want, rtol=5e-3, atol=5e-3)
             nxt = torch.from_numpy(want.argmax(-1))[:, None]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
+    """fa_add_rmsnorm / fa_rope_qk / fa_silu_mul against the chains of tensor ops they replace
+    (LlamaRMSNorm.forward after the residual add, apply_rotary_pos_emb, silu(gate) * up)."""
+    from fourierattention_amd import ops
+    from fourierattention_amd.attention import apply_rotary_pos_emb
+    from fourierattention_amd.llama import LlamaRMSNorm
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g, device="cuda", dtype=torch.float32)
+    ulp = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 2e-6}[dtype]
+    # residual add + RMSNorm (hidden not a multiple of the block size on purpose)
+    for rows, hidden in ((5, 4096), (3, 1000), (2, 1001)):   # the last one takes the element-wise variant
+        h, d = (rn(rows, 1, hidden) * 2).to(dtype), rn(rows, 1, hidden).to(dtype)
+        norm = LlamaRMSNorm(hidden, 1e-5).cuda().to(dtype)
+        norm.weight.data = (1 + 0.1 * rn(hidden)).to(dtype)
+        want_h = h + d
+        want_y = norm(want_h)
+        h2 = h.clone()
+        y = ops.add_rmsnorm(h2, d, norm.weight, 1e-5)
+        assert torch.equal(h2, want_h)                                    # the add rounds exactly like the tensor add
+        torch.testing.assert_close(y.float(), want_y.float(), rtol=ulp, atol=ulp)   # reduction order: last place only
+        y0 = ops.add_rmsnorm(h2, None, norm.weight, 1e-5)                 # no delta: h untouched
+        assert torch.equal(h2, want_h) and torch.equal(y0, y)
+    # rotary embedding: no reduction anywhere, so bit for bit
+    B, q_len, Hq, Hkv, D = 3, 2, 6, 2, 64
+    q, k = rn(B, q_len, Hq * D).to(dtype), rn(B, q_len, Hkv * D).to(dtype)
+    ang = rn(B, q_len, D) * 3
+    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+    wq, wk = apply_rotary_pos_emb(q.view(B, q_len, Hq, D).transpose(1, 2), k.view(B, q_len, Hkv, D).transpose(1, 2), cos, sin)
+    q2, k2 = q.clone(), k.clone()
+    ops.rope_qk_(q2, k2, cos, sin, D)
+    assert torch.equal(q2.view(B, q_len, Hq, D).transpose(1, 2), wq) and torch.equal(k2.view(B, q_len, Hkv, D).transpose(1, 2), wk)
+    # SwiGLU gate: the exponential may differ in the last place
+    gate, up = (rn(7, 1, 1111) * 3).to(dtype), rn(7, 1, 1111).to(dtype)
+    want = torch.nn.functional.silu(gate) * up
+    torch.testing.assert_close(ops.silu_mul(gate, up).float(), want.float(), rtol=2 * ulp, atol=2 * ulp)
+
+
+@pytest.mark.gpu
+def test_fused_decoder_path_matches_the_module_chain():
+    """The same bf16 model stepped with and without the fused elementwise launches."""
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import LlamaConfig, random_init
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=64, vocab_size=301)
+    model = random_init(cfg, dtype=torch.bfloat16, device="cuda:0", seed=7, std=0.05)
+    masks = _masks(3, 2, 64, [32, 32], [32, 32], seed=4)
+    ec = lambda: _cfg(masks, numinittokens=4, maxlocallen=32, maxmidstates=64, num_key_value_heads=2, max_new_tokens=8,
+                      max_position_embeddings=1024)
+    ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(3)).cuda()
+    outs = []
+    with torch.no_grad():
+        for fused in (True, False):
+            model.model.fused_elementwise = fused
+            cache = DynamicCache(ec())
+            logits = [model(input_ids=ids, past_key_values=cache, num_logits_to_keep=1).logits[:, -1]]
+            tok = logits[0].argmax(-1, keepdim=True)
+            for _ in range(3):
+                logits.append(model(input_ids=tok, past_key_values=cache, num_logits_to_keep=1).logits[:, -1])
+                tok = logits[-1].argmax(-1, keepdim=True)
+            outs.append(torch.stack(logits))
+    # identical rounding points; only reduction order (norm) and the exponential differ in the last place of bf16
+    torch.testing.assert_close(outs[0], outs[1], rtol=3e-2, atol=3e-2)
+    assert (outs[0] - outs[1]).abs().mean().item() < 3e-3
