@@ -30,6 +30,7 @@ constexpr int kPart = 36;  // padded row (tokens) of the LDS score partials, flo
 // (row tile rt = 2s + v/2, lane group lg, pair v%2) of the g GEMM's rows: per lane the same set
 __device__ __forceinline__ int freq_of(int rt, int lg, int fi2) { return rt * 8 + lg * 2 + fi2; }
 
+constexpr float kLazyLog2 = 8.0f;   // slack of the running softmax reference, in powers of two
 constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one slice per SIMD)
 
 // ---------------------------------------------------------------------------
@@ -116,17 +117,40 @@ __device__ __forceinline__ void rot_pair(float c, float s, float& x, float& y) {
   x = __builtin_fmaf(c, x, sy);
   y = __builtin_fmaf(c, y, -sx);
 }
-// The same with the results in the registers of the operands.  State that lives across loop iterations in plain
-// registers (not in accumulators of the matrix unit) is otherwise left wherever the last instruction of a rotation
-// put it, and every iteration ends with one move per value to bring the registers back in order.
-__device__ __forceinline__ void rot_pair_in_place(float c, float s, float& x, float& y) {
-  float sy, sx;
-  asm("v_mul_f32 %0, %4, %3\n\t"
-      "v_mul_f32 %1, %4, %2\n\t"
-      "v_fma_f32 %2, %5, %2, %0\n\t"
-      "v_fma_f32 %3, %5, %3, -%1"
-      : "=&v"(sy), "=&v"(sx), "+v"(x), "+v"(y)
-      : "v"(s), "v"(c));
+// The same for the four pairs of two row tiles with the results in the registers of the operands.  State that lives
+// across loop iterations in plain registers (not in accumulators of the matrix unit) is otherwise left wherever the
+// last instruction of a rotation put it, and every iteration ends with one move per value to bring the registers
+// back in order.  Four pairs per statement: the compiler separates every asm statement from what follows by a
+// wait state, so one statement per pair would cost as many idle issue slots as it saves moves.
+// k0, k1: {c, s, c', s'} of the two row tiles; x*, y*: (cos-row, sin-row) values of the pairs (tile, 0), (tile, 1).
+__device__ __forceinline__ void rot_two_tiles_in_place(uint4v k0, uint4v k1, float& x00, float& y00, float& x01, float& y01,
+                                                       float& x10, float& y10, float& x11, float& y11) {
+  const unsigned c00 = k0[0], s00 = k0[1], c01 = k0[2], s01 = k0[3];   // scalars first: see fa_swap16
+  const unsigned c10 = k1[0], s10 = k1[1], c11 = k1[2], s11 = k1[3];
+  float t0, t1;
+  asm volatile(
+      "v_mul_f32 %0, %11, %3\n\tv_mul_f32 %1, %11, %2\n\tv_fma_f32 %2, %10, %2, %0\n\tv_fma_f32 %3, %10, %3, -%1\n\t"
+      "v_mul_f32 %0, %13, %5\n\tv_mul_f32 %1, %13, %4\n\tv_fma_f32 %4, %12, %4, %0\n\tv_fma_f32 %5, %12, %5, -%1\n\t"
+      "v_mul_f32 %0, %15, %7\n\tv_mul_f32 %1, %15, %6\n\tv_fma_f32 %6, %14, %6, %0\n\tv_fma_f32 %7, %14, %7, -%1\n\t"
+      "v_mul_f32 %0, %17, %9\n\tv_mul_f32 %1, %17, %8\n\tv_fma_f32 %8, %16, %8, %0\n\tv_fma_f32 %9, %16, %9, -%1"
+      : "=&v"(t0), "=&v"(t1), "+v"(x00), "+v"(y00), "+v"(x01), "+v"(y01), "+v"(x10), "+v"(y10), "+v"(x11), "+v"(y11)
+      : "v"(c00), "v"(s00), "v"(c01), "v"(s01), "v"(c10), "v"(s10), "v"(c11), "v"(s11));
+}
+// The page-step rotation of the 2*KS row tiles held in x[rt][f2], y[rt][f2] with that helper; the first two batches
+// of constants must be in flight in rc[0], rc[1]
+template <int NT, int B>
+__device__ __forceinline__ void rot_apply_in_place_from(unsigned lane_base, uint4v (&rc)[2][4], float (&x)[NT][2], float (&y)[NT][2]) {
+  constexpr int NB = NT / 4;
+  if constexpr (B < NB) {
+    if (B + 1 < NB) lds_wait_for4<4>(rc[B % 2]);
+    else lds_wait_for4<0>(rc[B % 2]);
+    rot_two_tiles_in_place(rc[B % 2][0], rc[B % 2][1], x[4 * B][0], y[4 * B][0], x[4 * B][1], y[4 * B][1],
+                           x[4 * B + 1][0], y[4 * B + 1][0], x[4 * B + 1][1], y[4 * B + 1][1]);
+    rot_two_tiles_in_place(rc[B % 2][2], rc[B % 2][3], x[4 * B + 2][0], y[4 * B + 2][0], x[4 * B + 2][1], y[4 * B + 2][1],
+                           x[4 * B + 3][0], y[4 * B + 3][0], x[4 * B + 3][1], y[4 * B + 3][1]);
+    if constexpr (B + 2 < NB) rot_issue_after<B + 2>(lane_base, rc[B % 2], y[4 * B + 3][1]);
+    rot_apply_in_place_from<NT, B + 1>(lane_base, rc, x, y);
+  }
 }
 // pair(rt, f2, c, s) applies one rotation and returns one of its results; pin(b) passes the results of
 // batch b (row tiles 4b .. 4b+3) through an empty asm volatile, which keeps their arithmetic above the
@@ -447,14 +471,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
         }
         // advance W' by one page step
-        rot_apply<2 * KS, 2>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
-          rot_pair_in_place(c, sn, Wc[rt][f2], Ws[rt][f2]);
-          return Ws[rt][f2];
-        }, [&](int b) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            asm volatile("" : "+v"(Wc[4 * b + j][0]), "+v"(Wc[4 * b + j][1]), "+v"(Ws[4 * b + j][0]), "+v"(Ws[4 * b + j][1]));
-        });
+        rot_apply_in_place_from<2 * KS, 0>(rot_lane, rc, Wc, Ws);
         float4v accm[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
         if (has_k) {
 #pragma unroll
@@ -492,7 +509,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int vp0 = p.vpad_h[h], dpv = p.vpad_h[h + 1] - vp0;
     const int ndg = dpv >> 4;
     const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
-    const bool has_v = has_mn && ndg > 0;
+    const bool streams_v = has_mn && ndg > 0;
     auto issue_v = [&](int t) {            // page t -> stage (t - t_beg) % NST
       const E* vp = vbase + (int64_t)t * dpv * 32;
       unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
@@ -500,7 +517,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int f = 0; f < VMAX; ++f)
         if (f < ndg) load_frag_to_lds<2>(vp + f * 512 + lane * 8, st + f * 1024);
     };
-    if (has_v) {   // first pages requested before the tables (see the score waves)
+    if (streams_v) {   // first pages requested before the tables (see the score waves)
 #pragma unroll
       for (int i = 0; i < NST - 1; ++i)
         if (i < n_it) issue_v(t_beg + i);
@@ -547,7 +564,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // one page of the value stage (page it - 1 of the split)
-    auto value_page = [&](int it, auto first_tag) {
+    // (whether this wave streams V is fixed for the whole loop: a parameter of the body, not a branch in it)
+    auto value_page = [&](int it, auto first_tag, auto stream_tag) {
+        constexpr bool has_v = decltype(stream_tag)::value;
         const int t = t_beg + it - 1, buf = (it - 1) & 1;
         const int pg = it - 1;   // page index within the split
         constexpr int RCB = VMAX > 4 ? 1 : 2;   // the wide variant has no registers to spare for a second batch
@@ -567,7 +586,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             asm volatile("" : "+v"(sc[e]));
           }
         }
-        if (has_v) {
+        if constexpr (has_v) {
           if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
           else wait_vmcnt<0>();
           if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
@@ -616,7 +635,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         uint4v vraw[4];   // four dim groups at a time
         const unsigned vst = lds_addr_of(&s_stage[MODE == 0 ? w : stw][pg % NST][0]) + lane * 16;
-        if (has_v) {
+        if constexpr (has_v) {
           vraw[0] = lds_read_b128_async_at<0>(vst);
           vraw[1] = lds_read_b128_async_at<1024>(vst);
           vraw[2] = lds_read_b128_async_at<2048>(vst);
@@ -630,8 +649,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         float tmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
         tmax = fa_rows_max(tmax);
-        const float m_new = fmaxf(m_run, tmax);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first page (m_run = -inf)
+        // The softmax reference of a column moves only when the page maximum exceeds it by more than kLazyLog2:
+        // until then the probabilities are taken against the old reference (at most 2^kLazyLog2, exact in the
+        // 16-bit operands and far from any overflow) and nothing accumulated so far has to be rescaled.  With a
+        // reference that follows every new maximum, some column of the sixteen moves it on most pages, and each
+        // time the whole g history and the outputs are multiplied through.
+        const float m_new = tmax > m_run + kLazyLog2 ? tmax : m_run;   // first page: m_run = -inf, so tmax
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first page
         float psum = 0.f;
         half8 pf;
         vec8 pe;
@@ -658,7 +682,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         } else {
           et1_accumulate<2 * KS, 0>(et1_lane, pf, hacc, rc[0]);   // the constant buffer is idle on these pages
         }
-        if (has_v) {
+        if constexpr (has_v) {
 #pragma unroll
           for (int f0 = 0; f0 < VMAX; f0 += 4) {
             if (f0 > 0) {
@@ -671,29 +695,34 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             lds_wait_for4<0>(vraw);
 #pragma unroll
             for (int f = 0; f < 4; ++f)
-              if (f0 + f < ndg) oacc[f0 + f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f0 + f]);
+              oacc[f0 + f] = M::mma(__builtin_bit_cast(vec8, vraw[f]), pe, oacc[f0 + f]);   // a fragment the head does not
+              // have multiplies whatever its stage slot holds into an accumulator that is never stored
           }
         }
     };
-    if constexpr (MODE == 2) {
-      for (int it = 1; it <= n_it; ++it) value_page(it, std::true_type{});
-    } else if constexpr (TWO) {
-      barrier_lds_only();   // iteration 0: the score waves are one page ahead
-      for (int it = 1; it <= n_it; it += 2) {
-        value_page(it, std::true_type{});
-        barrier_lds_only();
-        if (it + 1 <= n_it) {
-          value_page(it + 1, std::false_type{});
+    auto value_loop = [&](auto stream_tag) {
+      if constexpr (MODE == 2) {
+        for (int it = 1; it <= n_it; ++it) value_page(it, std::true_type{}, stream_tag);
+      } else if constexpr (TWO) {
+        barrier_lds_only();   // iteration 0: the score waves are one page ahead
+        for (int it = 1; it <= n_it; it += 2) {
+          value_page(it, std::true_type{}, stream_tag);
+          barrier_lds_only();
+          if (it + 1 <= n_it) {
+            value_page(it + 1, std::false_type{}, stream_tag);
+            barrier_lds_only();
+          }
+        }
+      } else {
+        barrier_lds_only();   // iteration 0: the score waves are one page ahead
+        for (int it = 1; it <= n_it; ++it) {
+          value_page(it, std::true_type{}, stream_tag);
           barrier_lds_only();
         }
       }
-    } else {
-      barrier_lds_only();   // iteration 0: the score waves are one page ahead
-      for (int it = 1; it <= n_it; ++it) {
-        value_page(it, std::true_type{});
-        barrier_lds_only();
-      }
-    }
+    };
+    if (streams_v) value_loop(std::true_type{});
+    else value_loop(std::false_type{});
 
     // ---- partials of this split ------------------------------------------------------
     const float dsum = fa_rows_sum(d_run);
