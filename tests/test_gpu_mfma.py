@@ -88,6 +88,41 @@ def test_mfma_decode_matches_oracle_and_generic(case):
         assert e_mfma <= 5e-3, e_mfma
 
 
+@pytest.mark.parametrize("shape", ["ramp", "spike"])
+def test_mfma_softmax_reference_moves(shape):
+    """Key magnitudes that grow along the sequence (the running softmax reference has to move again and again)
+    and a late burst of keys with scores far above everything before (it moves by much more than its slack)."""
+    from fourierattention_amd import DynamicCache
+    dtype, B, Hq, Hkv, D, I, W, M, prompt = torch.bfloat16, 2, 8, 2, 128, 4, 32, 256, 1500
+    masks = _masks(1, Hkv, D, [64, 64], [64, 64], seed=11)
+    cfg = _cfg(masks, numinittokens=I, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=16)
+    gpu = DynamicCache(cfg)
+    cpu = OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
+    r = np.random.default_rng(77)
+    k0 = r.standard_normal((B, Hkv, prompt, D))
+    if shape == "ramp":
+        k0 *= (0.1 + 4.0 * np.arange(prompt) / prompt)[None, None, :, None]
+    else:
+        k0[:, :, 1100:1110, :] *= 12.0
+    k0 = H.to_dtype_np(k0, dtype)
+    v0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)) + 0.1, dtype)
+    gpu.update(H.to_gpu(k0, dtype), H.to_gpu(v0, dtype), 0)
+    cpu.update(k0, v0, 0)
+    kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype); vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+    q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)) * 1.5, dtype)
+    gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), 0)
+    kw, vw = cpu.update(kn, vn, 0)
+    for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average"):
+        getattr(cpu, n)[0] = getattr(gpu, n)[0].float().cpu().numpy()
+    want = cpu.attend(q, kw, vw, 0, Hq, Hkv)
+    assert gpu._tables is not None
+    got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv).cpu().numpy()
+    assert np.isfinite(got).all()
+    err = np.abs(got - want).max()
+    assert err <= 2e-2, err        # the stated bound
+    assert err <= 8e-3, err        # sharply peaked softmax: the bf16 probabilities dominate
+
+
 def test_full_size_properties():
     """BASELINE config 3 at full size (B=8, 32k context): properties that need no CPU oracle.
     (1) the matrix-core path and the generic path (independent kernels, each checked against the oracle at
