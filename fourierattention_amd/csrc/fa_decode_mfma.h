@@ -231,7 +231,7 @@ struct MidParams {
 //   waves 4-7 ("value waves")  page t  : sum the four partials, online softmax, rotate/rescale the g history,
 //                              g' += E^T . P (their frequency slice), o_n += V_mn^T . P (their batch element)
 // Score wave i and value wave i own the same frequencies and stream the same batch element of the group.
-// KS: ksteps (32 coefficient rows) per slice = N / 64.  KMAX: ksteps of stored K dims a head may have
+// KS: ksteps (32 coefficient rows) per slice = N / (16 * slices).  KMAX: ksteps of stored K dims a head may have
 // (dp_k / 32).  VMAX: V dim groups of 16 (dp_v / 16).
 // NST: page stages per wave in LDS; the K / V pages travel HBM -> LDS with global_load_lds (no registers
 // held while in flight), NST - 1 pages ahead of their use.
