@@ -146,5 +146,17 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_mat_fourier(p, 7, 0, 0, None, p, 1, 1, 1, 1, 1, 0, 0, None, 0, None) == -3
     assert lib.fa_mat_avg_std(p, 0, 0, 0, None, p, p, 1, 4, 4, 2, None, 0, None) == -4
     assert lib.fa_coeff_update(p, None, 0, 0, None, 1, 1, 1, 0, 1, None) == -1
+    # the decoder-side elementwise entry points and the streaming update
+    assert lib.fa_add_rmsnorm(None, None, p, p, 1, 64, 1e-5, 0, None) == -1
+    assert lib.fa_add_rmsnorm(p, None, p, p, 1, 9000, 1e-5, 0, None) == -2     # rows longer than 8192
+    assert lib.fa_add_rmsnorm(p, None, p, p, 1, 64, 1e-5, 5, None) == -3
+    assert lib.fa_add_rmsnorm(p, None, p, p, 0, 64, 1e-5, 0, None) == 0         # nothing to do
+    assert lib.fa_rope_qk(p, None, p, p, 1, 4, 2, 64, 0, None) == -1
+    assert lib.fa_rope_qk(p, p, p, p, 1, 4, 2, 63, 0, None) == -2              # odd head_dim
+    assert lib.fa_silu_mul(p, p, None, 8, 0, None) == -1
+    assert lib.fa_silu_mul(p, p, p, -1, 0, None) == -2
+    assert lib.fa_stream_update(None, None) == -1
+    sa = _lib.StreamArgs()
+    assert lib.fa_stream_update(ctypes.byref(sa), None) == -2                  # empty shape
     assert lib.fa_stats_workspace_bytes(2, 10, 1000) == 3 * 2 * 4 * 10 * 4
     assert lib.fa_decode_attn_workspace_bytes(8, 32, 8, 128, 512, 1028, 31740) > 0
