@@ -376,9 +376,38 @@ def triton_fourier_attn(q, k_il, v_il, k_mc, v_mc, k_mn, v_mn,
     lists = tuple(as_i32(t) for t in (kc_list, kc_h_list, kn_list, kn_h_list, vc_list, vc_h_list, vn_list, vn_h_list))
     k_mc = k_mc if k_mc.dtype == torch.float32 else k_mc.float()
     v_mc = v_mc if v_mc.dtype == torch.float32 else v_mc.float()
+    k_mn, v_mn = _paged_if_worthwhile(q, k_mn, v_mn, k_mc if kc_list.numel() else v_mc, lists[3], lists[7], num_head_q,
+                                      num_head_kv, int(seq_len_m))
     return decode_attn_raw(q.contiguous(), [(k_il, v_il)], k_mc.contiguous(), v_mc.contiguous(), k_mn, v_mn,
                            (f32(avg_k_u), f32(avg_k_d), f32(scale_k)), (f32(avg_v_u), f32(avg_v_d), f32(scale_v)),
                            lists, num_head_q, num_head_kv, seq_len_m, T, sm_scale)
+
+
+# below this many mid rows the any-layout kernels are quicker than re-paging first
+_REPACK_MIN_ROWS = 2048
+
+
+def _paged_if_worthwhile(q, k_mn, v_mn, coef, kn_h32, vn_h32, num_head_q, num_head_kv, seq_len_m):
+    """The reference hands ``k_mn`` / ``v_mn`` over token-major (``torch.cat`` of gathered columns,
+    cache_utils_fourier.py:735, 741).  The matrix-core kernels stream pages; for long contexts copying the
+    rows into a temporary page store first (two passes over them) and taking those kernels is several times
+    faster than the kernels that read the token-major layout in place.  ``DynamicCache`` keeps its rows paged
+    and never comes through here."""
+    from .midstore import MidStore
+    if isinstance(k_mn, MidStore) or seq_len_m < _REPACK_MIN_ROWS or q.dtype not in (torch.bfloat16, torch.float16):
+        return k_mn, v_mn
+    D = q.shape[2] // num_head_q
+    n_f = coef.shape[1] // 2
+    if n_f not in (128, 256, 512, 1024) or D > 128 or num_head_q // num_head_kv > 8 or k_mn.dtype != q.dtype:
+        return k_mn, v_mn
+    stores = []
+    for t, n_h, is_v in ((k_mn, kn_h32, False), (v_mn, vn_h32, True)):
+        n_h_host = [int(x) for x in n_h.tolist()]
+        ident = torch.arange(n_h_host[-1], dtype=torch.int32, device=q.device)   # the columns are gathered already
+        st = MidStore(t.shape[0], ident, n_h, n_h_host, num_head_kv, D, seq_len_m, t.dtype, q.device, is_v)
+        st.pack(t, 0, seq_len_m)
+        stores.append(st)
+    return stores[0], stores[1]
 
 
 fourier_attn = triton_fourier_attn

@@ -129,6 +129,26 @@ def test_decode_attention_matches_oracle(case_id, dtype, tol):
     assert err <= 5e-4, err
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_function_level_drop_in_repages_long_token_major_inputs(dtype, monkeypatch):
+    """``triton_fourier_attn`` with the reference's token-major ``k_mn`` / ``v_mn`` and a long mid: the rows are
+    copied into a temporary page store and the matrix-core kernels run; the result must agree with the oracle
+    and with the kernels that read the token-major tensors in place."""
+    from fourierattention_amd import ops
+    B, Hq, Hkv, D, n_il, L, n_f, T = 2, 8, 2, 128, 40, 2500, 128, 2700
+    case = H.attn_case(321, B, Hq, Hkv, D, n_il, L, n_f, T, [64, 100], [30, 64], dtype)
+    want = fo.fourier_attn(**case)
+    g = H.attn_case_gpu(case, dtype)
+    got = ops.triton_fourier_attn(**g).cpu().numpy()
+    monkeypatch.setattr(ops, "_REPACK_MIN_ROWS", 1 << 30)
+    in_place = ops.triton_fourier_attn(**g).cpu().numpy()
+    assert np.abs(in_place - want).max() <= 5e-4
+    err = np.abs(got - want).max()
+    assert err <= 2e-2, err          # the stated bound for 16-bit storage
+    assert err <= 5e-3, err          # f16 basis and 16-bit probabilities on the matrix cores
+    assert np.abs(got - in_place).max() > 0     # it did take the other kernels
+
+
 def test_decode_attention_window_only_and_errors():
     from fourierattention_amd import ops, _lib
     case = H.attn_case(7, 2, 8, 2, 64, 300, 0, 4, 50, [10, 10], [10, 10], torch.bfloat16)
