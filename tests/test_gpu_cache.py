@@ -109,6 +109,38 @@ def test_cache_prefill_and_streaming(dtype, prompt, max_new, max_pos, expect_T):
         assert gpu._seen_tokens == cpu._seen_tokens == prompt + s + 1
 
 
+def test_streaming_wraps_the_window_buffer_and_crosses_pages():
+    """More decode steps than the window buffer has slots (the write / evict slots wrap around several times)
+    and enough evicted rows to cross page boundaries of the mid store: parts and attention after every step."""
+    from fourierattention_amd import DynamicCache
+    dtype, B, Hq, Hkv, D, W, prompt, steps = torch.bfloat16, 2, 4, 2, 64, 8, 90, 41
+    masks = _masks(1, Hkv, D, [40, 17], [64, 0], seed=5)
+    cfg = _cfg(masks, maxlocallen=W, max_new_tokens=64, max_position_embeddings=4096)
+    gpu = DynamicCache(cfg)
+    cpu = OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
+    r = np.random.default_rng(21)
+    k0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    v0 = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    gpu.update(H.to_gpu(k0, dtype), H.to_gpu(v0, dtype), 0)
+    cpu.update(k0, v0, 0)
+    for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average"):
+        getattr(cpu, n)[0] = getattr(gpu, n)[0].float().cpu().numpy()
+    for s in range(steps):
+        kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+        vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+        q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)), dtype)
+        kp, vp = gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), 0)
+        kw, vw = cpu.update(kn, vn, 0)
+        if s % 5 == 0 or s == steps - 1:
+            _compare_parts(kp, kw, "k", dtype)       # window rows in order, evicted rows appended, coefficients
+            _compare_parts(vp, vw, "v", dtype)
+        assert gpu.get_seq_length(0) == cpu.get_seq_length(0) == prompt + s + 1
+        got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv).cpu().numpy()
+        err = np.abs(got - cpu.attend(q, kw, vw, 0, Hq, Hkv)).max()
+        assert err <= 2e-2 and err <= 1e-3, (s, err)
+    assert gpu._layers[0].n_mid == cpu.key_cache[0]["k_uncompressed"].shape[1] == prompt - 4 - W + steps > 96   # pages crossed
+
+
 def test_short_prompt_stays_in_window_and_matches_exact_attention():
     from fourierattention_amd import DynamicCache, fourier_attention
     B, Hq, Hkv, D = 2, 8, 2, 64
