@@ -109,13 +109,14 @@ def test_cache_prefill_and_streaming(dtype, prompt, max_new, max_pos, expect_T):
         assert gpu._seen_tokens == cpu._seen_tokens == prompt + s + 1
 
 
-def test_streaming_wraps_the_window_buffer_and_crosses_pages():
+@pytest.mark.parametrize("max_pos", [4096, 100])   # 100: the page store is sized for 96 rows and has to grow on the way
+def test_streaming_wraps_the_window_buffer_and_crosses_pages(max_pos):
     """More decode steps than the window buffer has slots (the write / evict slots wrap around several times)
     and enough evicted rows to cross page boundaries of the mid store: parts and attention after every step."""
     from fourierattention_amd import DynamicCache
     dtype, B, Hq, Hkv, D, W, prompt, steps = torch.bfloat16, 2, 4, 2, 64, 8, 90, 41
     masks = _masks(1, Hkv, D, [40, 17], [64, 0], seed=5)
-    cfg = _cfg(masks, maxlocallen=W, max_new_tokens=64, max_position_embeddings=4096)
+    cfg = _cfg(masks, maxlocallen=W, max_new_tokens=64, max_position_embeddings=max_pos)
     gpu = DynamicCache(cfg)
     cpu = OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
     r = np.random.default_rng(21)
@@ -139,6 +140,8 @@ def test_streaming_wraps_the_window_buffer_and_crosses_pages():
         err = np.abs(got - cpu.attend(q, kw, vw, 0, Hq, Hkv)).max()
         assert err <= 2e-2 and err <= 1e-3, (s, err)
     assert gpu._layers[0].n_mid == cpu.key_cache[0]["k_uncompressed"].shape[1] == prompt - 4 - W + steps > 96   # pages crossed
+    if max_pos == 100:
+        assert gpu._layers[0].k.mid.cap_tokens > 96      # it grew
 
 
 def test_short_prompt_stays_in_window_and_matches_exact_attention():
