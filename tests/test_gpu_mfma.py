@@ -123,6 +123,42 @@ def test_mfma_softmax_reference_moves(shape):
     assert err <= 8e-3, err        # sharply peaked softmax: the bf16 probabilities dominate
 
 
+def test_mfma_random_shapes_agree_with_the_generic_kernels():
+    """Seeded random geometry (batch 1-9, 1-4 KV heads, grouping 1-8, head_dim 64 / 128, 128-1024 frequencies,
+    ragged per-head masks, odd sink / window / prompt lengths): the matrix-core path against the plain kernels."""
+    from fourierattention_amd import DynamicCache
+    rng = np.random.default_rng(2024)
+    for case in range(16):
+        dtype = [torch.bfloat16, torch.float16][rng.integers(2)]
+        D = [64, 128][rng.integers(2)]
+        Hkv = int(rng.integers(1, 5)); G = int([1, 2, 3, 4, 6, 8][rng.integers(6)]); Hq = Hkv * G
+        B = int(rng.integers(1, 10)); I = int(rng.integers(0, 6)); W = int(rng.integers(1, 70))
+        M = int([256, 512, 1024, 2048][rng.integers(4)])
+        prompt = int(I + W + M + rng.integers(1, 1500))
+        kc = [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)]
+        vc = [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)]
+        tag = f"case {case}: {dtype} B={B} Hq={Hq} Hkv={Hkv} D={D} I={I} W={W} M={M} prompt={prompt} k={kc} v={vc}"
+        print(tag, flush=True)
+        masks = _masks(1, Hkv, D, kc, vc, seed=case)
+        cfg = _cfg(masks, numinittokens=I, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=8,
+                   max_position_embeddings=1 << 20)
+        gpu = DynamicCache(cfg)
+        g = torch.Generator(device="cuda").manual_seed(case)
+        rn = lambda *sh: torch.randn(*sh, generator=g, device="cuda")
+        gpu.update(rn(B, Hkv, prompt, D).to(dtype), rn(B, Hkv, prompt, D).to(dtype), 0)
+        assert gpu._tables is not None, tag
+        for _ in range(2):
+            gpu.update(rn(B, Hkv, 1, D).to(dtype), rn(B, Hkv, 1, D).to(dtype), 0)
+            q = (rn(B, Hq, 1, D) * 1.5).to(dtype)
+            got = gpu.decode_attention(q, 0, Hq, Hkv)
+            gpu.force_generic = True
+            ref = gpu.decode_attention(q, 0, Hq, Hkv)
+            gpu.force_generic = False
+            assert torch.isfinite(got).all(), tag
+            err = (got - ref).abs().max().item()
+            assert err <= 5e-3, (tag, err)
+
+
 def test_full_size_properties():
     """BASELINE config 3 at full size (B=8, 32k context): properties that need no CPU oracle.
     (1) the matrix-core path and the generic path (independent kernels, each checked against the oracle at
