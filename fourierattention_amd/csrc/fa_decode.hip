@@ -488,7 +488,7 @@ __device__ __forceinline__ float weighted_sum(const float* __restrict__ ptr, int
   return a;
 }
 
-constexpr int kMergeChunks = 4;  // blocks per (b, KV head): each applies the V coefficients of a quarter of the dims
+constexpr int kMergeChunksMax = 8;  // blocks per (b, KV head): each applies the V coefficients of its share of the dims
 
 __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
@@ -512,14 +512,14 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   float* s_o = s_part + 1024 * G;        // [G][D]
   int* s_own = (int*)(s_o + G * D);      // [D]: bit 0 = some list holds the dim, bit 1 = this block writes it
   const int tid = threadIdx.x;
-  const int h = blockIdx.x, b = blockIdx.y, z = blockIdx.z;
+  const int h = blockIdx.x, b = blockIdx.y, z = blockIdx.z, n_chunks = gridDim.z;
   const int64_t r0 = (int64_t)b * Hq + h * G;
   const int vc0 = vc_h[h], vc_len = vc_h[h + 1] - vc0;
   const int vn0 = vn_h[h], vn_len = vn_h[h + 1] - vn0;
   // this block's share of the compressed and of the stored dims (by position in the head's lists)
-  const int cw = (vc_len + kMergeChunks - 1) / kMergeChunks;
+  const int cw = (vc_len + n_chunks - 1) / n_chunks;
   const int c_lo = min(vc_len, z * cw), cn = min(vc_len, c_lo + cw) - c_lo;
-  const int nw = (vn_len + kMergeChunks - 1) / kMergeChunks;
+  const int nw = (vn_len + n_chunks - 1) / n_chunks;
   const int n_lo = min(vn_len, z * nw), nn = min(vn_len, n_lo + nw) - n_lo;
   const bool has_coef = n_mid_split > 0 && cn > 0;
   int cwp = 1;                           // power of two >= cw: threads = (dim, row class)
@@ -995,7 +995,9 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_mg = take((mfma ? (size_t)p.n_groups * Hkv * 16 : rows) * p.n_mid_split * 2 * N * 4);
   p.off_mon = take(rows * p.n_mid_split * D * 4);
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
-  p.n_merge_chunks = 1;
+  // merge: as many blocks per (b, KV head) as still run side by side on the device (a block fills one compute unit)
+  p.n_merge_chunks = kMergeChunksMax;
+  while (p.n_merge_chunks > 1 && (int64_t)B * Hkv * p.n_merge_chunks > device_cu_count()) p.n_merge_chunks >>= 1;
   p.off_cpart = take(256);
   // two-pass mid rows (eight frequency slices): the scores of every page travel through memory
   p.off_scores = take(mfma && fa_mfma::table_slices(N) > 4 ? (size_t)p.n_groups * Hkv * fa_cdiv(L_m, 32) * 512 * 4 : 0);
@@ -1165,7 +1167,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
     }
-    decode_merge_kernel<<<dim3(a.Hkv, a.B, kMergeChunks), 1024, lds, st>>>(
+    decode_merge_kernel<<<dim3(a.Hkv, a.B, p.n_merge_chunks), 1024, lds, st>>>(
         ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
         a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv,
         p.path == Path::Mfma ? p.nbpg : 0);
