@@ -538,7 +538,10 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   // g partials: two neighbouring threads share four consecutive coefficient rows of one head, one takes the even
   // splits, the other the odd ones (16-byte loads: a quarter of the load instructions of a row-per-thread map)
   constexpr int kGPre = kMergePre / 2;
-  const int g_items = G * 2 * N / 4;                 // 2N is a multiple of 4
+  // (a row-per-head g whose rows of 2N values are not multiples of 16 bytes is read value by value: E4 = 1)
+  const int E4 = (g_nbpg > 0 || (2 * N) % 4 == 0) ? 4 : 1;
+  const int g_items = G * (2 * N / E4);
+  auto g_load = [&](const float* ptr) { return E4 == 4 ? *(const float4*)ptr : make_float4(*ptr, 0.f, 0.f, 0.f); };
   const int g_item = tid >> 1, g_half = tid & 1;
   const int64_t g_split_stride = g_nbpg > 0 ? (int64_t)16 * 2 * N : (int64_t)2 * N;
   // item -> (query head g, group of four values n4) and the address of its values in split 0
@@ -549,16 +552,16 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
       const int grp = b / g_nbpg, lc = (b - grp * g_nbpg) * G + g;
       return md_g + (int64_t)(grp * Hkv + h) * n_mid_split * g_split_stride + (int64_t)(n4 >> 2) * 256 + (lc * 4 + (n4 & 3)) * 4;
     }
-    g = item / (2 * N / 4);
-    n4 = item - g * (2 * N / 4);
-    return md_g + (r0 + g) * n_mid_split * 2 * N + 4 * n4;
+    g = item / (2 * N / E4);
+    n4 = item - g * (2 * N / E4);
+    return md_g + (r0 + g) * n_mid_split * 2 * N + E4 * n4;
   };
   float4 g_pre[kGPre];
   if (has_coef && g_item < g_items) {
     int g, n4;
     const float* gp = g_locate(g_item, g, n4);
 #pragma unroll
-    for (int u = 0; u < kGPre; ++u) g_pre[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * u, n_mid_split - 1) * g_split_stride);
+    for (int u = 0; u < kGPre; ++u) g_pre[u] = g_load(gp + (int64_t)min(g_half + 2 * u, n_mid_split - 1) * g_split_stride);
   }
   // V coefficients: rows part, part + parts, ... of dim c_lo + j
   const int j = tid & (cwp - 1), part = tid / cwp;
@@ -651,7 +654,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
           float4 v[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u)
-            v[u] = *(const float4*)(gp + (int64_t)min(g_half + 2 * (u0 + u), n_mid_split - 1) * g_split_stride);
+            v[u] = g_load(gp + (int64_t)min(g_half + 2 * (u0 + u), n_mid_split - 1) * g_split_stride);
 #pragma unroll
           for (int u = 0; u < 4; ++u) fold1(v[u], g_half + 2 * (u0 + u), wg, a);
         }
@@ -661,8 +664,10 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
           if (g_nbpg > 0) {   // {cos f, sin f, cos f+1, sin f+1} with f = 2 * n4
             *(float2*)(s_g + g * 2 * N + 2 * n4) = make_float2(a.x, a.z);
             *(float2*)(s_g + g * 2 * N + N + 2 * n4) = make_float2(a.y, a.w);
-          } else {
+          } else if (E4 == 4) {
             *(float4*)(s_g + g * 2 * N + 4 * n4) = a;
+          } else {
+            s_g[g * 2 * N + n4] = a.x;
           }
         }
       }

@@ -107,6 +107,9 @@ CASES = [
     (1, 6, 2, 128, 5, 700, 24, 733, [0, 128], [128, 1]),          # heads with nothing / everything compressed
     (3, 4, 4, 32, 260, 513, 8, 600, [7, 9, 11, 13], [1, 2, 3, 4]),  # MHA, window longer than one tile
     (2, 24, 8, 128, 20, 130, 40, 1000, [64] * 8, [64] * 8),        # 3:1 grouping
+    (2, 4, 2, 64, 9, 150, 3, 200, [10, 50], [33, 64]),             # odd numbers of frequencies: coefficient
+    (1, 6, 2, 32, 70, 90, 5, 97, [31, 2], [5, 32]),                # rows that are no multiple of 16 bytes
+    (1, 2, 1, 32, 3, 40, 1, 64, [16], [16]),
 ]
 
 
