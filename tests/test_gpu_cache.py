@@ -109,14 +109,16 @@ def test_cache_prefill_and_streaming(dtype, prompt, max_new, max_pos, expect_T):
         assert gpu._seen_tokens == cpu._seen_tokens == prompt + s + 1
 
 
-@pytest.mark.parametrize("max_pos", [4096, 100])   # 100: the page store is sized for 96 rows and has to grow on the way
-def test_streaming_wraps_the_window_buffer_and_crosses_pages(max_pos):
+# max_pos 100: the page store is sized for 96 rows and has to grow on the way; 6 and 7 states: an odd number of
+# frequencies (coefficient rows that are no multiple of 16 bytes), and a state count that is odd itself
+@pytest.mark.parametrize("max_pos,states", [(4096, 16), (100, 16), (4096, 6), (4096, 7)])
+def test_streaming_wraps_the_window_buffer_and_crosses_pages(max_pos, states):
     """More decode steps than the window buffer has slots (the write / evict slots wrap around several times)
     and enough evicted rows to cross page boundaries of the mid store: parts and attention after every step."""
     from fourierattention_amd import DynamicCache
     dtype, B, Hq, Hkv, D, W, prompt, steps = torch.bfloat16, 2, 4, 2, 64, 8, 90, 41
     masks = _masks(1, Hkv, D, [40, 17], [64, 0], seed=5)
-    cfg = _cfg(masks, maxlocallen=W, max_new_tokens=64, max_position_embeddings=max_pos)
+    cfg = _cfg(masks, maxlocallen=W, max_new_tokens=64, max_position_embeddings=max_pos, maxmidstates=states)
     gpu = DynamicCache(cfg)
     cpu = OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
     r = np.random.default_rng(21)
