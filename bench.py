@@ -202,6 +202,7 @@ def e2e_bench(name, device, steps=None, warmup=3):
                      non_critical_dims_path=None, max_position_embeddings=1 << 20,
                      num_key_value_heads=cfg.num_key_value_heads, max_new_tokens=e["new"] + warmup + 8, model_type="llama")
     model = random_init(cfg, torch.bfloat16, device, seed=0)
+    model.model.fuse_projections()
     cache = DynamicCache(ec, device=device)
     t0 = time.perf_counter()
     synthetic_prefill(cache, cfg, e["B"], e["prompt"], torch.bfloat16, device, seed=0)

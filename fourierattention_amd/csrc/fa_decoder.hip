@@ -86,14 +86,17 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(E* __restrict__ h, con
   }
 }
 
-// grid (rows, Hq + Hkv), block D / 2: x <- x * cos + rotate_half(x) * sin on one head of q or k
+// grid (rows, Hq + Hkv), block D / 2: x <- x * cos + rotate_half(x) * sin on one head of q or k.  The rows of
+// q_in and k may be slices of wider rows (a fused projection output); q goes out densely packed (q_out may be
+// q_in when that is dense), k in place.
 template <typename E>
-__global__ void rope_qk_kernel(E* __restrict__ q, E* __restrict__ k, const E* __restrict__ cs, const E* __restrict__ sn,
-                               int Hq, int Hkv, int D) {
+__global__ void rope_qk_kernel(const E* q_in, int64_t q_stride, E* q_out, E* k, int64_t k_stride,
+                               const E* __restrict__ cs, const E* __restrict__ sn, int Hq, int Hkv, int D) {
   const int64_t row = blockIdx.x;
   const int head = blockIdx.y, i = threadIdx.x, half = D >> 1;
-  E* x = head < Hq ? q + (row * Hq + head) * D : k + (row * Hkv + (head - Hq)) * D;
-  const float x1 = fa_to_float(x[i]), x2 = fa_to_float(x[i + half]);
+  const E* src = head < Hq ? q_in + row * q_stride + head * D : k + row * k_stride + (head - Hq) * D;
+  E* x = head < Hq ? q_out + (row * Hq + head) * D : k + row * k_stride + (head - Hq) * D;
+  const float x1 = fa_to_float(src[i]), x2 = fa_to_float(src[i + half]);
   const float c1 = fa_to_float(cs[row * D + i]), c2 = fa_to_float(cs[row * D + i + half]);
   const float s1 = fa_to_float(sn[row * D + i]), s2 = fa_to_float(sn[row * D + i + half]);
   // rotate_half(x) = (-x2, x1)
@@ -101,13 +104,15 @@ __global__ void rope_qk_kernel(E* __restrict__ q, E* __restrict__ k, const E* __
   x[i + half] = Rounder<E>::put(rnd<E>(x2 * c2) + rnd<E>(x1 * s2));
 }
 
+// grid (column blocks, rows): gate and up rows may be slices of wider rows (a fused projection output)
 template <typename E>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const E* __restrict__ gate, const E* __restrict__ up,
-                                                        E* __restrict__ out, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  const float g = fa_to_float(gate[i]);
-  out[i] = Rounder<E>::put(rnd<E>(g / (1.0f + expf(-g))) * fa_to_float(up[i]));
+                                                        E* __restrict__ out, int cols, int64_t in_stride) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= cols) return;
+  const int64_t row = blockIdx.y;
+  const float g = fa_to_float(gate[row * in_stride + i]);
+  out[row * cols + i] = Rounder<E>::put(rnd<E>(g / (1.0f + expf(-g))) * fa_to_float(up[row * in_stride + i]));
 }
 
 template <typename F>
@@ -139,28 +144,35 @@ extern "C" int fa_add_rmsnorm(void* h, const void* delta, const void* weight, vo
   return rc != FA_OK ? rc : fa_check_launch("fa_add_rmsnorm");
 }
 
-extern "C" int fa_rope_qk(void* q, void* k, const void* cos, const void* sin, int rows, int Hq, int Hkv, int D, int dtype,
-                          fa_stream_t stream) {
-  FA_REQUIRE(q && k && cos && sin, FA_ERR_NULL_POINTER, "fa_rope_qk: null pointer");
+extern "C" int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, void* k, int64_t k_stride, const void* cos,
+                          const void* sin, int rows, int Hq, int Hkv, int D, int dtype, fa_stream_t stream) {
+  FA_REQUIRE(q_in && q_out && k && cos && sin, FA_ERR_NULL_POINTER, "fa_rope_qk: null pointer");
   FA_REQUIRE(rows >= 0 && Hq > 0 && Hkv > 0 && D > 0 && D % 2 == 0 && D <= 2048, FA_ERR_BAD_SHAPE,
              "fa_rope_qk: rows=%d Hq=%d Hkv=%d D=%d", rows, Hq, Hkv, D);
+  FA_REQUIRE(q_in_stride >= (int64_t)Hq * D && k_stride >= (int64_t)Hkv * D, FA_ERR_BAD_SHAPE,
+             "fa_rope_qk: row strides %lld, %lld shorter than the rows", (long long)q_in_stride, (long long)k_stride);
+  FA_REQUIRE(q_out != q_in || q_in_stride == (int64_t)Hq * D, FA_ERR_BAD_SHAPE,
+             "fa_rope_qk: in place needs densely packed q rows");
   if (rows == 0) return FA_OK;
   hipStream_t st = fa_hip_stream(stream);
   int rc = by_dtype(dtype, "fa_rope_qk", [&](auto tag) {
     using E = decltype(tag);
-    rope_qk_kernel<E><<<dim3(rows, Hq + Hkv), D / 2, 0, st>>>((E*)q, (E*)k, (const E*)cos, (const E*)sin, Hq, Hkv, D);
+    rope_qk_kernel<E><<<dim3(rows, Hq + Hkv), D / 2, 0, st>>>((const E*)q_in, q_in_stride, (E*)q_out, (E*)k, k_stride,
+                                                              (const E*)cos, (const E*)sin, Hq, Hkv, D);
   });
   return rc != FA_OK ? rc : fa_check_launch("fa_rope_qk");
 }
 
-extern "C" int fa_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, fa_stream_t stream) {
+extern "C" int fa_silu_mul(const void* gate, const void* up, void* out, int rows, int cols, int64_t in_stride, int dtype,
+                           fa_stream_t stream) {
   FA_REQUIRE(gate && up && out, FA_ERR_NULL_POINTER, "fa_silu_mul: null pointer");
-  FA_REQUIRE(n >= 0, FA_ERR_BAD_SHAPE, "fa_silu_mul: n=%lld", (long long)n);
-  if (n == 0) return FA_OK;
+  FA_REQUIRE(rows >= 0 && cols >= 0 && rows <= 65535 && in_stride >= cols, FA_ERR_BAD_SHAPE,
+             "fa_silu_mul: rows=%d cols=%d stride=%lld", rows, cols, (long long)in_stride);
+  if (rows == 0 || cols == 0) return FA_OK;
   hipStream_t st = fa_hip_stream(stream);
   int rc = by_dtype(dtype, "fa_silu_mul", [&](auto tag) {
     using E = decltype(tag);
-    silu_mul_kernel<E><<<fa_cdiv(n, 256), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out, n);
+    silu_mul_kernel<E><<<dim3(fa_cdiv(cols, 256), rows), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out, cols, in_stride);
   });
   return rc != FA_OK ? rc : fa_check_launch("fa_silu_mul");
 }

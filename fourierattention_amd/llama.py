@@ -102,6 +102,23 @@ class LlamaDecoderLayer(nn.Module):
         self.mlp = LlamaMLP(config)
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+        self._qkv_weight = self._gate_up_weight = None
+
+    def fuse_projections(self):
+        """Moves the q/k/v weights into one tensor and the gate/up weights into another; the five modules keep
+        views of them (same values, same state dict), ``forward_fused`` runs one GEMM per group.  A decode step
+        reads every weight once, so five short launches become two that stream the same bytes."""
+        at, mlp = self.self_attn, self.mlp
+        if at.q_proj.bias is not None or mlp.gate_proj.bias is not None:
+            return
+        for name, mods in (("_qkv_weight", (at.q_proj, at.k_proj, at.v_proj)), ("_gate_up_weight", (mlp.gate_proj, mlp.up_proj))):
+            fused = torch.cat([m.weight.data for m in mods], dim=0)
+            row = 0
+            for m in mods:
+                n = m.weight.shape[0]
+                m.weight.data = fused[row:row + n]
+                row += n
+            setattr(self, name, fused)
 
     def forward(self, hidden_states, position_embeddings, past_key_value, cache_position=None):
         h, _, _ = self.self_attn(self.input_layernorm(hidden_states), past_key_value=past_key_value, use_cache=True,
@@ -116,16 +133,24 @@ class LlamaDecoderLayer(nn.Module):
         at = self.self_attn
         y = ops.add_rmsnorm(h, delta, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
         bsz, q_len, _ = y.shape
-        q, k, v = at.q_proj(y), at.k_proj(y), at.v_proj(y)
+        if self._qkv_weight is not None:
+            nq, nk = at.num_heads * at.head_dim, at.num_key_value_heads * at.head_dim
+            q, k, v = F.linear(y, self._qkv_weight).split((nq, nk, nk), dim=-1)
+        else:
+            q, k, v = at.q_proj(y), at.k_proj(y), at.v_proj(y)
         cos, sin = position_embeddings
-        ops.rope_qk_(q, k, cos, sin, at.head_dim)
+        q = ops.rope_qk(q, k, cos, sin, at.head_dim)
         split = lambda t, n: t.view(bsz, q_len, n, at.head_dim).transpose(1, 2)
         o = fourier_attention(split(q, at.num_heads), split(k, at.num_key_value_heads), split(v, at.num_key_value_heads),
                               past_key_value, at.layer_idx, at.num_heads, at.num_key_value_heads,
                               {"sin": sin, "cos": cos, "cache_position": cache_position})
         y = ops.add_rmsnorm(h, at.o_proj(o), self.post_attention_layernorm.weight,
                             self.post_attention_layernorm.variance_epsilon)
-        return self.mlp.down_proj(ops.silu_mul(self.mlp.gate_proj(y), self.mlp.up_proj(y)))
+        if self._gate_up_weight is not None:
+            gate, up = F.linear(y, self._gate_up_weight).chunk(2, dim=-1)
+        else:
+            gate, up = self.mlp.gate_proj(y), self.mlp.up_proj(y)
+        return self.mlp.down_proj(ops.silu_mul(gate, up))
 
 
 class LlamaModel(nn.Module):
@@ -139,6 +164,11 @@ class LlamaModel(nn.Module):
         # on the GPU: residual add + RMSNorm, rotary embedding and the SwiGLU gate as one launch each (same
         # arithmetic and rounding points as the module chain below); False keeps the chain of tensor ops
         self.fused_elementwise = True
+
+    def fuse_projections(self):
+        for layer in self.layers:
+            layer.fuse_projections()
+        return self
 
     def forward(self, input_ids, past_key_values: DynamicCache, position_ids=None):
         """A cache object is required (modeling_llama_fourier.py:946-949 would otherwise build one without

@@ -232,26 +232,52 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     return y
 
 
-def rope_qk_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, head_dim: int) -> None:
-    """Rotary embedding in place on ``q (B, q_len, Hq*D)`` and ``k (B, q_len, Hkv*D)`` (the projection outputs);
-    ``cos, sin (B or 1, q_len, D)`` (modeling_llama_fourier.py:213-244)."""
+def _row_sliced(t: torch.Tensor) -> bool:
+    """(B, q_len, width) whose rows are evenly spaced slices of wider rows (or dense)."""
+    return t.dim() == 3 and t.stride(2) == 1 and (t.shape[1] == 1 or t.stride(0) == t.shape[1] * t.stride(1))
+
+
+def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, head_dim: int) -> torch.Tensor:
+    """Rotary embedding of ``q (B, q_len, Hq*D)`` and ``k (B, q_len, Hkv*D)`` (the projection outputs, possibly
+    column slices of one fused projection output); ``cos, sin (B or 1, q_len, D)`` (modeling_llama_fourier.py:213-244).
+    ``k`` is rotated in place; the rotated ``q`` is returned densely packed (``q`` itself when it was dense)."""
     _require_gpu(q, "q")
-    assert q.is_contiguous() and k.is_contiguous() and q.dtype == k.dtype
+    assert _row_sliced(q) and _row_sliced(k) and q.dtype == k.dtype
     rows = q.shape[0] * q.shape[1]
     if cos.shape[0] != q.shape[0]:
         cos, sin = cos.expand(q.shape[0], -1, -1), sin.expand(q.shape[0], -1, -1)
     cos, sin = cos.to(q.dtype).contiguous(), sin.to(q.dtype).contiguous()
-    check(_lib.load().fa_rope_qk(q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, q.shape[2] // head_dim,
-                                 k.shape[2] // head_dim, head_dim, dtype_code(q.dtype), _stream(q.device)))
+    q_out = q if q.is_contiguous() else torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    qs = q.stride(1) if q.shape[1] > 1 else q.stride(0)
+    ks = k.stride(1) if k.shape[1] > 1 else k.stride(0)
+    check(_lib.load().fa_rope_qk(q.data_ptr(), qs, q_out.data_ptr(), k.data_ptr(), ks, cos.data_ptr(), sin.data_ptr(), rows,
+                                 q.shape[2] // head_dim, k.shape[2] // head_dim, head_dim, dtype_code(q.dtype),
+                                 _stream(q.device)))
+    return q_out
+
+
+def rope_qk_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, head_dim: int) -> None:
+    """``rope_qk`` in place on densely packed ``q`` and ``k``."""
+    assert q.is_contiguous() and k.is_contiguous()
+    rope_qk(q, k, cos, sin, head_dim)
 
 
 def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """``silu(gate) * up`` in one launch (modeling_llama_fourier.py:277)."""
+    """``silu(gate) * up`` in one launch (modeling_llama_fourier.py:277); ``gate, up (..., cols)`` dense or column
+    slices of one fused projection output (rows evenly spaced, the same spacing for both); the result is dense."""
     _require_gpu(gate, "gate")
-    assert gate.is_contiguous() and up.is_contiguous() and gate.shape == up.shape and gate.dtype == up.dtype
-    out = torch.empty_like(gate)
-    check(_lib.load().fa_silu_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), dtype_code(gate.dtype),
-                                  _stream(gate.device)))
+    assert gate.shape == up.shape and gate.dtype == up.dtype and gate.stride() == up.stride() and gate.stride(-1) == 1
+    cols = gate.shape[-1]
+    rows = gate.numel() // max(cols, 1)
+    stride = gate.stride(-2) if gate.dim() >= 2 and rows > 1 else cols
+    assert all(gate.shape[d] == 1 or gate.stride(d) == gate.stride(d + 1) * gate.shape[d + 1] for d in range(gate.dim() - 2)), \
+        "rows are not evenly spaced"
+    out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    es = gate.element_size()
+    for r0 in range(0, rows, 65535):   # the row index is the launch's second grid dimension
+        check(_lib.load().fa_silu_mul(gate.data_ptr() + r0 * stride * es, up.data_ptr() + r0 * stride * es,
+                                      out.data_ptr() + r0 * cols * es, min(65535, rows - r0), cols, stride,
+                                      dtype_code(gate.dtype), _stream(gate.device)))
     return out
 
 

@@ -281,15 +281,23 @@ int fa_decode_attn_timed(const fa_decode_args* args, fa_stream_t stream, float* 
 int fa_add_rmsnorm(void* h, const void* delta, const void* weight, void* y, int rows, int hidden,
                    float eps, int dtype, fa_stream_t stream);
 
-/* apply_rotary_pos_emb (MODEL:213-244) in place: x <- x * cos + rotate_half(x) * sin
- * on every head of q (rows, Hq * D) and k (rows, Hkv * D); cos, sin: (rows, D) in
- * `dtype`.  Products and sum are rounded to `dtype` one by one like the tensor ops. */
-int fa_rope_qk(void* q, void* k, const void* cos, const void* sin, int rows, int Hq, int Hkv, int D,
-               int dtype, fa_stream_t stream);
+/* apply_rotary_pos_emb (MODEL:213-244): x <- x * cos + rotate_half(x) * sin on every
+ * head of q and k; cos, sin: (rows, D) in `dtype`.  Products and sum are rounded to
+ * `dtype` one by one like the tensor ops.  Row r of q is read at q_in + r * q_in_stride
+ * (Hq * D elements; the rows may be slices of a wider fused projection output) and
+ * written to q_out as (rows, Hq * D) densely packed; q_out may be q_in when q_in is
+ * densely packed itself.  k: row r at k + r * k_stride, Hkv * D elements, in place.
+ * Strides in elements. */
+int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, void* k, int64_t k_stride,
+               const void* cos, const void* sin, int rows, int Hq, int Hkv, int D, int dtype,
+               fa_stream_t stream);
 
 /* act_fn(gate_proj(x)) * up_proj(x) of LlamaMLP.forward (MODEL:277) with
- * act_fn = silu: out[i] = silu(gate[i]).to(dtype) * up[i], n elements. */
-int fa_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, fa_stream_t stream);
+ * act_fn = silu: out[r][i] = silu(gate[r][i]).to(dtype) * up[r][i]; gate and up rows
+ * in_stride elements apart (slices of a fused projection output, or in_stride = cols),
+ * out (rows, cols) densely packed; rows <= 65535. */
+int fa_silu_mul(const void* gate, const void* up, void* out, int rows, int cols, int64_t in_stride,
+                int dtype, fa_stream_t stream);
 
 #ifdef __cplusplus
 }

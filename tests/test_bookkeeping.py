@@ -151,10 +151,13 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_add_rmsnorm(p, None, p, p, 1, 9000, 1e-5, 0, None) == -2     # rows longer than 8192
     assert lib.fa_add_rmsnorm(p, None, p, p, 1, 64, 1e-5, 5, None) == -3
     assert lib.fa_add_rmsnorm(p, None, p, p, 0, 64, 1e-5, 0, None) == 0         # nothing to do
-    assert lib.fa_rope_qk(p, None, p, p, 1, 4, 2, 64, 0, None) == -1
-    assert lib.fa_rope_qk(p, p, p, p, 1, 4, 2, 63, 0, None) == -2              # odd head_dim
-    assert lib.fa_silu_mul(p, p, None, 8, 0, None) == -1
-    assert lib.fa_silu_mul(p, p, p, -1, 0, None) == -2
+    assert lib.fa_rope_qk(p, 256, p, None, 128, p, p, 1, 4, 2, 64, 0, None) == -1
+    assert lib.fa_rope_qk(p, 252, p, p, 126, p, p, 1, 4, 2, 63, 0, None) == -2    # odd head_dim
+    assert lib.fa_rope_qk(p, 255, p, p, 128, p, p, 1, 4, 2, 64, 0, None) == -2    # stride shorter than a row
+    assert lib.fa_rope_qk(p, 512, p, p, 128, p, p, 1, 4, 2, 64, 0, None) == -2    # in place on sliced rows
+    assert lib.fa_silu_mul(p, p, None, 1, 8, 8, 0, None) == -1
+    assert lib.fa_silu_mul(p, p, p, -1, 8, 8, 0, None) == -2
+    assert lib.fa_silu_mul(p, p, p, 2, 8, 4, 0, None) == -2                        # stride shorter than a row
     assert lib.fa_stream_update(None, None) == -1
     sa = _lib.StreamArgs()
     assert lib.fa_stream_update(ctypes.byref(sa), None) == -2                  # empty shape

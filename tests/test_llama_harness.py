@@ -47,6 +47,32 @@ def test_greedy_loop_matches_full_recompute_cpu():
     torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4)
 
 
+def test_fused_projection_weights_keep_modules_and_state_dict():
+    """After ``fuse_projections`` the five projection modules are views of two wider tensors: same values, the
+    module chain computes the same logits, and a state dict loaded afterwards lands in the fused tensors."""
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import random_init
+    cfg = _tiny()
+    model = random_init(cfg, dtype=torch.float32, device="cpu", seed=3, std=0.3)
+    other = random_init(cfg, dtype=torch.float32, device="cpu", seed=4, std=0.3)
+    masks = _masks(cfg.num_hidden_layers, cfg.num_key_value_heads, cfg.head_dim, [8, 8], [8, 8])
+    ec = lambda: _cfg(masks, numinittokens=2, maxlocallen=64, maxmidstates=8, num_key_value_heads=cfg.num_key_value_heads,
+                      max_new_tokens=16, max_position_embeddings=256)
+    ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(0))
+    want = model(input_ids=ids, past_key_values=DynamicCache(ec(), device="cpu")).logits
+    sd = {k: v.clone() for k, v in model.state_dict().items()}
+    model.model.fuse_projections()
+    assert all(torch.equal(v, sd[k]) for k, v in model.state_dict().items())
+    assert torch.equal(model(input_ids=ids, past_key_values=DynamicCache(ec(), device="cpu")).logits, want)
+    layer = model.model.layers[1]
+    at, mlp = layer.self_attn, layer.mlp
+    assert torch.equal(layer._qkv_weight, torch.cat([at.q_proj.weight, at.k_proj.weight, at.v_proj.weight]))
+    assert torch.equal(layer._gate_up_weight, torch.cat([mlp.gate_proj.weight, mlp.up_proj.weight]))
+    model.load_state_dict(other.state_dict())
+    assert torch.equal(layer._qkv_weight[-at.v_proj.weight.shape[0]:], other.model.layers[1].self_attn.v_proj.weight)
+    assert torch.equal(layer._gate_up_weight[:mlp.gate_proj.weight.shape[0]], other.model.layers[1].mlp.gate_proj.weight)
+
+
 def test_model_requires_a_cache():
     from fourierattention_amd.llama import random_init
     model = random_init(_tiny(layers=1), dtype=torch.float32, device="cpu")
@@ -165,10 +191,20 @@ def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
     q2, k2 = q.clone(), k.clone()
     ops.rope_qk_(q2, k2, cos, sin, D)
     assert torch.equal(q2.view(B, q_len, Hq, D).transpose(1, 2), wq) and torch.equal(k2.view(B, q_len, Hkv, D).transpose(1, 2), wk)
+    # the same on column slices of one fused projection output: q comes back densely packed, k is rotated where it lies
+    qkv = torch.cat([q, k, rn(B, q_len, Hkv * D).to(dtype)], dim=-1)
+    qs, ks, vs = qkv.split((Hq * D, Hkv * D, Hkv * D), dim=-1)
+    v_before = vs.clone()
+    q3 = ops.rope_qk(qs, ks, cos, sin, D)
+    assert q3.is_contiguous() and torch.equal(q3, q2) and torch.equal(ks, k2) and torch.equal(vs, v_before)
     # SwiGLU gate: the exponential may differ in the last place
     gate, up = (rn(7, 1, 1111) * 3).to(dtype), rn(7, 1, 1111).to(dtype)
     want = torch.nn.functional.silu(gate) * up
-    torch.testing.assert_close(ops.silu_mul(gate, up).float(), want.float(), rtol=2 * ulp, atol=2 * ulp)
+    got = ops.silu_mul(gate, up)
+    torch.testing.assert_close(got.float(), want.float(), rtol=2 * ulp, atol=2 * ulp)
+    g2, u2 = torch.cat([gate, up], dim=-1).chunk(2, dim=-1)              # column slices of one wider row
+    got2 = ops.silu_mul(g2, u2)
+    assert got2.is_contiguous() and torch.equal(got2, got)
 
 
 @pytest.mark.gpu
@@ -185,8 +221,14 @@ def test_fused_decoder_path_matches_the_module_chain():
     ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(3)).cuda()
     outs = []
     with torch.no_grad():
-        for fused in (True, False):
-            model.model.fused_elementwise = fused
+        for fused in (True, False, "projections"):
+            model.model.fused_elementwise = bool(fused)
+            if fused == "projections":       # q/k/v and gate/up as one GEMM each; the modules keep views of the weights
+                before = {n: p.detach().clone() for n, p in model.named_parameters()}
+                model.model.fuse_projections()
+                assert all(torch.equal(p, before[n]) for n, p in model.named_parameters())
+                at = model.model.layers[0].self_attn
+                assert at.k_proj.weight.data_ptr() == at.q_proj.weight.data_ptr() + at.q_proj.weight.numel() * 2
             cache = DynamicCache(ec())
             logits = [model(input_ids=ids, past_key_values=cache, num_logits_to_keep=1).logits[:, -1]]
             tok = logits[0].argmax(-1, keepdim=True)
@@ -197,3 +239,6 @@ def test_fused_decoder_path_matches_the_module_chain():
     # identical rounding points; only reduction order (norm) and the exponential differ in the last place of bf16
     torch.testing.assert_close(outs[0], outs[1], rtol=3e-2, atol=3e-2)
     assert (outs[0] - outs[1]).abs().mean().item() < 3e-3
+    # a wider GEMM may pick another tiling, hence another summation order inside the dot products
+    torch.testing.assert_close(outs[2], outs[0], rtol=3e-2, atol=3e-2)
+    assert (outs[2] - outs[0]).abs().mean().item() < 3e-3
