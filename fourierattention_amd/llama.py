@@ -104,14 +104,19 @@ class LlamaDecoderLayer(nn.Module):
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self._qkv_weight = self._gate_up_weight = None
 
-    def fuse_projections(self):
+    def fuse_projections(self, max_rows: int = 16384):
         """Moves the q/k/v weights into one tensor and the gate/up weights into another; the five modules keep
         views of them (same values, same state dict), ``forward_fused`` runs one GEMM per group.  A decode step
-        reads every weight once, so five short launches become two that stream the same bytes."""
+        reads every weight once, so five short launches become two that stream the same bytes.  A group whose
+        fused weight would have more than ``max_rows`` rows stays as it is: for a handful of tokens the GEMM
+        library answers a very wide output with a tile shape that streams the weights at half the rate of the two
+        separate calls (measured at 2 x 14336 rows of 4096)."""
         at, mlp = self.self_attn, self.mlp
         if at.q_proj.bias is not None or mlp.gate_proj.bias is not None:
             return
         for name, mods in (("_qkv_weight", (at.q_proj, at.k_proj, at.v_proj)), ("_gate_up_weight", (mlp.gate_proj, mlp.up_proj))):
+            if sum(m.weight.shape[0] for m in mods) > max_rows:
+                continue
             fused = torch.cat([m.weight.data for m in mods], dim=0)
             row = 0
             for m in mods:
@@ -165,9 +170,9 @@ class LlamaModel(nn.Module):
         # arithmetic and rounding points as the module chain below); False keeps the chain of tensor ops
         self.fused_elementwise = True
 
-    def fuse_projections(self):
+    def fuse_projections(self, max_rows: int = 16384):
         for layer in self.layers:
-            layer.fuse_projections()
+            layer.fuse_projections(max_rows)
         return self
 
     def forward(self, input_ids, past_key_values: DynamicCache, position_ids=None):
