@@ -48,7 +48,7 @@ class DecodeArgs(ctypes.Structure):
         ("kc_list", c_void_p), ("kc_h_list", c_void_p), ("kn_list", c_void_p), ("kn_h_list", c_void_p),
         ("vc_list", c_void_p), ("vc_h_list", c_void_p), ("vn_list", c_void_p), ("vn_h_list", c_void_p),
         ("Ck", c_int32), ("Cnk", c_int32), ("Cv", c_int32), ("Cnv", c_int32),
-        ("out", c_void_p),
+        ("out", c_void_p), ("out_cast", c_void_p),
         ("B", c_int32), ("Hq", c_int32), ("Hkv", c_int32), ("D", c_int32),
         ("q_len", c_int32), ("N", c_int32), ("L_m", c_int32), ("T", c_int32),
         ("sm_scale", c_float), ("dtype", c_int32),

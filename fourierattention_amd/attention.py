@@ -54,12 +54,14 @@ def fourier_attention(query_states: torch.Tensor, key_states: torch.Tensor, valu
     k_parts, v_parts = past_key_value.update(key_states, value_states, layer_idx, cache_kwargs)
     if k_parts["k_init"] is None and k_parts["k_compressed"] is None and k_parts["k_uncompressed"] is None:
         if q_len == 1 and query_states.is_cuda:
-            o = past_key_value.decode_attention(query_states, layer_idx, num_heads, num_key_value_heads)
+            o = past_key_value.decode_attention(query_states, layer_idx, num_heads, num_key_value_heads,
+                                                out_dtype=query_states.dtype)
             o = o.transpose(1, 2)
         else:
             o = _exact_attention(query_states, k_parts["k_local"], v_parts["v_local"], num_key_value_heads, head_dim)
     elif isinstance(k_parts, CacheParts):
-        o = past_key_value.decode_attention(query_states, layer_idx, num_heads, num_key_value_heads).transpose(1, 2)
+        o = past_key_value.decode_attention(query_states, layer_idx, num_heads, num_key_value_heads,
+                                            out_dtype=query_states.dtype).transpose(1, 2)
     else:  # plain tensors in the reference's layout
         pkv = past_key_value
         o = ops.triton_fourier_attn(

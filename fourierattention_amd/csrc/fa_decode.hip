@@ -496,7 +496,17 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ md_on, int n_mid_split, const float* __restrict__ v_mc,
     const float* __restrict__ avg_u, const float* __restrict__ avg_d, const float* __restrict__ scale,
     const int32_t* __restrict__ vc_list, const int32_t* __restrict__ vc_h, const int32_t* __restrict__ vn_list,
-    const int32_t* __restrict__ vn_h, float* __restrict__ out, int Hq, int Hkv, int D, int N, int Cv, int g_nbpg) {
+    const int32_t* __restrict__ vn_h, float* __restrict__ out, void* __restrict__ out_cast, int cast_dtype, int Hq, int Hkv,
+    int D, int N, int Cv, int g_nbpg) {
+  // the result goes out as fp32 (out) and / or rounded to the storage type of the model (out_cast)
+  auto put = [&](int64_t at, float v) {
+    if (out) out[at] = v;
+    if (out_cast) {
+      if (cast_dtype == FA_BF16) ((bf16_t*)out_cast)[at] = bf16_t{fa_f32_to_bf16_bits(v)};
+      else if (cast_dtype == FA_FP16) ((f16_t*)out_cast)[at] = f16_t{(_Float16)v};
+      else ((float*)out_cast)[at] = v;
+    }
+  };
   // g_nbpg > 0: the g partials come from the matrix-core kernel in its own layout, per (batch group of g_nbpg,
   // KV head, split) N/8 tiles of [column][pair of frequencies] x {cos f, sin f, cos f+1, sin f+1},
   // column = (batch element within the group) * G + query head within the KV head; otherwise one row of 2N per
@@ -737,7 +747,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     if ((own & 2) || (z == 0 && own == 0)) {
       float a = s_o[tid];
       if (n_il_split > 0) a += weighted_sum_pre(il_pre, il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
-      out[(r0 + g) * D + d] = a / s_sc[g];
+      put((r0 + g) * D + d, a / s_sc[g]);
     }
   }
   for (int idx = tid + 1024; idx < G * D; idx += 1024) {
@@ -746,7 +756,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     if ((own & 2) || (z == 0 && own == 0)) {
       float a = s_o[idx];
       if (n_il_split > 0) a += weighted_sum(il_o + (r0 + g) * n_il_split * D + d, D, s_w + g * n_all, n_il_split);
-      out[(r0 + g) * D + d] = a / s_sc[g];
+      put((r0 + g) * D + d, a / s_sc[g]);
     }
   }
 }
@@ -1174,7 +1184,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     }
     decode_merge_kernel<<<dim3(a.Hkv, a.B, p.n_merge_chunks), 1024, lds, st>>>(
         ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
-        a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.Hq, a.Hkv, a.D, a.N, a.Cv,
+        a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.out_cast, a.dtype, a.Hq, a.Hkv, a.D, a.N, a.Cv,
         p.path == Path::Mfma ? p.nbpg : 0);
   }
   if (ev) hipEventRecord(ev[4], st);
@@ -1223,7 +1233,7 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
   FA_REQUIRE(a->Hq % a->Hkv == 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: Hq %d not a multiple of Hkv %d", a->Hq, a->Hkv);
   FA_REQUIRE(a->il_rows[0] >= 0 && a->il_rows[1] >= 0 && a->L_m >= 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: negative row count");
   FA_REQUIRE(a->il_rows[0] + a->il_rows[1] + a->L_m > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: no keys");
-  FA_REQUIRE(a->q && a->out, FA_ERR_NULL_POINTER, "fa_decode_attn: q/out null");
+  FA_REQUIRE(a->q && (a->out || a->out_cast), FA_ERR_NULL_POINTER, "fa_decode_attn: q/out null");
   FA_REQUIRE(a->dtype == FA_BF16 || a->dtype == FA_FP16 || a->dtype == FA_FP32, FA_ERR_BAD_DTYPE, "fa_decode_attn: dtype %d", a->dtype);
   for (int i = 0; i < 2; ++i)
     FA_REQUIRE(a->il_rows[i] == 0 || (a->k_il[i] && a->v_il[i]), FA_ERR_NULL_POINTER, "fa_decode_attn: il segment %d null", i);

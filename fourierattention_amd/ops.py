@@ -315,8 +315,9 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
-                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None):
-    """Thin call into ``fa_decode_attn``.
+                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None):
+    """Thin call into ``fa_decode_attn``.  The result is float32 like the reference's (TRI:779) unless ``out_dtype``
+    names the dtype of ``q``: then the merge launch rounds it to that type itself (the caller's ``.to(dtype)``).
 
     ``il_segments``: up to two ``(k, v)`` pairs of ``(B, rows, Hkv*D)`` views (last dim contiguous).
     ``k_mn`` / ``v_mn``: token-major ``(B, >=L_m, Cn)`` tensors or ``MidStore`` objects (paged).
@@ -370,8 +371,14 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()
     a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list = vc.data_ptr(), vc_h.data_ptr(), vn.data_ptr(), vn_h.data_ptr()
     if out is None:
-        out = torch.empty((B, num_head_q, 1, D), device=q.device, dtype=torch.float32)
-    a.out = out.data_ptr()
+        cast = out_dtype is not None and out_dtype != torch.float32
+        assert not cast or out_dtype == q.dtype, "out_dtype must be float32 or the dtype of q"
+        out = torch.empty((B, num_head_q, 1, D), device=q.device, dtype=q.dtype if cast else torch.float32)
+    if out.dtype == torch.float32:
+        a.out = out.data_ptr()
+    else:
+        assert out.dtype == q.dtype and out.is_contiguous()
+        a.out_cast = out.data_ptr()
     a.B, a.Hq, a.Hkv, a.D = B, num_head_q, num_head_kv, D
     a.q_len, a.N, a.L_m, a.T = q_len, N, int(seq_len_m), int(T)
     a.sm_scale = float(sm_scale)

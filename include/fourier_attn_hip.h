@@ -192,8 +192,11 @@ typedef struct fa_decode_args {
   const int32_t* vc_list; const int32_t* vc_h_list;
   const int32_t* vn_list; const int32_t* vn_h_list;
   int32_t Ck, Cnk, Cv, Cnv;
-  /* output (B, Hq, 1, D) fp32 contiguous (TRI:779) */
+  /* output (B, Hq, 1, D) contiguous: fp32 in `out` (TRI:779) and / or rounded to `dtype`
+   * in `out_cast` (what the caller's `.to(query_states.dtype)` of MODEL:663 would make of
+   * it); either may be NULL, not both */
   float* out;
+  void* out_cast;
   int32_t B, Hq, Hkv, D;
   int32_t q_len;      /* must be 1 (TRI:692) */
   int32_t N;          /* frequencies = coefficient rows / 2 */

@@ -106,6 +106,9 @@ def test_cache_prefill_and_streaming(dtype, prompt, max_new, max_pos, expect_T):
             got = gpu.decode_attention(H.to_gpu(q, dtype), l, Hq, Hkv)
             err = np.abs(got.cpu().numpy() - want).max()
             assert err <= 2e-2 and err <= 1e-3, err
+            # the same rounded to the model's type by the merge launch itself
+            got16 = gpu.decode_attention(H.to_gpu(q, dtype), l, Hq, Hkv, out_dtype=dtype)
+            assert got16.dtype == dtype and torch.equal(got16, got.to(dtype))
         assert gpu._seen_tokens == cpu._seen_tokens == prompt + s + 1
 
 
