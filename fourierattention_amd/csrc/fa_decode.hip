@@ -957,7 +957,7 @@ struct Plan {
   Path path;
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
   int n_merge_chunks;
-  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_cpart, off_scores, total;
+  size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_scores, total;
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
@@ -1013,7 +1013,6 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   // merge: as many blocks per (b, KV head) as still run side by side on the device (a block fills one compute unit)
   p.n_merge_chunks = kMergeChunksMax;
   while (p.n_merge_chunks > 1 && (int64_t)B * Hkv * p.n_merge_chunks > device_cu_count()) p.n_merge_chunks >>= 1;
-  p.off_cpart = take(256);
   // two-pass mid rows (eight frequency slices): the scores of every page travel through memory
   p.off_scores = take(mfma && fa_mfma::table_slices(N) > 4 ? (size_t)p.n_groups * Hkv * fa_cdiv(L_m, 32) * 512 * 4 : 0);
   p.total = o;
@@ -1078,7 +1077,6 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   float* md = (float*)(ws + p.off_md);
   float* mg = (float*)(ws + p.off_mg);
   float* mon = (float*)(ws + p.off_mon);
-  float* cpart = (float*)(ws + p.off_cpart);
   const int G = a.Hq / a.Hkv;
   const float sm_log2e = sm_scale * kLog2e;
   Seg s0{a.k_il[0], a.v_il[0], a.il_rows[0], a.il_batch_stride[0], a.il_row_stride[0]};
