@@ -31,7 +31,7 @@ def _masks(layers, Hkv, D, kcounts, vcounts, seed=0):
     return out
 
 
-def _compare_parts(kp, kw, tag, dtype):
+def _compare_parts(kp, kw, tag, dtype, coef_tol=2e-5):
     for part in ("init", "compressed", "uncompressed", "local"):
         g, w = kp[f"{tag}_{part}"], kw[f"{tag}_{part}"]
         assert tuple(g.shape) == tuple(w.shape), (tag, part, g.shape, w.shape)
@@ -40,7 +40,7 @@ def _compare_parts(kp, kw, tag, dtype):
             if w.size:
                 err = np.linalg.norm(g.cpu().numpy() - w) / np.linalg.norm(w)
                 assert err <= 1e-3, err       # stated bound; fp32 accumulation gives ~1e-6
-                assert err <= 2e-5, err
+                assert err <= coef_tol, err
         else:
             assert g.dtype == dtype
             np.testing.assert_array_equal(g.float().cpu().numpy(), w.astype(np.float32))  # stored rows are copies
@@ -207,3 +207,47 @@ def test_append_branch_of_a_short_mid():
         got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv)
         assert np.abs(got.cpu().numpy() - want).max() <= 1e-3
         _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype)
+
+
+def test_one_full_length_sequence_against_the_oracle():
+    """One sequence of the benchmark's headline configuration at full length (32768 tokens, 8 KV heads of 128 dims,
+    32 query heads, 1024 states, 1024-token window, 64 of 128 dims per head compressed, bf16): prefill, one
+    streaming step and the decode attention against the CPU restatement on identical inputs.  The short cases
+    above never reach this depth: 31740 mid rows, 992 pages, 31 pages per workgroup."""
+    from fourierattention_amd import DynamicCache, ExtraConfig, masks as pm
+    dtype, B, Hq, Hkv, D, S = torch.bfloat16, 1, 32, 8, 128, 32768
+    m = pm.synthetic_masks(1, Hkv, D, 64, seed=0)
+    cfg = ExtraConfig(numinittokens=4, maxlocallen=1024, maxmidstates=1024, non_critical_dims=m, non_critical_dims_path=None,
+                      max_position_embeddings=1 << 20, num_key_value_heads=Hkv, max_new_tokens=8, model_type="llama")
+    r = np.random.default_rng(0)
+    cos, sin = fo.rope_tables(np.arange(S), D)
+    k = H.to_dtype_np(fo.apply_rope(r.standard_normal((B, Hkv, S, D)), cos, sin), dtype)
+    v = H.to_dtype_np(r.standard_normal((B, Hkv, S, D)), dtype)
+    gpu = DynamicCache(cfg)
+    cpu = OracleCache(cfg, masks=m, model_dtype="bf16")
+    gpu.update(H.to_gpu(k, dtype), H.to_gpu(v, dtype), 0)
+    cpu.update(k, v, 0)
+    del k, v
+    assert gpu._tables is not None                      # the matrix-core kernels take this shape
+    assert (gpu._book.t_x, gpu._book.t_c) == (cpu._t_x(), cpu.t_c) and gpu.curr_tokennum == cpu.curr_tokennum
+    # stored rows exact; coefficients within 1e-3 (a prompt this long is compressed on the matrix cores with the
+    # basis rounded to f16: about 2e-4)
+    _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype, coef_tol=5e-4)
+    _compare_parts(gpu.value_cache[0], cpu.value_cache[0], "v", dtype, coef_tol=5e-4)
+    for name, tol in (("k_scale", 4e-3), ("k_layer_average", 1e-2), ("kd_layer_average", 2e-3),
+                      ("v_scale", 4e-3), ("v_layer_average", 1e-2), ("vd_layer_average", 2e-3)):
+        np.testing.assert_allclose(getattr(gpu, name)[0].float().cpu().numpy(), getattr(cpu, name)[0], rtol=tol, atol=tol)
+        getattr(cpu, name)[0] = getattr(gpu, name)[0].float().cpu().numpy()   # attention below on identical statistics
+    cq, sq = fo.rope_tables(np.array([S]), D)
+    kn = H.to_dtype_np(fo.apply_rope(r.standard_normal((B, Hkv, 1, D)), cq, sq), dtype)
+    vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+    q = H.to_dtype_np(fo.apply_rope(r.standard_normal((B, Hq, 1, D)), cq, sq), dtype)
+    kp, vp = gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), 0)
+    kw, vw = cpu.update(kn, vn, 0)
+    _compare_parts(kp, kw, "k", dtype, coef_tol=5e-4)
+    _compare_parts(vp, vw, "v", dtype, coef_tol=5e-4)
+    assert gpu.get_seq_length(0) == cpu.get_seq_length(0) == S + 1
+    want = cpu.attend(q, kw, vw, 0, Hq, Hkv)
+    got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv).cpu().numpy()
+    err = np.abs(got - want).max()
+    assert err <= 2e-2 and err <= 1e-3, err              # stated bound, and what fp32 accumulation really leaves

@@ -188,3 +188,26 @@ def test_full_size_properties():
     assert cache.get_seq_length(0) == n0 + 1
     out2 = cache.decode_attention(q, 0, Hq, Hkv)
     assert torch.isfinite(out2).all() and (out2 - out).abs().max().item() < 1.0
+
+
+@pytest.mark.parametrize("workload", ["config4_decode_attn_8b_64k", "config5_decode_attn_3b_128k"])
+def test_long_splits_agree_with_the_generic_kernels(workload):
+    """The two long-context geometries of the benchmark at full size: a workgroup walks 252 pages (config 4) or
+    127 pages in two passes with 1024 frequencies (config 5), so the page-to-page rotation of the
+    coefficient-domain state is applied that many times in a row.  The generic kernels evaluate every phase from
+    its exactly reduced integer argument instead; both must agree as they do on short contexts."""
+    import bench
+    w = bench.WORKLOADS[workload]
+    dev = torch.device("cuda", 0)
+    cache, q, kn, vn = bench.build_cache(w, torch.bfloat16, dev)
+    Hq, Hkv = w["Hq"], w["Hkv"]
+    assert cache._tables is not None
+    out = cache.decode_attention(q, 0, Hq, Hkv)
+    cache.force_generic = True
+    ref = cache.decode_attention(q, 0, Hq, Hkv)
+    cache.force_generic = False
+    assert torch.isfinite(out).all()
+    err = (out - ref).abs().max().item()
+    assert err <= 5e-3, err
+    del cache
+    torch.cuda.empty_cache()
