@@ -54,33 +54,46 @@ __global__ __launch_bounds__(256) void stream_update_kernel(const StreamParams p
   const int bx = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   if (bx < p.c_end[1]) {
     // ---- rank-1 coefficient update: block = 64 columns x 64 frequencies, thread = (column, 16 frequencies)
+    // The phase factors depend on the frequency only: 64 threads evaluate one each (exactly reduced phase, as
+    // fa_coeff_update) while the coefficient loads of all threads are on their way, and hand them over in LDS.
+    __shared__ float2 s_cs[64];
     const int which = bx >= p.c_end[0];
     const StreamTensor& t = p.t[which];
     const int rel = bx - (which ? p.c_end[0] : 0);
     const int cb = rel / p.cblk_n, nb = rel - cb * p.cblk_n;
     const int lane = tid & 63, ng = tid >> 6;
     const int m = cb * 64 + lane;
-    if (m >= t.C) return;
-    const E* old_row = (const E*)t.ring + (int64_t)b * p.ring_bs + (int64_t)p.evict_slot * p.ring_rs;
-    const float e = fa_to_float(old_row[t.c_list[m]]);
-    float* cbase = t.coef + (int64_t)b * 2 * p.N * t.C + m;
+    const bool live = m < t.C;
     const int n_beg = nb * 64;
     const int n_end = min(p.N, n_beg + 64);
+    float e = 0.f;
+    float* cbase = t.coef + (int64_t)b * 2 * p.N * t.C + (live ? m : 0);
     float cv[16], sv[16];
+    if (live) {
+      const E* old_row = (const E*)t.ring + (int64_t)b * p.ring_bs + (int64_t)p.evict_slot * p.ring_rs;
+      e = fa_to_float(old_row[t.c_list[m]]);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int n = min(n_beg + ng + 4 * i, p.N - 1);
-      cv[i] = cbase[(int64_t)n * t.C];
-      sv[i] = cbase[(int64_t)(p.N + n) * t.C];
+      for (int i = 0; i < 16; ++i) {
+        const int n = min(n_beg + ng + 4 * i, p.N - 1);
+        cv[i] = cbase[(int64_t)n * t.C];
+        sv[i] = cbase[(int64_t)(p.N + n) * t.C];
+      }
     }
+    if (tid < 64) {
+      float sn, co;
+      fa_sincos_phase(min(n_beg + tid, p.N - 1), p.phase, p.T, &sn, &co);
+      s_cs[tid] = make_float2(co, sn);
+    }
+    __syncthreads();
+    if (live) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int n = n_beg + ng + 4 * i;
-      if (n < n_end) {
-        float sn, co;
-        fa_sincos_phase(n, p.phase, p.T, &sn, &co);   // exactly reduced phase, as fa_coeff_update
-        cbase[(int64_t)n * t.C] = cv[i] + co * e;
-        cbase[(int64_t)(p.N + n) * t.C] = sv[i] + sn * e;
+      for (int i = 0; i < 16; ++i) {
+        const int n = n_beg + ng + 4 * i;
+        if (n < n_end) {
+          const float2 cs = s_cs[ng + 4 * i];
+          cbase[(int64_t)n * t.C] = cv[i] + cs.x * e;
+          cbase[(int64_t)(p.N + n) * t.C] = sv[i] + cs.y * e;
+        }
       }
     }
     return;
