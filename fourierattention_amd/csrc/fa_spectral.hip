@@ -270,17 +270,42 @@ template <typename E>
 __global__ __launch_bounds__(256) void coeff_update_kernel(
     float* __restrict__ c, const E* __restrict__ row, int64_t row_bs, const int32_t* __restrict__ cols,
     int N, int Mc, int64_t p, int T) {
-  const int lane = threadIdx.x & 63, ng = threadIdx.x >> 6;
+  // block = 64 columns x 64 frequencies, thread = (column, 16 frequencies).  The phase factors depend on the
+  // frequency only: 64 threads evaluate one each while the coefficient loads are on their way.
+  __shared__ float2 s_cs[64];
+  const int tid = threadIdx.x, lane = tid & 63, ng = tid >> 6;
   const int m = blockIdx.x * 64 + lane, b = blockIdx.z;
-  if (m >= Mc) return;
-  const float e = fa_to_float(row[(int64_t)b * row_bs + (cols ? cols[m] : m)]);
-  float* cb = c + (int64_t)b * 2 * N * Mc + m;
+  const bool live = m < Mc;
   const int n_beg = blockIdx.y * 64;
-  for (int n = n_beg + ng; n < min(N, n_beg + 64); n += 4) {
-    float s, co;
-    fa_sincos_phase(n, p, T, &s, &co);
-    cb[(int64_t)n * Mc] += co * e;
-    cb[(int64_t)(N + n) * Mc] += s * e;
+  const int n_end = min(N, n_beg + 64);
+  float e = 0.f;
+  float* cb = c + (int64_t)b * 2 * N * Mc + (live ? m : 0);
+  float cv[16], sv[16];
+  if (live) {
+    e = fa_to_float(row[(int64_t)b * row_bs + (cols ? cols[m] : m)]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int n = min(n_beg + ng + 4 * i, N - 1);
+      cv[i] = cb[(int64_t)n * Mc];
+      sv[i] = cb[(int64_t)(N + n) * Mc];
+    }
+  }
+  if (tid < 64) {
+    float sn, co;
+    fa_sincos_phase(min(n_beg + tid, N - 1), p, T, &sn, &co);
+    s_cs[tid] = make_float2(co, sn);
+  }
+  __syncthreads();
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int n = n_beg + ng + 4 * i;
+      if (n < n_end) {
+        const float2 cs = s_cs[ng + 4 * i];
+        cb[(int64_t)n * Mc] = cv[i] + cs.x * e;
+        cb[(int64_t)(N + n) * Mc] = sv[i] + cs.y * e;
+      }
+    }
   }
 }
 
