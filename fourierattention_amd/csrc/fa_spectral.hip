@@ -102,11 +102,18 @@ __global__ __launch_bounds__(256) void col_stats_partial_kernel(
   if (m < Mc) {
     const int col = cols ? cols[m] : m;
     const E* p = a + (int64_t)b * a_bs + col;
-    for (int k = k0 + kg; k < k1; k += 4) {
-      float v = fa_to_float(p[(int64_t)k * a_rs]);
-      sum += v;
-      mx = fmaxf(mx, v);
-      mn = fminf(mn, v);
+    // eight rows in flight per thread (clamped, so that none of the loads is conditional)
+    for (int k = k0 + kg; k < k1; k += 4 * 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = fa_to_float(p[(int64_t)min(k + 4 * u, k1 - 1) * a_rs]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (k + 4 * u < k1) {
+          sum += v[u];
+          mx = fmaxf(mx, v[u]);
+          mn = fminf(mn, v[u]);
+        }
     }
   }
   s_sum[kg][lane] = sum;
