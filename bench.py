@@ -366,14 +366,24 @@ def main():
     for _ in range(5):
         cache.update(kn, vn, 0)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
+    # The launch is shorter than the host takes to issue it.  For the device-side figure the 50 updates are queued
+    # behind a few milliseconds of other work, so that the device runs them back to back; the wall figure is the
+    # host-paced loop.
+    busy = torch.empty((8192, 8192), dtype=torch.bfloat16, device=device).normal_()
+    for _ in range(4):
+        busy = busy @ busy
     start.record()
     for _ in range(50):
         cache.update(kn, vn, 0)
     stop.record()
     torch.cuda.synchronize()
-    upd_wall = (time.perf_counter() - t0) / 50
     upd_ms = start.elapsed_time(stop) / 50
+    del busy
+    t0 = time.perf_counter()
+    for _ in range(50):
+        cache.update(kn, vn, 0)
+    torch.cuda.synchronize()
+    upd_wall = (time.perf_counter() - t0) / 50
     upd_bytes = w["B"] * 2 * 2 * w["M"] * ck * 4
     result["stream_update"] = {"ms_per_step": round(upd_ms, 5), "wall_ms_per_step": round(upd_wall * 1e3, 5),
                                "algorithmic_bytes": upd_bytes, "GB_s": round(upd_bytes / (upd_ms * 1e-3) / 1e9, 1)}
