@@ -209,18 +209,20 @@ def test_append_branch_of_a_short_mid():
         _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype)
 
 
-@pytest.mark.parametrize("mask", ["uniform", "Layer_0", "Layer_31"])
-def test_one_full_length_sequence_against_the_oracle(mask):
+@pytest.mark.parametrize("mask,dtype,Hq", [("uniform", torch.bfloat16, 32), ("Layer_0", torch.bfloat16, 32),
+                                           ("Layer_31", torch.bfloat16, 32), ("uniform", torch.float16, 24)])
+def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq):
     """One sequence of the benchmark's headline configuration at full length (32768 tokens, 8 KV heads of 128 dims,
     32 query heads, 1024 states, 1024-token window, bf16): prefill, one streaming step and the decode attention
     against the CPU restatement on identical inputs.  The short cases above never reach this depth: 31740 mid rows,
     992 pages, 31 pages per workgroup.  Masks: the benchmark's (64 of 128 dims per head compressed) and two layers
     of the reference's own mask for this model and context (ragged heads: layer 0 compresses 90 % / 95 % of the
-    K / V dims, layer 31 50 % / 70 % with heads above 64 stored dims, which take the wide kernel instance)."""
+    K / V dims, layer 31 50 % / 70 % with heads above 64 stored dims, which take the wide kernel instance); the last
+    case is the 3B geometry (three query heads per KV head) in fp16."""
     import json
     import os
     from fourierattention_amd import DynamicCache, ExtraConfig, masks as pm
-    dtype, B, Hq, Hkv, D, S = torch.bfloat16, 1, 32, 8, 128, 32768
+    B, Hkv, D, S = 1, 8, 128, 32768
     if mask == "uniform":
         m = pm.synthetic_masks(1, Hkv, D, 64, seed=0)
     else:
@@ -233,7 +235,7 @@ def test_one_full_length_sequence_against_the_oracle(mask):
     k = H.to_dtype_np(fo.apply_rope(r.standard_normal((B, Hkv, S, D)), cos, sin), dtype)
     v = H.to_dtype_np(r.standard_normal((B, Hkv, S, D)), dtype)
     gpu = DynamicCache(cfg)
-    cpu = OracleCache(cfg, masks=m, model_dtype="bf16")
+    cpu = OracleCache(cfg, masks=m, model_dtype=H.NP_ROUND[dtype])
     gpu.update(H.to_gpu(k, dtype), H.to_gpu(v, dtype), 0)
     cpu.update(k, v, 0)
     del k, v
