@@ -209,26 +209,29 @@ def test_append_branch_of_a_short_mid():
         _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype)
 
 
-@pytest.mark.parametrize("mask,dtype,Hq", [("uniform", torch.bfloat16, 32), ("Layer_0", torch.bfloat16, 32),
-                                           ("Layer_31", torch.bfloat16, 32), ("uniform", torch.float16, 24)])
-def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq):
+@pytest.mark.parametrize("mask,dtype,Hq,S,states", [
+    ("uniform", torch.bfloat16, 32, 32768, 1024), ("Layer_0", torch.bfloat16, 32, 32768, 1024),
+    ("Layer_31", torch.bfloat16, 32, 32768, 1024), ("uniform", torch.float16, 24, 32768, 1024),
+    ("uniform", torch.bfloat16, 24, 40000, 2048)])
+def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq, S, states):
     """One sequence of the benchmark's headline configuration at full length (32768 tokens, 8 KV heads of 128 dims,
     32 query heads, 1024 states, 1024-token window, bf16): prefill, one streaming step and the decode attention
     against the CPU restatement on identical inputs.  The short cases above never reach this depth: 31740 mid rows,
     992 pages, 31 pages per workgroup.  Masks: the benchmark's (64 of 128 dims per head compressed) and two layers
     of the reference's own mask for this model and context (ragged heads: layer 0 compresses 90 % / 95 % of the
     K / V dims, layer 31 50 % / 70 % with heads above 64 stored dims, which take the wide kernel instance); the last
-    case is the 3B geometry (three query heads per KV head) in fp16."""
+    fourth case is the 3B geometry (three query heads per KV head) in fp16, the fifth the same geometry with 2048
+    states (1024 frequencies: the mid rows run as a score pass and a value pass) on a 40000-token sequence."""
     import json
     import os
     from fourierattention_amd import DynamicCache, ExtraConfig, masks as pm
-    B, Hkv, D, S = 1, 8, 128, 32768
+    B, Hkv, D = 1, 8, 128
     if mask == "uniform":
         m = pm.synthetic_masks(1, Hkv, D, 64, seed=0)
     else:
         fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "masks_extract.json")))
         m = {"Layer_0": fx["llama3.1-8b-fourier/compressed_dims_32k_1024states"]["layers"][mask]["splithead"]}
-    cfg = ExtraConfig(numinittokens=4, maxlocallen=1024, maxmidstates=1024, non_critical_dims=m, non_critical_dims_path=None,
+    cfg = ExtraConfig(numinittokens=4, maxlocallen=1024, maxmidstates=states, non_critical_dims=m, non_critical_dims_path=None,
                       max_position_embeddings=1 << 20, num_key_value_heads=Hkv, max_new_tokens=8, model_type="llama")
     r = np.random.default_rng(0)
     cos, sin = fo.rope_tables(np.arange(S), D)
