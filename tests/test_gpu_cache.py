@@ -209,11 +209,11 @@ def test_append_branch_of_a_short_mid():
         _compare_parts(gpu.key_cache[0], cpu.key_cache[0], "k", dtype)
 
 
-@pytest.mark.parametrize("mask,dtype,Hq,S,states", [
-    ("uniform", torch.bfloat16, 32, 32768, 1024), ("Layer_0", torch.bfloat16, 32, 32768, 1024),
-    ("Layer_31", torch.bfloat16, 32, 32768, 1024), ("uniform", torch.float16, 24, 32768, 1024),
-    ("uniform", torch.bfloat16, 24, 40000, 2048)])
-def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq, S, states):
+@pytest.mark.parametrize("mask,dtype,Hq,S,states,D", [
+    ("uniform", torch.bfloat16, 32, 32768, 1024, 128), ("Layer_0", torch.bfloat16, 32, 32768, 1024, 128),
+    ("Layer_31", torch.bfloat16, 32, 32768, 1024, 128), ("uniform", torch.float16, 24, 32768, 1024, 128),
+    ("uniform", torch.bfloat16, 24, 40000, 2048, 128), ("uniform", torch.bfloat16, 16, 20000, 512, 64)])
+def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq, S, states, D):
     """One sequence of the benchmark's headline configuration at full length (32768 tokens, 8 KV heads of 128 dims,
     32 query heads, 1024 states, 1024-token window, bf16): prefill, one streaming step and the decode attention
     against the CPU restatement on identical inputs.  The short cases above never reach this depth: 31740 mid rows,
@@ -221,13 +221,14 @@ def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq, S, states)
     of the reference's own mask for this model and context (ragged heads: layer 0 compresses 90 % / 95 % of the
     K / V dims, layer 31 50 % / 70 % with heads above 64 stored dims, which take the wide kernel instance); the last
     fourth case is the 3B geometry (three query heads per KV head) in fp16, the fifth the same geometry with 2048
-    states (1024 frequencies: the mid rows run as a score pass and a value pass) on a 40000-token sequence."""
+    states (1024 frequencies: the mid rows run as a score pass and a value pass) on a 40000-token sequence, the
+    last one heads of 64 dims (two query heads per KV head, 512 states)."""
     import json
     import os
     from fourierattention_amd import DynamicCache, ExtraConfig, masks as pm
-    B, Hkv, D = 1, 8, 128
+    B, Hkv = 1, 8
     if mask == "uniform":
-        m = pm.synthetic_masks(1, Hkv, D, 64, seed=0)
+        m = pm.synthetic_masks(1, Hkv, D, D // 2, seed=0)
     else:
         fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "masks_extract.json")))
         m = {"Layer_0": fx["llama3.1-8b-fourier/compressed_dims_32k_1024states"]["layers"][mask]["splithead"]}
