@@ -80,6 +80,60 @@ __global__ __launch_bounds__(256) void mid_pack_kernel(
   }
 }
 
+// The same for 16-bit rows that are 16-byte aligned: the head's whole slice of the 32 token rows is read with
+// 16-byte loads into LDS (every line of the source is needed anyway: stored and compressed dims interleave), and
+// the gather along the stored dims happens on the way out of LDS.
+template <typename E>
+__global__ __launch_bounds__(256) void mid_pack_rows_kernel(
+    const E* __restrict__ src, int64_t src_bs, int64_t src_rs, int64_t row0, int L, E* __restrict__ store,
+    int64_t st_bs, int cap_pages, const int32_t* __restrict__ n_list, const int32_t* __restrict__ n_h,
+    const int32_t* __restrict__ pad_h, int D, int is_v) {
+  constexpr int kMaxD = 256;                        // head dim, and padded stored dims of a head
+  constexpr int kPitch = kMaxD + 8;                 // elements; keeps rows 16-byte aligned
+  struct alignas(sizeof(E) * 8) Piece { E v[8]; };
+  __shared__ __attribute__((aligned(32))) E tile[32][kPitch];
+  __shared__ int s_col[kMaxD];
+  const int page = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int n0 = n_h[h], n_len = n_h[h + 1] - n0;
+  const int p0 = pad_h[h], dp = pad_h[h + 1] - p0;
+  if (n_len == 0) return;
+  const int tid = threadIdx.x;
+  // dim within the head of every stored position (clamped into the head: the reads below stay inside the tile)
+  for (int j = tid; j < dp; j += 256) s_col[j] = min(max(n_list[n0 + min(j, n_len - 1)] - h * D, 0), D - 1);
+  const E* sb = src + (int64_t)b * src_bs + row0 * src_rs + (int64_t)h * D;
+  const int ppr = D >> 3;                           // 16-byte pieces per row of the head
+  const int64_t last = (int64_t)L - 1;
+  for (int p = tid; p < 32 * ppr; p += 256) {
+    const int t = p / ppr, c = p - t * ppr;
+    const int64_t token = (int64_t)page * 32 + t;
+    *(Piece*)&tile[t][c * 8] = *(const Piece*)(sb + (token < last ? token : last) * src_rs + c * 8);
+  }
+  __syncthreads();
+  Piece* out = (Piece*)(store + (int64_t)b * st_bs + (int64_t)p0 * 32 * cap_pages + (int64_t)page * dp * 32);
+  const int n_pieces = dp * 32 / 8;
+  for (int piece = tid; piece < n_pieces; piece += 256) {
+    const int frag = piece >> 6, lane = piece & 63;
+    Piece o;
+    if (!is_v) {
+      const int nks = dp >> 5;
+      const int tb = frag / nks, s_ = frag - tb * nks;
+      const int t = tb * 16 + (lane & 15), j0 = s_ * 32 + 8 * (lane >> 4);
+      const bool row_ok = (int64_t)page * 32 + t < L;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o.v[e] = (row_ok && j0 + e < n_len) ? tile[t][s_col[j0 + e]] : E{};
+    } else {
+      const int j = frag * 16 + (lane & 15);
+      const int col = s_col[j];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int t = 8 * (lane >> 4) + i;
+        o.v[i] = (j < n_len && (int64_t)page * 32 + t < L) ? tile[t][col] : E{};
+      }
+    }
+    out[piece] = o;
+  }
+}
+
 template <typename E>
 __global__ __launch_bounds__(256) void mid_append_kernel(
     const E* __restrict__ row, int64_t row_bs, int64_t pos, E* __restrict__ store, int64_t st_bs, int cap_pages,
@@ -135,8 +189,17 @@ extern "C" int fa_mid_pack(const void* src, int dtype, int64_t src_bs, int64_t s
   FA_REQUIRE(D > 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: head_dim %d", D);
   FA_REQUIRE(D <= 256, FA_ERR_UNSUPPORTED, "fa_mid_pack: head_dim %d above 256", D);
   dim3 grid(fa_cdiv(L, 32), Hkv, B);
+  const bool rows16 = ((uintptr_t)src & 15) == 0 && src_bs % 8 == 0 && src_rs % 8 == 0 && D % 8 == 0 &&
+                      src_rs >= (int64_t)Hkv * D;
   int rc = dispatch16(dtype, "fa_mid_pack", [&](auto tag) {
     using E = decltype(tag);
+    if constexpr (sizeof(E) == 2) {
+      if (rows16) {
+        mid_pack_rows_kernel<E><<<grid, 256, 0, st>>>((const E*)src, src_bs, src_rs, row0, L, (E*)store, st_bs, cap_pages,
+                                                     n_list, n_h, pad_h, D, is_v);
+        return;
+      }
+    }
     mid_pack_kernel<E><<<grid, 256, 0, st>>>((const E*)src, src_bs, src_rs, row0, L, (E*)store, st_bs, cap_pages, n_list,
                                             n_h, pad_h, is_v);
   });
