@@ -81,6 +81,25 @@ def fourier_attention(query_states: torch.Tensor, key_states: torch.Tensor, valu
     return o.reshape(bsz, q_len, -1).to(query_states.dtype)
 
 
+class LlamaRotaryEmbedding(nn.Module):
+    """Plain ("default") rotary tables: ``inv_freq = theta^(-2i/D)``, angles in fp32, tables in the
+    activation dtype (modeling_llama_fourier.py:165-187).  ``config`` needs ``head_dim`` (or ``hidden_size`` and
+    ``num_attention_heads``) and optionally ``rope_theta`` (default 10000, as the stock config)."""
+
+    def __init__(self, config):
+        super().__init__()
+        d = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+        theta = float(getattr(config, "rope_theta", 10000.0))
+        inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    @torch.no_grad()
+    def forward(self, x, position_ids):
+        freqs = position_ids[:, :, None].float() * self.inv_freq[None, None, :].float().to(position_ids.device)
+        emb = torch.cat((freqs, freqs), dim=-1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
 class LlamaSdpaAttention(nn.Module):
     """Projection + RoPE + Fourier-cache attention with the reference's forward contract
     (modeling_llama_fourier.py:547-667).  ``config`` needs ``hidden_size``, ``num_attention_heads``,
@@ -99,6 +118,9 @@ class LlamaSdpaAttention(nn.Module):
         self.k_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
         self.v_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, self.hidden_size, bias=bias)
+        # only used when a caller passes position_ids instead of position_embeddings
+        # (modeling_llama_fourier.py:332, 604-612)
+        self.rotary_emb = LlamaRotaryEmbedding(config)
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 position_ids: Optional[torch.LongTensor] = None, past_key_value: Optional[DynamicCache] = None,
@@ -109,13 +131,16 @@ class LlamaSdpaAttention(nn.Module):
             raise NotImplementedError("attention weights are never materialised on this path")
         if past_key_value is None:
             raise ValueError("a Fourier DynamicCache must be passed as past_key_value")
-        if position_embeddings is None:
-            raise ValueError("position_embeddings (cos, sin) are required")
+        if position_embeddings is None and position_ids is None:
+            raise ValueError("either position_embeddings (cos, sin) or position_ids must be passed")
         bsz, q_len, _ = hidden_states.size()
         q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
         k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        cos, sin = position_embeddings
+        if position_embeddings is None:   # modeling_llama_fourier.py:604-612
+            cos, sin = self.rotary_emb(v, position_ids)
+        else:
+            cos, sin = position_embeddings
         q, k = apply_rotary_pos_emb(q, k, cos, sin)
         cache_kwargs = {"sin": sin, "cos": cos, "cache_position": cache_position}
         o = fourier_attention(q, k, v, past_key_value, self.layer_idx, self.num_heads, self.num_key_value_heads,

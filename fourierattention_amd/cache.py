@@ -97,13 +97,58 @@ class CacheParts(Mapping):
         return self.cache._window_in_order(layer, t)
 
 
-class DynamicCache:
+class Cache(torch.nn.Module):
+    """Base class of every cache object, as in cache_utils_fourier.py:39-125 (a ``torch.nn.Module`` there too).
+    The modified LLaMA imports this name next to ``DynamicCache`` and ``StaticCache``
+    (modeling_llama_fourier.py:29) and routes on ``isinstance(past_key_values, Cache)``
+    (modeling_llama_fourier.py:946): an object that is not a ``Cache`` is taken for a legacy tuple."""
+
+    def __init__(self) -> None:
+        super().__init__()
+
+    def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
+        raise NotImplementedError("Make sure to implement `update` in a subclass.")
+
+    def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
+        raise NotImplementedError("Make sure to implement `get_seq_length` in a subclass.")
+
+    def get_max_cache_shape(self) -> Optional[int]:
+        raise NotImplementedError("Make sure to implement `get_max_cache_shape` in a subclass.")
+
+    def get_max_length(self) -> Optional[int]:
+        return self.get_max_cache_shape()
+
+    def get_usable_length(self, new_seq_length: int, layer_idx: Optional[int] = 0) -> int:
+        """cache_utils_fourier.py:93-102: everything is usable unless the cache has a capacity."""
+        max_length = self.get_max_cache_shape()
+        previous_seq_length = self.get_seq_length(layer_idx)
+        if max_length is not None and previous_seq_length + new_seq_length > max_length:
+            return max_length - new_seq_length
+        return previous_seq_length
+
+    @property
+    def seen_tokens(self):
+        return getattr(self, "_seen_tokens", None)
+
+
+class StaticCache(Cache):
+    """The name the modified LLaMA tests with ``isinstance(past_key_values, StaticCache)``
+    (modeling_llama_fourier.py:1052).  The Fourier path never uses a static cache (the reference's own
+    class, cache_utils_fourier.py:1386, is the stock one and unrelated to the Fourier cache), so the class exists
+    for those tests only and cannot be constructed."""
+
+    def __init__(self, *args, **kwargs) -> None:
+        raise NotImplementedError("StaticCache is not part of the Fourier cache path; only DynamicCache is provided")
+
+
+class DynamicCache(Cache):
     """See module docstring.  ``extra_config`` needs: ``max_new_tokens``, ``maxlocallen``,
     ``maxmidstates``, ``numinittokens``, ``num_key_value_heads``, ``max_position_embeddings``,
     ``non_critical_dims_path`` (cache_utils_fourier.py:394-403).  As an extension,
     ``extra_config.non_critical_dims`` may hold the already-parsed mask dict instead of a path."""
 
     def __init__(self, extra_config, num_hidden_layers: Optional[int] = None, device=None) -> None:
+        super().__init__()
         self._seen_tokens = 0
         self.maxnewtokens = extra_config.max_new_tokens
         self.maxlocallen = extra_config.maxlocallen

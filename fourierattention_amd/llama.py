@@ -20,7 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops, synth
-from .attention import LlamaSdpaAttention, fourier_attention
+from .attention import LlamaRotaryEmbedding, LlamaSdpaAttention, fourier_attention
 from .cache import DynamicCache
 
 
@@ -65,23 +65,6 @@ class LlamaRMSNorm(nn.Module):
         x = x.float()
         x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
         return self.weight * x.to(dt)
-
-
-class LlamaRotaryEmbedding(nn.Module):
-    """Plain ("default") rotary tables: ``inv_freq = theta^(-2i/D)``, angles in fp32, tables in the
-    activation dtype (modeling_llama_fourier.py:165-187)."""
-
-    def __init__(self, config: LlamaConfig):
-        super().__init__()
-        d = config.head_dim
-        inv_freq = 1.0 / (config.rope_theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
-        self.register_buffer("inv_freq", inv_freq, persistent=False)
-
-    @torch.no_grad()
-    def forward(self, x, position_ids):
-        freqs = position_ids[:, :, None].float() * self.inv_freq[None, None, :].float().to(position_ids.device)
-        emb = torch.cat((freqs, freqs), dim=-1)
-        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
 
 
 class LlamaMLP(nn.Module):
