@@ -92,6 +92,30 @@ def _phase_matrix(rows: np.ndarray, cols: np.ndarray, period: int) -> np.ndarray
     return prod.astype(np.float64) * (TWO_PI / float(period))
 
 
+_BASIS_CACHE: dict = {}
+
+
+def _basis(rows: int, n_f: int, period: int) -> np.ndarray:
+    """``(rows, 2 n_f)`` float64: ``cos(2 pi l n / period)`` for ``n < n_f`` then the ``sin`` columns, row ``l``
+    a position, phases reduced exactly in integers.  Rows do not depend on each other, so the largest table built
+    for an ``(n_f, period)`` pair is kept (two pairs at most) and shorter requests are slices of it: building the
+    table, not the contraction, dominates the cost of long sequences."""
+    key = (int(n_f), int(period))
+    have = _BASIS_CACHE.get(key)
+    if have is None or have.shape[0] < rows:
+        if have is None and len(_BASIS_CACHE) >= 2:
+            _BASIS_CACHE.pop(next(iter(_BASIS_CACHE)))
+        build = int(rows) if rows < 4096 else int(rows) + 64      # room for a few streaming steps
+        have = np.empty((build, 2 * n_f), dtype=np.float64)
+        cols = np.arange(n_f)
+        for r0 in range(0, build, 8192):
+            ph = _phase_matrix(np.arange(r0, min(build, r0 + 8192)), cols, period)
+            np.cos(ph, out=have[r0: r0 + ph.shape[0], :n_f])
+            np.sin(ph, out=have[r0: r0 + ph.shape[0], n_f:])
+        _BASIS_CACHE[key] = have
+    return have[:rows]
+
+
 # ----------------------------------------------------------------------------
 # compression  (TRI:840-865 FFT branch == TRI:21-102 with K_start = 0)
 # ----------------------------------------------------------------------------
@@ -108,11 +132,8 @@ def compress_prefill(x: np.ndarray, n_f: int, t_c: int, dtype=np.float64) -> np.
     x = np.asarray(x, dtype=dtype)
     b, l, c = x.shape
     l_eff = min(l, int(t_c))
-    n = np.arange(n_f)
-    t = np.arange(l_eff)
-    ph = _phase_matrix(n, t, t_c)  # (n_f, l_eff)
-    basis = np.concatenate([np.cos(ph), np.sin(ph)], axis=0).astype(dtype)  # (2 n_f, l_eff)
-    return np.ascontiguousarray(np.einsum("nt,btc->bnc", basis, x[:, :l_eff, :], optimize=True))
+    basis = _basis(l_eff, n_f, t_c).astype(dtype, copy=False)  # (l_eff, 2 n_f): the phase n*t is symmetric in n and t
+    return np.ascontiguousarray(np.einsum("tn,btc->bnc", basis, x[:, :l_eff, :], optimize=True))
 
 
 def coeff_update(coef: np.ndarray, evicted: np.ndarray, p: int, t_c: int, dtype=np.float64) -> np.ndarray:
@@ -154,8 +175,7 @@ def reconstruct(coef: np.ndarray, k: int, t_x: int, dtype=np.float64) -> np.ndar
     """
     coef = np.asarray(coef, dtype=dtype)
     n_f = coef.shape[1] // 2
-    ph = _phase_matrix(np.arange(k), np.arange(n_f), t_x)  # (k, n_f)
-    basis = np.concatenate([np.cos(ph), np.sin(ph)], axis=1).astype(dtype)  # (k, 2 n_f)
+    basis = _basis(int(k), n_f, t_x).astype(dtype, copy=False)  # (k, 2 n_f)
     return np.ascontiguousarray(np.einsum("ln,bnc->blc", basis, coef, optimize=True)) / n_f
 
 
