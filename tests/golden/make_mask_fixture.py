@@ -20,7 +20,9 @@ def main():
     for stem, layers in PICK.items():
         raw = json.load(open(os.path.join(SRC, stem + ".json")))
         split = json.load(open(os.path.join(SRC, stem + "_splithead.json")))
-        out[stem] = {"num_layers": len(split), "layers": {}}
+        # lengths of the raw lists of every layer: they pin the per-layer fraction schedule of the search
+        lengths = {k: [len(raw[k]["self_attn.k_proj"]), len(raw[k]["self_attn.v_proj"])] for k in sorted(raw, key=lambda s: int(s.split("_")[1]))}
+        out[stem] = {"num_layers": len(split), "raw_lengths": lengths, "layers": {}}
         for l in layers:
             key = f"Layer_{l}"
             out[stem]["layers"][key] = {"raw": raw[key], "splithead": split[key]}

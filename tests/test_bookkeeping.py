@@ -78,6 +78,96 @@ def test_state_machine_trace_matches_reference_restatement(I, W, M, max_new, max
             check(l, st)
 
 
+# Literal expectations, derived by hand from cache_utils_fourier.py:494-761 (not from either restatement).
+# Each trace: configuration, then per call (layer, q_len) -> what the call returns ("local" = the three other parts
+# are None, line 613 / 686; "parts" = all four, line 748) and the state afterwards:
+# (k_init rows, k_compressed rows, k_uncompressed rows, k_local rows, curr_tokennum[layer], _seen_tokens, seq length).
+LITERAL_TRACES = {
+    # prompt 50 > maxlen 36: sink 4, mid 50 - 4 - 16 = 30, window 16, 16 coefficient rows; maxtokens = min(50 + 10, 4096),
+    # period 60 - 20 = 40.  Decode: 4 + 16 + 30 + B(2) + 1 = 53 > 37 -> streaming; the counter runs 31, 32, ...
+    "stream": dict(cfg=dict(I=4, W=16, M=16, max_new=10, max_pos=4096, B=2), periods=(40, 40), maxtokens=60, calls=[
+        ((0, 50), "local", (4, 16, 30, 16, 30, 50, 50)),
+        ((1, 50), "local", (4, 16, 30, 16, 30, 50, 50)),     # _seen_tokens moves at layer 0 only (line 520)
+        ((0, 1), "parts", (4, 16, 31, 16, 31, 51, 51)),
+        ((1, 1), "parts", (4, 16, 31, 16, 31, 51, 51)),
+        ((0, 1), "parts", (4, 16, 32, 16, 32, 52, 52)),
+    ]),
+    # prompt 30 <= maxlen 36: everything stays in the window, the other parts are empty (lines 598-611); decode:
+    # 0 + 0 + 0 + B + 1 <= 36 for ever -> the window grows and the layer is never compressed
+    "window_only": dict(cfg=dict(I=4, W=16, M=16, max_new=10, max_pos=4096, B=2), periods=(20, 20), maxtokens=40, calls=[
+        ((0, 30), "local", (0, 0, 0, 30, 0, 30, 30)),
+        ((0, 1), "local", (0, 0, 0, 31, 0, 31, 31)),
+        ((0, 1), "local", (0, 0, 0, 32, 0, 32, 32)),
+    ]),
+    # maxlen 76, prompt 128 -> mid 60, compressed (8 coefficient rows).  Batch 1: 4 + 8 + 60 + 1 + 1 = 74 <= 76 -> the
+    # append branch of a COMPRESSED layer (line 681): the window grows, the caller sees the window only, the
+    # counter and the mid rows stand still; the predicate does not depend on the window length, so it never ends
+    "append_batch1": dict(cfg=dict(I=4, W=64, M=8, max_new=8, max_pos=4096, B=1), periods=(68, 68), maxtokens=136, calls=[
+        ((0, 128), "local", (4, 8, 60, 64, 60, 128, 128)),
+        ((0, 1), "local", (4, 8, 60, 65, 60, 129, 129)),
+        ((0, 1), "local", (4, 8, 60, 66, 60, 130, 130)),
+    ]),
+    # the same cache and prompt with batch 5: 4 + 8 + 60 + 5 + 1 = 78 > 77 -> streaming.  Only k_local.size(0), the
+    # batch size, differs from the trace above (line 680)
+    "stream_batch5": dict(cfg=dict(I=4, W=64, M=8, max_new=8, max_pos=4096, B=5), periods=(68, 68), maxtokens=136, calls=[
+        ((0, 128), "local", (4, 8, 60, 64, 60, 128, 128)),
+        ((0, 1), "parts", (4, 8, 61, 64, 61, 129, 129)),
+        ((0, 1), "parts", (4, 8, 62, 64, 62, 130, 130)),
+    ]),
+    # maxtokens clamped by max_position_embeddings (line 542): min(120 + 10, 113) = 113, period 93, and
+    # int(1 / (1 / 93)) = 92; the mid (100 rows) is longer than that period
+    "clamped": dict(cfg=dict(I=4, W=16, M=16, max_new=10, max_pos=113, B=2), periods=(93, 92), maxtokens=113, calls=[
+        ((0, 120), "local", (4, 16, 100, 16, 100, 120, 120)),
+        ((0, 1), "parts", (4, 16, 101, 16, 101, 121, 121)),
+    ]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LITERAL_TRACES))
+def test_literal_trace_table(name):
+    """Both restatements of the state machine against hand-derived numbers, the oracle first."""
+    tr = LITERAL_TRACES[name]
+    c = tr["cfg"]
+    Hkv, D, layers = 2, 8, 2
+    masks = pm.synthetic_masks(layers, Hkv, D, 3, 5, seed=1)
+    cfg = ExtraConfig(numinittokens=c["I"], maxlocallen=c["W"], maxmidstates=c["M"], non_critical_dims_path=None,
+                      max_position_embeddings=c["max_pos"], num_key_value_heads=Hkv, max_new_tokens=c["max_new"])
+    cpu = OracleCache(cfg, masks=masks, model_dtype="fp32")
+    book = CacheBook(layers, c["I"], c["W"], c["M"], c["max_new"], c["max_pos"])
+    r = np.random.default_rng(0)
+    for (layer, q_len), returned, want in tr["calls"]:
+        x = r.standard_normal((c["B"], Hkv, q_len, D))
+        kd, vd = cpu.update(x, x, layer)
+        st = book.step(layer, c["B"], q_len)
+        none_pattern = [kd[k] is None for k in ("k_init", "k_compressed", "k_uncompressed")]
+        assert none_pattern == [returned == "local"] * 3 and kd["k_local"] is not None and vd["v_local"] is not None
+        assert (st.action is Action.STREAM) == (returned == "parts")
+        kc = cpu.key_cache[layer]
+        got = (kc["k_init"].shape[1], kc["k_compressed"].shape[1], kc["k_uncompressed"].shape[1], kc["k_local"].shape[1],
+               cpu.curr_tokennum[layer], cpu._seen_tokens, cpu.get_seq_length(layer))
+        assert got == want, (name, layer, q_len, got)
+        assert kd["k_local"].shape[1] == (q_len if q_len > 1 else want[3])      # prefill returns the whole prompt
+        lb = book.layers[layer]
+        assert (lb.n_init, lb.n_coef_rows, lb.n_mid, lb.n_local, lb.curr_tokennum, book.seen_tokens, lb.seq_length) == want
+        assert cpu.maxtokens == book.maxtokens == tr["maxtokens"]
+        assert (cpu._t_x(), cpu.t_c) == (book.t_x, book.t_c) == tr["periods"]
+    assert len(cpu) == 1 + max(l for (l, _), _, _ in tr["calls"])
+
+
+def test_batch_size_alone_can_land_in_the_unsupported_late_compression_branch():
+    """Between the two batch sizes of the traces above: 4 + 8 + 60 + 4 + 1 = 77 = maxlen + 1 (line 688)."""
+    masks = pm.synthetic_masks(1, 2, 8, 3, 5, seed=1)
+    cfg = ExtraConfig(numinittokens=4, maxlocallen=64, maxmidstates=8, non_critical_dims_path=None,
+                      max_position_embeddings=4096, num_key_value_heads=2, max_new_tokens=8)
+    cpu, book = OracleCache(cfg, masks=masks, model_dtype="fp32"), CacheBook(1, 4, 64, 8, 8, 4096)
+    x = np.zeros((4, 2, 128, 8))
+    cpu.update(x, x, 0)
+    book.step(0, 4, 128)
+    with pytest.raises(NotImplementedError):
+        cpu.update(x[:, :, :1], x[:, :, :1], 0)
+    assert book.step(0, 4, 1).action is Action.LATE_COMPRESS
+
+
 def test_layer_zero_must_come_first_and_stream_needs_one_token():
     book = CacheBook(2, 4, 16, 16, 10, 4096)
     with pytest.raises(RuntimeError):

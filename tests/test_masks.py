@@ -39,6 +39,14 @@ def test_percent_schedule_matches_list_lengths():
         layer = int(key.split("_")[1])
         assert len(pair["raw"]["self_attn.k_proj"]) == int(mo.percent_schedule(layer, "k") * 1024)
         assert len(pair["raw"]["self_attn.v_proj"]) == int(mo.percent_schedule(layer, "v") * 1024)
+    # every layer of that file, both band edges (3 | 4 and 19 | 20) and the 0.8 band between them
+    lengths = ex["llama3.2-3b-fourier/compressed_dims_4k_fourier"]["raw_lengths"]
+    assert len(lengths) == 28
+    for key, (nk, nv) in lengths.items():
+        layer = int(key.split("_")[1])
+        assert (nk, nv) == (int(mo.percent_schedule(layer, "k") * 1024), int(mo.percent_schedule(layer, "v") * 1024)), key
+    assert lengths["Layer_3"] == [921, 972] and lengths["Layer_4"] == [819, 819]
+    assert lengths["Layer_19"] == [819, 819] and lengths["Layer_20"] == [512, 716]
 
 
 def test_selection_rule():
