@@ -21,6 +21,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# max_position_embeddings of Llama-3.1-8B and Llama-3.2-3B: the cache clamps prompt + max_new_tokens to it
+# (cache_utils_fourier.py:542).  Only the 131072-token prompt of configuration 5 reaches it: there the periods are
+# T_x = 130044 and T_c = int(1 / (1 / T_x)) = 130043, as the reference would run that configuration.
+MODEL_MAX_POSITIONS = 131072
 
 WORKLOADS = {
     # name: B, ctx, Hq, Hkv, D, I, W, M, compressed dims per head, max_new_tokens
@@ -50,7 +54,7 @@ def build_cache(w, dtype, device, seed=0, layers=1):
     from fourierattention_amd import DynamicCache, ExtraConfig, masks, synth
     m = masks.synthetic_masks(layers, w["Hkv"], w["D"], w["cper"], seed=seed)
     cfg = ExtraConfig(numinittokens=w["I"], maxlocallen=w["W"], maxmidstates=w["M"], non_critical_dims=m,
-                      non_critical_dims_path=None, max_position_embeddings=1 << 20, num_key_value_heads=w["Hkv"],
+                      non_critical_dims_path=None, max_position_embeddings=MODEL_MAX_POSITIONS, num_key_value_heads=w["Hkv"],
                       max_new_tokens=w["max_new"], model_type="llama")
     cache = DynamicCache(cfg, device=device)
     g = torch.Generator(device=device).manual_seed(seed)
@@ -80,7 +84,7 @@ def parity_check(device):
     B, Hq, Hkv, D, S = 2, 8, 2, 128, 700
     m = masks.synthetic_masks(1, Hkv, D, 64, seed=3)
     cfg = ExtraConfig(numinittokens=4, maxlocallen=64, maxmidstates=64, non_critical_dims=m, non_critical_dims_path=None,
-                      max_position_embeddings=1 << 20, num_key_value_heads=Hkv, max_new_tokens=16, model_type="llama")
+                      max_position_embeddings=MODEL_MAX_POSITIONS, num_key_value_heads=Hkv, max_new_tokens=16, model_type="llama")
     r = np.random.default_rng(0)
     rd = lambda a: fo.round_bf16(a).astype(np.float64)
     k, v = rd(r.standard_normal((B, Hkv, S, D))), rd(r.standard_normal((B, Hkv, S, D)))
@@ -103,7 +107,7 @@ def _oracle_step_times(w, batch, dtype_name, reps, warm):
     from fourierattention_amd import ExtraConfig, masks
     m = masks.synthetic_masks(1, w["Hkv"], w["D"], w["cper"], seed=0)
     cfg = ExtraConfig(numinittokens=w["I"], maxlocallen=w["W"], maxmidstates=w["M"], non_critical_dims=m,
-                      non_critical_dims_path=None, max_position_embeddings=1 << 20, num_key_value_heads=w["Hkv"],
+                      non_critical_dims_path=None, max_position_embeddings=MODEL_MAX_POSITIONS, num_key_value_heads=w["Hkv"],
                       max_new_tokens=w["max_new"], model_type="llama")
     r = np.random.default_rng(0)
     B, Hq, Hkv, D, S = batch, w["Hq"], w["Hkv"], w["D"], w["ctx"]
@@ -146,12 +150,46 @@ def cpu_baseline():
     except Exception:
         threads = 1
     return {"value": round(bytes3 / med3 / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "cores_note": "threads of the BLAS pool numpy's contractions run on; the rest of the restatement is single-threaded numpy",
             "sample": f"config 3 with 1 of its 8 sequences (ctx 32768, Hq=32, Hkv=8, D=128, bf16-rounded inputs, M=1024, W=1024): "
                       f"update + attention of one layer, one decode step, median of 3 after 1 warm-up = {med3 * 1e3:.1f} ms "
                       f"(min {t3[0] * 1e3:.1f} ms), {bytes3} algorithmic bytes; host has {os.cpu_count()} logical CPUs",
             "config1": {"value": round(bytes1 / med1 / 1e9, 4), "unit": "GB/s",
                         "sample": f"config 1 (B=1, ctx 2048, Hq=24, Hkv=8, D=128, fp32 inputs, M=256, W=512): median of 10 after 3 "
                                   f"warm-ups = {med1 * 1e3:.2f} ms (min {t1[0] * 1e3:.2f} ms), {bytes1} algorithmic bytes"}}
+
+
+KERNEL_SOURCES = ("fa_decode.hip", "fa_decode_mfma.h", "fa_mfma_util.h", "fa_common.h")
+
+
+def kernel_source_digest():
+    """sha256 over the sources of the decode kernels: ties a counter summary under profiles/ to the code it was
+    taken from."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "fourierattention_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(dom, workload):
+    """HBM bytes per launch of the dominant kernel from the hardware-counter summary under profiles/ (rocprofv3
+    --pmc runs cannot happen inside this process).  The summary names the digest of the kernel sources it was
+    taken from; if the sources have changed since, the figure is stale and is not reported."""
+    tpath = os.path.join(ROOT, "profiles", "decode_mid_rows_traffic.txt")
+    if dom != "mid_rows" or not workload.startswith("config3") or not os.path.exists(tpath):
+        return None, None
+    traffic, digest = None, None
+    for line in open(tpath):
+        if line.startswith("hbm_bytes_per_launch:"):
+            traffic = int(float(line.split(":", 1)[1]))
+        if line.startswith("kernel_source_digest:"):
+            digest = line.split(":", 1)[1].strip()
+    now = kernel_source_digest()
+    if digest != now:
+        return None, f"profiles/decode_mid_rows_traffic.txt is stale: taken at kernel sources {digest}, now {now}"
+    return traffic, f"profiles/decode_mid_rows_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources {digest})"
 
 
 def compress_bench(device, reps=20):
@@ -200,7 +238,7 @@ def e2e_bench(name, device, steps=None, warmup=3):
     steps = steps or e["new"]
     m = masks.synthetic_masks(cfg.num_hidden_layers, cfg.num_key_value_heads, cfg.head_dim, e["cper"], seed=0)
     ec = ExtraConfig(numinittokens=e["I"], maxlocallen=e["W"], maxmidstates=e["M"], non_critical_dims=m,
-                     non_critical_dims_path=None, max_position_embeddings=1 << 20,
+                     non_critical_dims_path=None, max_position_embeddings=MODEL_MAX_POSITIONS,
                      num_key_value_heads=cfg.num_key_value_heads, max_new_tokens=e["new"] + warmup + 8, model_type="llama")
     model = random_init(cfg, torch.bfloat16, device, seed=0)
     model.model.fuse_projections()
@@ -237,7 +275,8 @@ def e2e_bench(name, device, steps=None, warmup=3):
             "data": "synthetic (random weights, random prompt K/V through the cache's prefill)",
             "config": {"workload": name, "model": e["preset"], "batch": e["B"], "prompt": e["prompt"],
                        "new_tokens": steps, "sink": e["I"], "window": e["W"], "coeff_rows": e["M"],
-                       "compressed_dims_per_head": e["cper"], "T_x": cache.period_reconstruct},
+                       "compressed_dims_per_head": e["cper"], "T_x": cache.period_reconstruct, "T_c": cache._book.t_c,
+                       "max_position_embeddings": MODEL_MAX_POSITIONS},
             "kv_cache_bytes": {"full_bf16": full, "fourier_in_use": used, "fourier_allocated": held,
                                "reduction_in_use": round(full / used, 3)},
             "synthetic_prefill_s": round(fill_s, 2)}
@@ -252,6 +291,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the leg that uses the CPU restatement: the parity check before the timed region and the "
                          "CPU baseline after it (for profiler runs)")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decodes of configs 4 and 5 in the default run")
     ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
                     help="run the end-to-end decode of a random-init model instead (its own JSON line); --steps caps the "
@@ -333,12 +373,7 @@ def main():
     }
     dom = max(kernel_ms, key=kernel_ms.get)
     dom_gbs = kbytes[dom] / (kernel_ms[dom] * 1e-3) / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "decode_mid_rows_traffic.txt")
-    if dom == "mid_rows" and args.workload.startswith("config3") and os.path.exists(tpath):
-        for line in open(tpath):   # counter summary kept with the profiles: "hbm_bytes_per_launch: <bytes>"
-            if line.startswith("hbm_bytes_per_launch:"):
-                traffic = int(float(line.split(":", 1)[1]))
+    traffic, traffic_source = recorded_traffic(dom, args.workload)
     full = 2 * w["ctx"] * hd * 2
     fourier = 2 * (w["I"] + w["W"]) * hd * 2 + 2 * L * (hd - ck) * 2 + 2 * w["M"] * ck * 4
     result = {
@@ -356,8 +391,12 @@ def main():
         "parity_max_abs_err": parity,
         "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
         "kernel_ms": {k: round(float(v), 5) for k, v in kernel_ms.items()},
+        # each launch of kernel_ms sits between its own pair of HIP events; the pairs cost a few microseconds each,
+        # which is why the three figures add up to more than ms_per_step (timed without events inside)
+        "event_overhead_ms": round(float(sum(kernel_ms.values())) - ms, 5),
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom,
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": dom,
                      "algorithmic_bytes_per_launch": kbytes[dom], "kernel_ms": round(float(kernel_ms[dom]), 5),
                      "whole_step_frac": round(gbs / HBM_PEAK_GBS, 4)},
     }
@@ -385,10 +424,38 @@ def main():
     torch.cuda.synchronize()
     upd_wall = (time.perf_counter() - t0) / 50
     upd_bytes = w["B"] * 2 * 2 * w["M"] * ck * 4
+    # a decode step in use: the streaming update, then the attention over the updated cache
+    for _ in range(5):
+        cache.update(kn, vn, 0)
+        cache.decode_attention(q, 0, Hq, Hkv)
+    start.record()
+    for _ in range(50):
+        cache.update(kn, vn, 0)
+        cache.decode_attention(q, 0, Hq, Hkv)
+    stop.record()
+    torch.cuda.synchronize()
+    both_ms = start.elapsed_time(stop) / 50
+    result["update_plus_attn"] = {"ms_per_step": round(both_ms, 5), "algorithmic_bytes": upd_bytes + nbytes,
+                                  "GB_s": round((upd_bytes + nbytes) / (both_ms * 1e-3) / 1e9, 1),
+                                  "pct_hbm_peak": round(100.0 * (upd_bytes + nbytes) / (both_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)}
     result["stream_update"] = {"ms_per_step": round(upd_ms, 5), "wall_ms_per_step": round(upd_wall * 1e3, 5),
                                "algorithmic_bytes": upd_bytes, "GB_s": round(upd_bytes / (upd_ms * 1e-3) / 1e9, 1)}
-    del cache
+    del cache, q, kn, vn, out
     result["prefill_compress"] = compress_bench(device)
+    if not args.no_e2e and args.workload.startswith("config3"):
+        # BASELINE configs 4 and 5 end to end (a few seconds each); the headline value above stays config 3
+        result["e2e"] = {}
+        for name in E2E:
+            torch.cuda.empty_cache()
+            try:
+                r = e2e_bench(name, device)
+                result["e2e"][name.split("_")[0]] = {
+                    "tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "steps": r["steps"], "warmup": r["warmup"],
+                    "batch": r["config"]["batch"], "prompt": r["config"]["prompt"], "model": r["config"]["model"],
+                    "T_x": r["config"]["T_x"], "T_c": r["config"]["T_c"], "max_position_embeddings": MODEL_MAX_POSITIONS,
+                    "kv_cache_bytes": r["kv_cache_bytes"], "synthetic_prefill_s": r["synthetic_prefill_s"]}
+            except Exception as exc:   # the headline figure above stands on its own; say what happened here
+                result["e2e"][name.split("_")[0]] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

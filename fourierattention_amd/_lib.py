@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libfourier_attn_hip.so")
 FA_BF16, FA_FP16, FA_FP32 = 0, 1, 2
 FA_NO_ROUND = FA_FP32
 FA_MID_TOKEN_MAJOR, FA_MID_PAGED = 0, 1
+FA_COLS_ANY, FA_COLS_HEAD_DIMS = 0, 1
 PAGE_TOKENS, K_DIM_PAD, V_DIM_PAD = 32, 32, 16
 
 STATUS_NAMES = {
@@ -97,7 +98,7 @@ _SIGNATURES = {
     "fa_decode_tables_bytes": (c_size_t, [c_int]),
     "fa_decode_tables_build": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),
     "fa_mid_pack": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p,
-                            c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fa_mid_append": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_void_p]),
     "fa_mid_unpack": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,

@@ -286,9 +286,9 @@ class DynamicCache(Cache):
         t.init.copy_(states[:, :I, :])
         t.ring[:, :W, :].copy_(states[:, S - W:, :])
         t.ring[:, W, :].zero_()
-        cap = max(self._book.t_x, L) + 1
+        cap = max(self._book.t_x, L + int(self.maxnewtokens)) + 1     # room for every row the decode will evict
         t.mid = MidStore(B, n32, nh32, nh_host, self.heads, self.head_dim, cap, states.dtype, states.device, is_v)
-        t.mid.pack(states, I, L)
+        t.mid.pack(states, I, L, head_dims=True)
         # spectral compression of the selected columns (gather fused into the kernel)
         t.coef = ops.mat_fourier(mid, n_f, self._book.t_c, 0, cols=c32, K=fft_rows)
         u_avg, u_std = ops.mat_avg_std(mid, cols=c32, round_dtype=states.dtype)

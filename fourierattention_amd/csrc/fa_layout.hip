@@ -180,8 +180,10 @@ int dispatch16(int dtype, const char* what, F&& f) {
 
 extern "C" int fa_mid_pack(const void* src, int dtype, int64_t src_bs, int64_t src_rs, int64_t row0, int L,
                            void* store, int64_t st_bs, int cap_pages, const int32_t* n_list, const int32_t* n_h,
-                           const int32_t* pad_h, int B, int Hkv, int D, int is_v, fa_stream_t stream) {
+                           const int32_t* pad_h, int B, int Hkv, int D, int is_v, int cols_kind, fa_stream_t stream) {
   FA_REQUIRE(src && store && n_h && pad_h, FA_ERR_NULL_POINTER, "fa_mid_pack: null pointer");
+  FA_REQUIRE(cols_kind == FA_COLS_ANY || cols_kind == FA_COLS_HEAD_DIMS, FA_ERR_BAD_SHAPE, "fa_mid_pack: cols_kind %d",
+             cols_kind);
   FA_REQUIRE(B > 0 && Hkv > 0 && L >= 0 && cap_pages > 0 && row0 >= 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: bad shape");
   FA_REQUIRE((int64_t)cap_pages * 32 >= L, FA_ERR_BAD_SHAPE, "fa_mid_pack: %d rows do not fit %d pages", L, cap_pages);
   if (L == 0) return FA_OK;
@@ -189,8 +191,12 @@ extern "C" int fa_mid_pack(const void* src, int dtype, int64_t src_bs, int64_t s
   FA_REQUIRE(D > 0, FA_ERR_BAD_SHAPE, "fa_mid_pack: head_dim %d", D);
   FA_REQUIRE(D <= 256, FA_ERR_UNSUPPORTED, "fa_mid_pack: head_dim %d above 256", D);
   dim3 grid(fa_cdiv(L, 32), Hkv, B);
-  const bool rows16 = ((uintptr_t)src & 15) == 0 && src_bs % 8 == 0 && src_rs % 8 == 0 && D % 8 == 0 &&
-                      src_rs >= (int64_t)Hkv * D;
+  // the row kernel reads head h's slice [h*D, (h+1)*D) of every source row and picks the stored dims out of it:
+  // only the caller knows whether the index list means that (it cannot be told from the strides)
+  const bool rows16 = cols_kind == FA_COLS_HEAD_DIMS && ((uintptr_t)src & 15) == 0 && src_bs % 8 == 0 &&
+                      src_rs % 8 == 0 && D % 8 == 0;
+  FA_REQUIRE(cols_kind != FA_COLS_HEAD_DIMS || src_rs >= (int64_t)Hkv * D, FA_ERR_BAD_SHAPE,
+             "fa_mid_pack: rows of %lld elements cannot hold %d heads of %d dims", (long long)src_rs, Hkv, D);
   int rc = dispatch16(dtype, "fa_mid_pack", [&](auto tag) {
     using E = decltype(tag);
     if constexpr (sizeof(E) == 2) {

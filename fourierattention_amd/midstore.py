@@ -40,8 +40,10 @@ class MidStore:
     def cap_tokens(self) -> int:
         return self.cap_pages * PAGE_TOKENS
 
-    def pack(self, src: torch.Tensor, row0: int, rows: int, n_list32=None) -> None:
-        """Store ``src[:, row0:row0+rows, n_list]`` (``src (B, S, width)``, last dim contiguous) from token 0."""
+    def pack(self, src: torch.Tensor, row0: int, rows: int, n_list32=None, head_dims: bool = False) -> None:
+        """Store ``src[:, row0:row0+rows, n_list]`` (``src (B, S, width)``, last dim contiguous) from token 0.
+        ``head_dims``: ``src`` holds full K/V rows and the list is the reference's ``kn_list`` / ``vn_list`` (flat
+        ``h*D + d`` entries, head by head); otherwise the entries are plain column numbers of ``src``."""
         assert src.dim() == 3 and src.stride(2) == 1 and src.dtype == self.dtype and rows <= self.cap_tokens
         if rows == 0 or self.Cn == 0:
             return
@@ -49,7 +51,8 @@ class MidStore:
         check(_lib.load().fa_mid_pack(src.data_ptr(), dtype_code(src.dtype), src.stride(0), src.stride(1), int(row0), int(rows),
                                       self.data.data_ptr(), self.batch_stride, self.cap_pages, nl.data_ptr(),
                                       self.n_h32.data_ptr(), self.pad_h32.data_ptr(), self.B, self.Hkv, self.D,
-                                      int(self.is_v), _stream(self.device)))
+                                      int(self.is_v), _lib.FA_COLS_HEAD_DIMS if head_dims else _lib.FA_COLS_ANY,
+                                      _stream(self.device)))
 
     def append(self, row: torch.Tensor, pos: int) -> None:
         """Store ``row[:, n_list]`` (``row (B, width)`` view) at token position ``pos``."""

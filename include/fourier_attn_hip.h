@@ -239,13 +239,23 @@ enum fa_mid_layout { FA_MID_TOKEN_MAJOR = 0, FA_MID_PAGED = 1 };
  * token slots must be zero: allocate the store zero-filled.
  * batch_stride >= pad_h[Hkv] * 32 * cap_pages. */
 
-/* Scatter rows [row0, row0 + L) of src (B, S, Hkv*D), taking for each head the
+/* What the entries of an index list handed to fa_mid_pack mean. */
+#define FA_COLS_ANY 0       /* plain column numbers of the source rows, in any order and range */
+#define FA_COLS_HEAD_DIMS 1 /* the source rows are full K/V rows of Hkv*D elements and the entries of head h
+                               lie in [h*D, (h+1)*D): the reference's kn_list / vn_list (CACHE:445-447) */
+
+/* Scatter rows [row0, row0 + L) of src (B, S, width), taking for each head the
  * columns n_list[n_h[h] .. n_h[h+1]) (the gather x[:, :, kn] of CACHE:560, 578),
- * into pages starting at token 0.  is_v selects the V fragment order. */
+ * into pages starting at token 0.  is_v selects the V fragment order.  With
+ * cols_kind == FA_COLS_HEAD_DIMS (and 16-bit, 16-byte aligned rows) the head's
+ * slice of every row is read whole and the stored dims are picked from it, which
+ * is faster; entries outside the head's range then read a clamped dim.  With
+ * FA_COLS_ANY (e.g. an identity list over rows that are gathered already) every
+ * element is fetched by its own column number. */
 int fa_mid_pack(const void* src, int dtype, int64_t src_batch_stride, int64_t src_row_stride, int64_t row0,
                 int L, void* store, int64_t store_batch_stride, int cap_pages, const int32_t* n_list,
                 const int32_t* n_h_list, const int32_t* pad_h_list, int B, int Hkv, int D, int is_v,
-                fa_stream_t stream);
+                int cols_kind, fa_stream_t stream);
 
 /* Write one row (the evicted window row, CACHE:735, 741) at token position pos. */
 int fa_mid_append(const void* row, int dtype, int64_t row_batch_stride, int64_t pos, void* store,

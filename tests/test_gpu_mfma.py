@@ -21,9 +21,11 @@ def test_mid_store_roundtrip_bit_exact():
         src = torch.randn((B, S, Hkv * D), device="cuda").to(torch.bfloat16)
         n32 = torch.from_numpy(n).int().cuda(); nh32 = torch.tensor(nh, dtype=torch.int32, device="cuda")
         st = MidStore(B, n32, nh32, nh, Hkv, D, 100, torch.bfloat16, "cuda", is_v)
-        st.pack(src, 7, 93)
         want = src[:, 7:100][:, :, torch.from_numpy(n).cuda()]
-        assert torch.equal(st.dense(93), want)
+        for head_dims in (True, False):       # the head's slice read whole / every element by its column number
+            st.data.zero_()
+            st.pack(src, 7, 93, head_dims=head_dims)
+            assert torch.equal(st.dense(93), want)
         st.append(src[:, 120, :], 93)                                   # one evicted row
         st.append(src[:, 121, :], 94)
         want2 = torch.cat([want, src[:, 120:122][:, :, torch.from_numpy(n).cuda()]], dim=1)
@@ -32,6 +34,32 @@ def test_mid_store_roundtrip_bit_exact():
         assert st.cap_tokens >= 400 and torch.equal(st.dense(95), want2)
         # padded dims and unused slots stay zero
         assert st.data.float().abs().sum().item() == pytest.approx(want2.float().abs().sum().item(), rel=1e-6)
+
+
+def test_mid_pack_of_rows_that_are_gathered_already():
+    """An identity list over rows that hold the stored dims only (what re-paging and the function-level drop-in
+    hand over), the rows being a column slice of a wider, 16-byte aligned buffer: the row stride is then at least
+    ``Hkv * D`` and says nothing about what the list means."""
+    from fourierattention_amd import _lib
+    from fourierattention_amd.midstore import MidStore
+    r = np.random.default_rng(1)
+    B, Hkv, D, S = 2, 4, 64, 70
+    n, _, _, _ = H.ragged_mask(r, Hkv, D, [20, 64, 0, 33])
+    nh = [0] + [int((n < (h + 1) * D).sum()) for h in range(Hkv)]
+    Cn = nh[-1]
+    wide = torch.randn((B, S, 512), device="cuda").to(torch.bfloat16)      # 512 >= Hkv * D = 256
+    gathered = wide[:, :, 8: 8 + Cn]                                       # (B, S, Cn) view, rows 1024 bytes apart
+    assert gathered.stride(1) >= Hkv * D and gathered.data_ptr() % 16 == 0
+    ident = torch.arange(Cn, dtype=torch.int32, device="cuda")
+    nh32 = torch.tensor(nh, dtype=torch.int32, device="cuda")
+    for is_v in (False, True):
+        st = MidStore(B, ident, nh32, nh, Hkv, D, S, torch.bfloat16, "cuda", is_v)
+        st.pack(gathered, 0, S)
+        assert torch.equal(st.dense(S), gathered)
+    # the other meaning of the list needs rows wide enough for every head
+    st = MidStore(B, ident, nh32, nh, Hkv, D, S, torch.bfloat16, "cuda", False)
+    with pytest.raises(_lib.FourierAttnError):
+        st.pack(wide[:, :, :128].contiguous(), 0, S, head_dims=True)
 
 
 MFMA_CASES = [
