@@ -16,6 +16,7 @@ FA_BF16, FA_FP16, FA_FP32 = 0, 1, 2
 FA_NO_ROUND = FA_FP32
 FA_MID_TOKEN_MAJOR, FA_MID_PAGED = 0, 1
 FA_COLS_ANY, FA_COLS_HEAD_DIMS = 0, 1
+DECODE_NOALLOC_SCRATCH_BYTES = 32 << 20
 PAGE_TOKENS, K_DIM_PAD, V_DIM_PAD = 32, 32, 16
 
 STATUS_NAMES = {
@@ -94,6 +95,7 @@ _SIGNATURES = {
                                 c_void_p]),
     "fa_decode_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "fa_decode_attn": (c_int, [POINTER(DecodeArgs), c_void_p]),
+    "fa_decode_attn_noalloc": (c_int, [POINTER(DecodeArgs), c_void_p]),
     "fa_decode_attn_timed": (c_int, [POINTER(DecodeArgs), c_void_p, POINTER(c_float)]),
     "fa_decode_tables_bytes": (c_size_t, [c_int]),
     "fa_decode_tables_build": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),

@@ -435,7 +435,7 @@ class DynamicCache(Cache):
 
     # -- attention over the cache's own buffers --------------------------------------
     def decode_attention(self, query_states: torch.Tensor, layer_idx: int, num_heads: int, num_kv_heads: int,
-                         sm_scale: float = -1.0, timings=None, out_dtype=None) -> torch.Tensor:
+                         sm_scale: float = -1.0, timings=None, out_dtype=None, out=None, no_alloc=False) -> torch.Tensor:
         """``query_states (B, Hq, 1, D)`` -> ``(B, Hq, 1, D)`` float32 over the current state of
         ``layer_idx`` (what modeling_llama_fourier.py:641-660 computes from the returned parts); with
         ``out_dtype = query_states.dtype`` the result comes back rounded to that type (the ``.to(dtype)`` of
@@ -446,9 +446,10 @@ class DynamicCache(Cache):
         l32 = self._lists32[layer_idx]
         if layer.window_only:
             return ops.decode_attn_raw(q, self._window_segments(layer), None, None, None, None, None, None, l32, num_heads,
-                                       num_kv_heads, 0, 1, sm_scale, timings=timings, out_dtype=out_dtype)
+                                       num_kv_heads, 0, 1, sm_scale, timings=timings, out_dtype=out_dtype, out=out,
+                                       no_alloc=no_alloc)
         segs = self._il_segments(layer)
         return ops.decode_attn_raw(q, segs, layer.k.coef, layer.v.coef, layer.k.mid, layer.v.mid, layer.k.stats32,
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
                                    sm_scale, tables=self._tables, force_generic=self.force_generic, timings=timings,
-                                   out_dtype=out_dtype)
+                                   out_dtype=out_dtype, out=out, no_alloc=no_alloc)

@@ -11,6 +11,7 @@
 #include <stdlib.h>
 
 #include "fa_common.h"
+#include <mutex>
 #include "fa_decode_mfma.h"
 
 namespace {
@@ -1281,6 +1282,54 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
 }
 
 extern "C" int fa_decode_attn(const fa_decode_args* a, fa_stream_t stream) { return decode_attn_impl(a, stream, nullptr); }
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------------
+// Device memory for the partial results of one decode call (what `workspace` brings in for fa_decode_attn), held
+// by every GPU the library runs on until the process ends.  In host code the array's name is a stand-in, not a
+// device address: the address on the current device comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) unsigned char scratch[FA_DECODE_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_on_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fa_set_error("fa_decode_attn_noalloc: no current device (or device index above %d)", kMaxDevices - 1);
+    return FA_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      fa_set_error("fa_decode_attn_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return FA_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FA_OK;
+}
+}  // namespace
+
+extern "C" int fa_decode_attn_noalloc(const fa_decode_args* a, fa_stream_t stream) {
+  FA_REQUIRE(a, FA_ERR_NULL_POINTER, "fa_decode_attn_noalloc: null argument block");
+  const size_t need = fa_decode_attn_workspace_bytes(a->B, a->Hq, a->Hkv, a->D, a->N, a->il_rows[0] + a->il_rows[1], a->L_m);
+  FA_REQUIRE(need > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn_noalloc: bad B/Hq/Hkv/D/N/row counts");
+  FA_REQUIRE(need <= (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES, FA_ERR_WORKSPACE,
+             "fa_decode_attn_noalloc: this shape needs %zu bytes of scratch, the built-in buffer holds %zu; use "
+             "fa_decode_attn with a workspace of the caller's", need, (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  int rc = scratch_on_current_device(&ptr);
+  if (rc != FA_OK) return rc;
+  fa_decode_args b = *a;
+  b.workspace = ptr;
+  b.workspace_bytes = (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES;
+  return decode_attn_impl(&b, stream, nullptr);
+}
 
 extern "C" int fa_decode_attn_timed(const fa_decode_args* a, fa_stream_t stream, float* ms_out) {
   FA_REQUIRE(ms_out, FA_ERR_NULL_POINTER, "fa_decode_attn_timed: ms_out null");

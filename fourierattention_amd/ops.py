@@ -315,14 +315,17 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
-                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None):
+                    T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None,
+                    no_alloc=False):
     """Thin call into ``fa_decode_attn``.  The result is float32 like the reference's (TRI:779) unless ``out_dtype``
     names the dtype of ``q``: then the merge launch rounds it to that type itself (the caller's ``.to(dtype)``).
 
     ``il_segments``: up to two ``(k, v)`` pairs of ``(B, rows, Hkv*D)`` views (last dim contiguous).
     ``k_mn`` / ``v_mn``: token-major ``(B, >=L_m, Cn)`` tensors or ``MidStore`` objects (paged).
     ``stats_*``: ``(avg_u, avg_d, scale)`` fp32 ``(B, C)``.  ``lists``: the eight int32 tensors
-    ``kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h`` (``*_h`` with the leading 0)."""
+    ``kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h`` (``*_h`` with the leading 0).
+    ``no_alloc``: call ``fa_decode_attn_noalloc`` (partial results in the library's own fixed buffer, no workspace
+    tensor; pass ``out`` as well and nothing is allocated on the device at all)."""
     from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
@@ -384,6 +387,9 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     a.sm_scale = float(sm_scale)
     a.dtype = dtype_code(q.dtype)
     lib = _lib.load()
+    if no_alloc:
+        check(lib.fa_decode_attn_noalloc(ctypes.byref(a), _stream(q.device)))
+        return out
     nbytes = lib.fa_decode_attn_workspace_bytes(B, num_head_q, num_head_kv, D, N, total_il, int(seq_len_m))
     ws = workspace(q.device, nbytes, "decode")
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()

@@ -277,6 +277,18 @@ int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_s
  * [sink ; local window ; mid rows (stored dims + dims rebuilt from coefficients)]. */
 int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
 
+/* fa_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  `args->workspace` and
+ * `args->workspace_bytes` are ignored; the partial results live in a buffer of FA_DECODE_NOALLOC_SCRATCH_BYTES
+ * that is part of the library image on every GPU it runs on (held until the process ends).  Nothing is allocated
+ * or freed, by this call or by anything it calls.  Shapes for which fa_decode_attn_workspace_bytes(...) exceeds
+ * that size are refused with FA_ERR_WORKSPACE.  Every call on one GPU shares that GPU's buffer: calls that may
+ * overlap on one GPU (two streams, two threads) race and must be serialised by the caller; consecutive calls on
+ * one stream are fine (every kernel writes what it later reads, nothing needs clearing).  The first call on a
+ * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture. */
+#define FA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
+
 /* Same call, bracketed by HIP events on `stream`; synchronises and returns in ms_out[0..3] the
  * milliseconds spent in (0) the coefficient-domain query kernel (plus the operand tables when
  * they are built in the workspace), (1) the mid-row kernel, (2) the sink/window kernel and

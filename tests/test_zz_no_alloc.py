@@ -1,0 +1,81 @@
+"""``fa_decode_attn_noalloc``: the decode-attention entry point that keeps its partial results in a buffer built into
+the library instead of a caller's workspace.  Called through the C ABI on the same operands as ``fa_decode_attn``,
+twice in a row with the second call on a smaller input (the buffer keeps the first call's contents), it must give
+the same result bit for bit: both run the same kernels with the same split of the work."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.cache_oracle import OracleCache
+from tests import helpers as H
+from tests.test_gpu_cache import _cfg, _masks
+
+
+def test_header_and_binding_agree_on_the_buffer_size():
+    import os
+    import re
+    from fourierattention_amd import _lib
+    text = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "fourier_attn_hip.h")).read()
+    m = re.search(r"#define FA_DECODE_NOALLOC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text)
+    assert m and int(m.group(1)) << int(m.group(2)) == _lib.DECODE_NOALLOC_SCRATCH_BYTES == 32 << 20
+
+
+def test_oversized_shape_is_refused_before_anything_is_touched():
+    """The streaming configuration (1024 frequencies, 131072 mid rows) needs about 100 MiB of partial results:
+    refused with the workspace code and a message that names both sizes.  Needs no GPU: the check comes first."""
+    from fourierattention_amd import _lib
+    lib = _lib.load()
+    a = _lib.DecodeArgs()
+    a.B, a.Hq, a.Hkv, a.D, a.N, a.L_m, a.q_len, a.T = 4, 24, 8, 128, 1024, 131072, 1, 131072
+    a.il_rows[0] = 1028
+    need = lib.fa_decode_attn_workspace_bytes(4, 24, 8, 128, 1024, 1028, 131072)
+    assert need > _lib.DECODE_NOALLOC_SCRATCH_BYTES
+    assert lib.fa_decode_attn_noalloc(ctypes.byref(a), None) == -4          # FA_ERR_WORKSPACE
+    msg = lib.fa_last_error_string().decode()
+    assert str(need) in msg and str(_lib.DECODE_NOALLOC_SCRATCH_BYTES) in msg
+    assert lib.fa_decode_attn_noalloc(None, None) == -1                     # FA_ERR_NULL_POINTER
+
+
+def _cache_case(dtype, B, Hq, Hkv, D, W, M, prompt, kcounts, vcounts, seed):
+    from fourierattention_amd import DynamicCache
+    masks = _masks(1, Hkv, D, kcounts, vcounts, seed=seed)
+    cfg = _cfg(masks, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=16, max_position_embeddings=1 << 20)
+    r = np.random.default_rng(seed)
+    k = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    v = H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)), dtype)
+    gpu, cpu = DynamicCache(cfg), OracleCache(cfg, masks=masks, model_dtype=H.NP_ROUND[dtype])
+    gpu.update(H.to_gpu(k, dtype), H.to_gpu(v, dtype), 0)
+    cpu.update(k, v, 0)
+    kn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+    vn = H.to_dtype_np(r.standard_normal((B, Hkv, 1, D)), dtype)
+    q = H.to_dtype_np(r.standard_normal((B, Hq, 1, D)), dtype)
+    gpu.update(H.to_gpu(kn, dtype), H.to_gpu(vn, dtype), 0)
+    kw, vw = cpu.update(kn, vn, 0)
+    for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average"):
+        getattr(cpu, n)[0] = getattr(gpu, n)[0].float().cpu().numpy()
+    want = cpu.attend(q, kw, vw, 0, Hq, Hkv)
+    return gpu, H.to_gpu(q, dtype), want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-3), (torch.float32, 2e-4)])
+def test_two_calls_in_a_row_match_the_entry_point_with_a_workspace(dtype, tol):
+    """bf16: the matrix-core kernels over the paged store; float32: the generic kernels.  The second call is a
+    smaller problem (fewer sequences, shorter context, fewer coefficient rows) that finds the first call's partial
+    results in the buffer."""
+    Hq, Hkv, D = 8, 2, 128
+    big = _cache_case(dtype, 5, Hq, Hkv, D, 64, 512, 3000, [64, 40], [64, 96], seed=1)
+    small = _cache_case(dtype, 2, Hq, Hkv, D, 32, 256, 700, [64, 64], [30, 64], seed=2)
+    for gpu, q, want in (big, small):
+        ref = gpu.decode_attention(q, 0, Hq, Hkv)                               # fa_decode_attn, caller's workspace
+        out = torch.full_like(ref, float("nan"))
+        got = gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True)       # fa_decode_attn_noalloc
+        assert got is out and torch.equal(got, ref)
+        err = np.abs(got.cpu().numpy() - want).max()
+        assert err <= 2e-2 and err <= tol, err
+    # and once more the larger one after the smaller: nothing of the smaller call's leftovers is read
+    gpu, q, want = big
+    out = torch.full((5, Hq, 1, D), float("nan"), device="cuda")
+    assert torch.equal(gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True), gpu.decode_attention(q, 0, Hq, Hkv))
