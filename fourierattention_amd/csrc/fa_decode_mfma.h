@@ -282,22 +282,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
 
   // Rotation constants of slice sl into LDS: one entry (row tile, pair of frequencies) per lane, requested early and
-  // stored once the other loads of the prologue are on their way.  Where both roles run, the value waves do it (they
-  // have time to spare before the first page).
-  float4v rot_one = float4v{0.f, 0.f, 0.f, 0.f}, rot_two = float4v{0.f, 0.f, 0.f, 0.f};
+  // stored once the other loads of the prologue are on their way.  Every wave stores the constants it reads itself
+  // (score waves the step of one page, value waves the step of their frame), so no wave waits for another one here.
+  float4v rot_c = float4v{0.f, 0.f, 0.f, 0.f};
   const bool rot_lane_ok = lane < 2 * KS * 4;
+  const bool rot_of_two = TWO && !score_wave;
   auto rot_fetch = [&]() {
     if (rot_lane_ok) {
       const int f = fbase + freq_of(lane >> 2, lane & 3, 0);   // even: (c, s)(f), (c, s)(f + 1) are 16 aligned bytes
-      rot_one = *(const float4v*)&p.rot[f];
-      if (TWO) rot_two = *(const float4v*)&p.rot[N + f];
+      rot_c = *(const float4v*)&p.rot[(rot_of_two ? N : 0) + f];
     }
   };
   auto rot_store = [&]() {
     if (rot_lane_ok) {
-      s_rot[(sl * 2 * KS) * 4 + lane] = rot_one;
-      if (TWO) s_rot2[(sl * 2 * KS) * 4 + lane] = rot_two;
+      if (rot_of_two) s_rot2[(sl * 2 * KS) * 4 + lane] = rot_c;
+      else s_rot[(sl * 2 * KS) * 4 + lane] = rot_c;
     }
+    asm volatile("" ::: "memory");   // the reads of these constants are asm statements the compiler cannot order
   };
 
   if (score_wave) {
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = 0; i < NST - 1; ++i)
         if (i < n_it) issue_k(t_beg + i);
     }
-    if (MODE == 1) rot_fetch();
+    rot_fetch();
     // the index list of the gathered query dims is requested now: the query loads that depend on it then go out
     // while the tables and the weights are still on their way, instead of starting a round trip of their own later
     int dim[KMAX][8];
@@ -419,8 +420,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
-    if (MODE == 1) rot_store();
-    __syncthreads();   // the rotation constants in LDS are complete
+    rot_store();
     const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
     // score pass: the complete scores of page pg of the split (sum of the eight partials; thread = (column,
     // token)) go to memory.  Called one page late, behind that page's barrier.
@@ -540,13 +540,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int f = 0; f < VMAX; ++f) oacc[f] = float4v{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, d_run = 0.f;
     const bool ragged_tail = (p.L_m & 31) != 0;
-    __syncthreads();   // the rotation constants in LDS are complete
-    // Only the rotation constants had to be there for the meeting above (the score waves need them for their first
-    // page); this wave's own operands may arrive while the score waves work on that page.  They must have landed
+    // This wave's own operands may arrive while the score waves work on the first page.  They must have landed
     // before the loop starts: inside it the only waits on vector memory are the explicit page waits.
     if (TWO) {
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) s_et1[(sl * 2 * KS + rt) * 64 + lane] = et1v[rt];
+      asm volatile("" ::: "memory");   // read back through asm statements
     }
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
