@@ -105,6 +105,9 @@ _SIGNATURES = {
                               c_int, c_int, c_int, c_int, c_void_p]),
     "fa_mid_unpack": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                               c_int, c_int, c_void_p]),
+    "fa_prefill_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "fa_prefill_attn": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int,
+                                c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "fa_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_void_p]),
     "fa_rope_qk": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_void_p]),

@@ -34,6 +34,9 @@ def _exact_attention(query_states, k_local, v_local, num_kv_heads, head_dim):
     modeling_llama_fourier.py:633; bottom-right aligned when ``q_len < kv_len``)."""
     B, Hq, q_len, D = query_states.shape
     S = k_local.shape[1]
+    if ops.prefill_attention_supported(query_states, k_local, head_dim) and v_local.stride() == k_local.stride():
+        return ops.prefill_attention(query_states, k_local, v_local, num_kv_heads)   # (B, q_len, Hq, D)
+    # other shapes (float32 storage, odd head dims) and the host-only tests: the framework's attention
     k = k_local.view(B, S, num_kv_heads, head_dim).transpose(1, 2)
     v = v_local.view(B, S, num_kv_heads, head_dim).transpose(1, 2)
     if q_len == S:

@@ -38,7 +38,9 @@ def audit_async_lds_reads(asm_text: str):
     registers do not hold the data, but the compiler believes they do and is free to copy them (it does when a
     read under a condition is merged with the other path).  The copy reads stale registers and nothing fails at
     build time, so every build checks the generated assembly: between such a read and the ``lgkmcnt`` wait
-    that covers it, no instruction outside an asm block may name its registers.  Returns the violations."""
+    that covers it, no instruction outside an asm block may name its registers.  The scan follows the layout of the
+    code, not its control flow: it runs straight through conditional branches and starts afresh behind an
+    unconditional one.  Returns the violations."""
     def regs(text):
         out = set()
         for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
@@ -65,6 +67,11 @@ def audit_async_lds_reads(asm_text: str):
         if not m:
             continue
         op, args = m.group(1), m.group(2)
+        if op in ("s_branch", "s_endpgm", "s_setpc_b64"):
+            # what follows is not reached by falling through: it is another block laid out here (a loop's exit
+            # after its body), entered from places of its own with their own outstanding reads
+            pending = []
+            continue
         if op == "s_waitcnt":
             mm = re.search(r"lgkmcnt\((\d+)\)", args)
             if mm:   # LDS operations complete in issue order: all but the last n are done

@@ -281,6 +281,37 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def prefill_attention_supported(q: torch.Tensor, k: torch.Tensor, head_dim: int) -> bool:
+    """Shapes the matrix-core prompt attention covers: 16-bit GPU tensors, heads of 64 or 128 dims, 16-byte rows."""
+    return (q.is_cuda and q.dtype in (torch.bfloat16, torch.float16) and k.dtype == q.dtype and head_dim in (64, 128)
+            and q.stride(-1) == 1 and k.stride(-1) == 1 and all(s % 8 == 0 for s in q.stride()[:-1])
+            and all(s % 8 == 0 for s in k.stride()[:-1]) and q.data_ptr() % 16 == 0 and k.data_ptr() % 16 == 0)
+
+
+def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_kv_heads: int, sm_scale: float = -1.0,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Exact causal attention of the prompt pass (modeling_llama_fourier.py:623-633, ``flash_attn_func(q, k, v,
+    causal=True)``).  ``q (B, Hq, q_len, D)`` (any strides with a contiguous last dim), ``k, v (B, S, Hkv*D)``
+    token-major with common strides; returns ``(B, q_len, Hq, D)`` in the dtype of ``q``.  Query row ``i`` sees keys
+    ``0 .. i + S - q_len``."""
+    _require_gpu(q, "q")
+    B, Hq, q_len, D = q.shape
+    S = k.shape[1]
+    assert k.shape == v.shape and k.stride() == v.stride() and k.shape[0] == B and k.shape[2] == num_kv_heads * D
+    assert prefill_attention_supported(q, k, D) and v.dtype == q.dtype and v.data_ptr() % 16 == 0, \
+        "prefill_attention: 16-bit GPU tensors, head_dim 64 or 128, 16-byte aligned rows"
+    if out is None:
+        out = torch.empty((B, q_len, Hq, D), dtype=q.dtype, device=q.device)
+    assert out.is_contiguous() and tuple(out.shape) == (B, q_len, Hq, D) and out.dtype == q.dtype
+    lib = _lib.load()
+    nbytes = lib.fa_prefill_attn_workspace_bytes(B, num_kv_heads, D, S)
+    ws = workspace(q.device, nbytes, "prefill")
+    check(lib.fa_prefill_attn(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), v.data_ptr(), k.stride(0),
+                              k.stride(1), out.data_ptr(), dtype_code(q.dtype), B, Hq, num_kv_heads, D, S, q_len,
+                              float(sm_scale), ws.data_ptr(), ws.numel(), _stream(q.device)))
+    return out
+
+
 class MultiDimHiPPO2(torch.nn.Module):
     """Same call contract as the reference class (TRI:840-865): without ``slice_input`` the
     whole ``base_input (B, L, C)`` is projected (period and length ``int(1/dt)``: longer inputs

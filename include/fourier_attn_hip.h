@@ -296,6 +296,25 @@ int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
 int fa_decode_attn_timed(const fa_decode_args* args, fa_stream_t stream, float* ms_out);
 
 /* ---------------------------------------------------------------------------
+ * Exact attention of the prompt pass
+ * ------------------------------------------------------------------------- */
+
+/* The other arm of the attention forward (MODEL:623-633): while the cache holds a layer's keys in full
+ * (`update` returned only `*_local`), attention is exact and causal - flash_attn_func(q, k, v, causal=True)
+ * in the reference.  q: (B, Hq, q_len, D) given by batch / head / row strides in elements with D contiguous
+ * (the transposed view of the projection output works as it is); k, v: token-major (B, S, Hkv*D) as `update`
+ * returns them, sharing their strides; out: (B, q_len, Hq, D) contiguous, of `dtype` (what the reference reshapes
+ * to (B, q_len, Hq*D), MODEL:663).  Query row i sees keys 0 .. i + (S - q_len) (bottom-right aligned, as
+ * flash-attn does when q_len < S).  16-bit dtypes, D in {64, 128}, rows 16-byte aligned; sm_scale <= 0 means
+ * 1/sqrt(D).  workspace: fa_prefill_attn_workspace_bytes(B, Hkv, D, S) bytes (a transposed copy of V in
+ * matrix-core operand order, written by a first launch). */
+size_t fa_prefill_attn_workspace_bytes(int B, int Hkv, int D, int S);
+int fa_prefill_attn(const void* q, int64_t q_batch_stride, int64_t q_head_stride, int64_t q_row_stride,
+                    const void* k, const void* v, int64_t kv_batch_stride, int64_t kv_row_stride, void* out,
+                    int dtype, int B, int Hq, int Hkv, int D, int S, int q_len, float sm_scale, void* workspace,
+                    size_t workspace_bytes, fa_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Elementwise steps of the decoder layer around the attention (one launch each)
  * ------------------------------------------------------------------------- */
 

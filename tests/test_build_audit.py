@@ -57,3 +57,41 @@ def test_copy_before_wait_is_reported():
 def test_counted_wait_releases_only_the_older_reads():
     found = audit_async_lds_reads(PARTIAL)
     assert len(found) == 1 and "v41" in found[0] and "v40" not in found[0]
+
+
+# a loop whose tail (with the wait) is laid out before its head and whose exit block follows the body: the exit is
+# entered from the loop's latch, where nothing is outstanding, not by falling through from the reads above it
+LOOP_EXIT_BEHIND_BODY = """
+_Zkernel_d:
+.LBB0_1:
+\t;;#ASMSTART
+\ts_waitcnt lgkmcnt(0)
+\t;;#ASMEND
+\tv_mul_f32_e32 v40, v28, v29
+\ts_cbranch_scc1 .LBB0_3
+.LBB0_2:
+\t;;#ASMSTART
+\tds_read_b128 v[28:31], v16 offset:0
+\t;;#ASMEND
+\ts_branch .LBB0_1
+.LBB0_3:
+\tv_accvgpr_read_b32 v29, a29
+\ts_endpgm
+"""
+
+FALLS_THROUGH_A_CONDITIONAL_BRANCH = """
+_Zkernel_e:
+\t;;#ASMSTART
+\tds_read_b128 v[28:31], v16 offset:0
+\t;;#ASMEND
+\ts_cbranch_scc1 .LBB0_3
+\tv_mov_b32_e32 v5, v30
+.LBB0_3:
+\ts_endpgm
+"""
+
+
+def test_scan_restarts_behind_an_unconditional_branch_only():
+    assert audit_async_lds_reads(LOOP_EXIT_BEHIND_BODY) == []
+    found = audit_async_lds_reads(FALLS_THROUGH_A_CONDITIONAL_BRANCH)
+    assert len(found) == 1 and "v_mov_b32_e32 v5, v30" in found[0]
