@@ -218,6 +218,31 @@ def compress_bench(device, reps=20):
             "operand_dtype": "f16 (basis and data), fp32 accumulation"}
 
 
+def prefill_attn_bench(device, S=32768, reps=5):
+    """Exact causal attention of the prompt pass (one layer of Llama-3.1-8B geometry, B=1, bf16) on the matrix-core
+    kernel, both launches (the transposing pass over V and the attention itself): matrix-core roofline."""
+    from fourierattention_amd import ops
+    B, Hq, Hkv, D = 1, 32, 8, 128
+    g = torch.Generator(device=device).manual_seed(0)
+    q = torch.randn((B, Hq, S, D), device=device, generator=g).to(torch.bfloat16)
+    k = torch.randn((B, S, Hkv * D), device=device, generator=g).to(torch.bfloat16)
+    v = torch.randn((B, S, Hkv * D), device=device, generator=g).to(torch.bfloat16)
+    for _ in range(2):
+        ops.prefill_attention(q, k, v, Hkv)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        ops.prefill_attention(q, k, v, Hkv)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    flops = 4.0 * D * Hq * B * S * (S + 1) / 2     # QK^T and PV over the causal half
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"workload": f"prompt attention, B=1, {S} tokens, Hq=32, Hkv=8, D=128, causal", "ms_per_layer": round(ms, 4),
+            "bound": "mfma", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4),
+            "algorithmic_flops": flops, "operand_dtype": "bf16, fp32 accumulation"}
+
+
 E2E = {
     # BASELINE configs 4 and 5: a random-init decoder with the Fourier cache on every layer
     "config4_e2e_8b_64k": dict(preset="llama-3.1-8b", B=16, prompt=65536, new=128, I=4, W=1024, M=1024, cper=64),
@@ -442,6 +467,7 @@ def main():
                                "algorithmic_bytes": upd_bytes, "GB_s": round(upd_bytes / (upd_ms * 1e-3) / 1e9, 1)}
     del cache, q, kn, vn, out
     result["prefill_compress"] = compress_bench(device)
+    result["prefill_attn"] = prefill_attn_bench(device)
     if not args.no_e2e and args.workload.startswith("config3"):
         # BASELINE configs 4 and 5 end to end (a few seconds each); the headline value above stays config 3
         result["e2e"] = {}
