@@ -2,8 +2,9 @@
 (compressed_dims_search/compressed_dim_search.py:135-161, 239-269, 321-397 with the transform of
 compressed_dims_search/hippo_function_approx_legt_fourier_awq.py:335-393), restated on this package's kernels.
 
-The reference hooks ``k_proj`` / ``v_proj`` of a model running calibration text; here the projection outputs
-are an argument (``(B, S, Hkv*D)`` tensors per layer), so the search runs on whatever produced them.  Per dim it
+``search`` takes the projection outputs as an argument (``(B, S, Hkv*D)`` tensors per layer), so it runs on
+whatever produced them; ``search_model`` is the reference's driver: it hooks ``k_proj`` / ``v_proj`` of a model that
+runs calibration samples (compressed_dim_search.py:195-291) and feeds the same scoring.  Per dim the search
 measures how well the middle of the sequence survives compress -> reconstruct -> mean / maximum-deviation
 matching, ranks the dims by that error and marks the best ``percent`` of them as compressible.  The output is
 the reference's raw mask format; ``masks.splithead_from_raw`` turns it into what the cache loads.
@@ -68,16 +69,72 @@ def search(layers_kv: Iterable[Tuple[Sequence[torch.Tensor], Sequence[torch.Tens
     compressible dims) and ``errors[(i, "k" | "v")]`` the mean error per dim over the samples."""
     layers_kv = list(layers_kv)
     n_layers = num_layers if num_layers is not None else len(layers_kv)
-    raw, errors = {}, {}
+    errors = {}
     for i, (ks, vs) in enumerate(layers_kv):
-        raw[f"Layer_{i}"] = {}
-        for tag, name, samples in (("k", "self_attn.k_proj", ks), ("v", "self_attn.v_proj", vs)):
+        for tag, samples in (("k", ks), ("v", vs)):
             acc = None
             for sample in samples:
                 e = reconstruction_mse(sample, numinittokens, maxlocallen, maxmidstates)[0]
                 acc = e if acc is None else acc + e
-            mean = acc / len(samples)
-            errors[(i, tag)] = mean
+            if acc is not None:
+                errors[(i, tag)] = acc / len(samples)
+    return _select(errors, n_layers, percents), errors
+
+
+def _select(errors, n_layers: int, percents) -> dict:
+    """The raw mask of every measured layer from its mean errors (compressed_dim_search.py:321-397); ``n_layers`` is
+    the depth of the model the layers belong to (it places them in the schedule of fractions)."""
+    raw = {}
+    for i in sorted({layer for layer, _ in errors}):
+        raw[f"Layer_{i}"] = {}
+        for tag, name in (("k", "self_attn.k_proj"), ("v", "self_attn.v_proj")):
+            if (i, tag) not in errors:
+                continue
             pct = percents[(i, tag)] if percents and (i, tag) in percents else percent_schedule(i, tag, n_layers)
-            raw[f"Layer_{i}"][name] = select_noncritical(mean, pct)
-    return raw, errors
+            raw[f"Layer_{i}"][name] = select_noncritical(errors[(i, tag)], pct)
+    return raw
+
+
+@torch.no_grad()
+def search_model(model, samples: Sequence[torch.Tensor], numinittokens: int = 4, maxlocallen: int = 1024,
+                 maxmidstates: int = 1024, percents: Optional[Dict[Tuple[int, str], float]] = None):
+    """The reference's driver (compressed_dim_search.py:164-291) on a decoder of ``fourierattention_amd.llama``:
+    every calibration sample (token ids ``(1, S)``, ``S > numinittokens + maxlocallen``) runs through the model's
+    prompt pass with a forward hook on ``k_proj`` and ``v_proj`` of every layer.  The hook recomputes the projection
+    from the module's input and weight (before the rotary embedding, compressed_dim_search.py:243-247) and scores
+    it at once, so no projection output outlives its layer; the errors are averaged over the samples and the best
+    dims of every layer selected (compressed_dim_search.py:321-397).  Returns ``(raw, errors)`` like ``search``."""
+    import torch.nn.functional as F
+    from . import masks as pm
+    from .cache import DynamicCache, ExtraConfig
+    cfg = model.config
+    layers = model.model.layers
+    sums: Dict[Tuple[int, str], torch.Tensor] = {}
+
+    def hook(module, inputs, output, layer_idx, tag):
+        proj = F.linear(inputs[0], module.weight)                  # independent of the module's own output
+        e = reconstruction_mse(proj, numinittokens, maxlocallen, maxmidstates)[0]
+        key = (layer_idx, tag)
+        sums[key] = e if key not in sums else sums[key] + e
+
+    handles = []
+    for i, layer in enumerate(layers):
+        for tag, mod in (("k", layer.self_attn.k_proj), ("v", layer.self_attn.v_proj)):
+            handles.append(mod.register_forward_hook(lambda m, a, o, i=i, tag=tag: hook(m, a, o, i, tag)))
+    fused = model.model.fused_elementwise
+    model.model.fused_elementwise = False     # the module chain calls k_proj / v_proj themselves
+    try:
+        placeholder = pm.synthetic_masks(len(layers), cfg.num_key_value_heads, cfg.head_dim, cfg.head_dim // 2, seed=0)
+        for sample in samples:
+            assert sample.dim() == 2 and sample.shape[0] == 1, "one calibration sample at a time: (1, S) token ids"
+            # a cache whose window holds the whole sample: the prompt pass is plain causal attention
+            ec = ExtraConfig(numinittokens=0, maxlocallen=sample.shape[1] + 1, maxmidstates=2, non_critical_dims=placeholder,
+                             non_critical_dims_path=None, max_position_embeddings=sample.shape[1] + 128,
+                             num_key_value_heads=cfg.num_key_value_heads, max_new_tokens=64, model_type="llama")
+            model.model(sample, DynamicCache(ec, device=sample.device))
+    finally:
+        model.model.fused_elementwise = fused
+        for h in handles:
+            h.remove()
+    errors = {key: total / len(samples) for key, total in sums.items()}
+    return _select(errors, len(layers), percents), errors

@@ -58,3 +58,44 @@ def test_reconstruction_error_matches_the_reference_formulation_and_ranks_smooth
     sp = masks.splithead_from_raw(raw, Hkv, D)
     masks.validate_layer(sp["Layer_0"], Hkv, D)
     assert sp["Layer_0"]["kc_h_list"] == [D // 2, D]
+
+
+@pytest.mark.gpu
+def test_model_hook_driver_scores_the_projections_before_the_rotary_embedding():
+    """``search_model`` against ``search`` fed with the same projections taken by hand: the hooks see ``k_proj`` /
+    ``v_proj`` of every layer for every sample, the flags of the model and its hooks are left as they were."""
+    import torch.nn.functional as F
+    from fourierattention_amd import dim_search
+    from fourierattention_amd.llama import LlamaConfig, random_init
+    cfg = LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=16, vocab_size=97)
+    model = random_init(cfg, dtype=torch.bfloat16, device="cuda", seed=5, std=0.3)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    samples = [torch.randint(0, 97, (1, n), generator=g, device="cuda") for n in (200, 260)]
+    kw = dict(numinittokens=4, maxlocallen=64, maxmidstates=32)
+    raw, errors = dim_search.search_model(model, samples, **kw)
+    assert model.model.fused_elementwise is True
+    assert all(len(m._forward_hooks) == 0 for m in model.modules())
+    # the same projections by hand: the input of a layer's attention is its normalised residual stream
+    taken = [([], []) for _ in range(3)]
+    hooks = []
+    for i, layer in enumerate(model.model.layers):
+        def grab(m, a, o, i=i):
+            x = a[0]
+            taken[i][0].append(F.linear(x, model.model.layers[i].self_attn.k_proj.weight))
+            taken[i][1].append(F.linear(x, model.model.layers[i].self_attn.v_proj.weight))
+        hooks.append(layer.self_attn.q_proj.register_forward_hook(grab))
+    model.model.fused_elementwise = False
+    from fourierattention_amd import DynamicCache, ExtraConfig, masks as pm
+    for s_ in samples:
+        ec = ExtraConfig(numinittokens=0, maxlocallen=s_.shape[1] + 1, maxmidstates=2, non_critical_dims_path=None,
+                         non_critical_dims=pm.synthetic_masks(3, 2, 16, 8), max_position_embeddings=s_.shape[1] + 128,
+                         num_key_value_heads=2, max_new_tokens=64, model_type="llama")
+        model.model(s_, DynamicCache(ec, device="cuda"))
+    for h in hooks:
+        h.remove()
+    raw2, errors2 = dim_search.search(taken, **kw)
+    assert raw == raw2 and set(raw) == {"Layer_0", "Layer_1", "Layer_2"}
+    for key in errors:
+        assert torch.equal(errors[key], errors2[key])
+    assert len(raw["Layer_0"]["self_attn.k_proj"]) == int(dim_search.percent_schedule(0, "k", 3) * 32)
