@@ -34,6 +34,30 @@ WORKLOADS = {
     "config5_decode_attn_3b_128k": dict(B=4, ctx=131072, Hq=24, Hkv=8, D=128, I=4, W=1024, M=2048, cper=64, max_new=512),
     "config1_cpu_geometry_3b_2k": dict(B=1, ctx=2048, Hq=24, Hkv=8, D=128, I=4, W=512, M=256, cper=64, max_new=64),
 }
+# Config 3 with the head-by-head counts of three layers of the mask the reference ships for this model and
+# context (compressed_dims_32k_1024states_splithead.json: compressed dims per KV head, K and V; which dims of a head
+# they are is drawn from a seed, the kernels only see the counts and the gathers)
+_RAGGED = {
+    "layer0": ([121, 124, 103, 127, 128, 117, 83, 118], [115, 122, 119, 126, 122, 125, 122, 121]),
+    "layer15": ([83, 116, 117, 96, 122, 88, 116, 81], [120, 128, 110, 111, 8, 122, 128, 92]),
+    "layer31": ([47, 86, 44, 60, 75, 64, 69, 67], [82, 127, 124, 61, 114, 1, 81, 126]),
+}
+for _name, (_kc, _vc) in _RAGGED.items():
+    WORKLOADS[f"config3_ragged_{_name}"] = dict(WORKLOADS["config3_decode_attn_8b_32k"], cper=None, kc_heads=_kc, vc_heads=_vc)
+
+
+def compressed_counts(w):
+    """Compressed dims of a whole row (all KV heads), K and V."""
+    if w.get("kc_heads"):
+        return sum(w["kc_heads"]), sum(w["vc_heads"])
+    return w["cper"] * w["Hkv"], w["cper"] * w["Hkv"]
+
+
+def workload_masks(w, layers, seed):
+    from fourierattention_amd import masks
+    if w.get("kc_heads"):
+        return masks.synthetic_masks(layers, w["Hkv"], w["D"], w["kc_heads"], w["vc_heads"], seed=seed)
+    return masks.synthetic_masks(layers, w["Hkv"], w["D"], w["cper"], seed=seed)
 
 
 def algorithmic_bytes(w, coef_bytes=4, elem_bytes=2):
@@ -41,9 +65,8 @@ def algorithmic_bytes(w, coef_bytes=4, elem_bytes=2):
     sink+window K,V (all dims) + stored dims of the mid rows (K,V) + coefficients (K,V) + q + out."""
     L = w["ctx"] - w["I"] - w["W"]
     hd = w["Hkv"] * w["D"]
-    ck = w["cper"] * w["Hkv"]
-    cn = hd - ck
-    per_b = 2 * (w["I"] + w["W"]) * hd * elem_bytes + 2 * L * cn * elem_bytes + 2 * w["M"] * ck * coef_bytes \
+    ck, cv = compressed_counts(w)
+    per_b = 2 * (w["I"] + w["W"]) * hd * elem_bytes + L * (2 * hd - ck - cv) * elem_bytes + w["M"] * (ck + cv) * coef_bytes \
         + 2 * w["Hq"] * w["D"] * elem_bytes
     return per_b * w["B"]
 
@@ -51,8 +74,8 @@ def algorithmic_bytes(w, coef_bytes=4, elem_bytes=2):
 def build_cache(w, dtype, device, seed=0, layers=1):
     """Random K/V of the workload's shape pushed through the cache's own prefill (split, spectral
     compression, statistics), so the timed decode reads exactly what a real prompt leaves behind."""
-    from fourierattention_amd import DynamicCache, ExtraConfig, masks, synth
-    m = masks.synthetic_masks(layers, w["Hkv"], w["D"], w["cper"], seed=seed)
+    from fourierattention_amd import DynamicCache, ExtraConfig, synth
+    m = workload_masks(w, layers, seed)
     cfg = ExtraConfig(numinittokens=w["I"], maxlocallen=w["W"], maxmidstates=w["M"], non_critical_dims=m,
                       non_critical_dims_path=None, max_position_embeddings=MODEL_MAX_POSITIONS, num_key_value_heads=w["Hkv"],
                       max_new_tokens=w["max_new"], model_type="llama")
@@ -420,7 +443,7 @@ def main():
     gbs = nbytes / (ms * 1e-3) / 1e9
     L = w["ctx"] - w["I"] - w["W"]
     hd = w["Hkv"] * w["D"]
-    ck = w["cper"] * w["Hkv"]
+    ck, cv = compressed_counts(w)
     # per-kernel durations, HIP events recorded inside the library on the launch stream
     reps = max(10, min(50, args.steps))
     per = np.zeros(4)
@@ -435,14 +458,14 @@ def main():
     # algorithmic bytes of each kernel's own launch
     kbytes = {
         "query_and_sink_window": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4 + w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,
-        "mid_rows": w["B"] * 2 * L * (hd - ck) * 2,
-        "merge": w["B"] * w["M"] * ck * 4,
+        "mid_rows": w["B"] * L * (2 * hd - ck - cv) * 2,
+        "merge": w["B"] * w["M"] * cv * 4,
     }
     dom = max(kernel_ms, key=kernel_ms.get)
     dom_gbs = kbytes[dom] / (kernel_ms[dom] * 1e-3) / 1e9
     traffic, traffic_source = recorded_traffic(dom, args.workload)
     full = 2 * w["ctx"] * hd * 2
-    fourier = 2 * (w["I"] + w["W"]) * hd * 2 + 2 * L * (hd - ck) * 2 + 2 * w["M"] * ck * 4
+    fourier = 2 * (w["I"] + w["W"]) * hd * 2 + L * (2 * hd - ck - cv) * 2 + w["M"] * (ck + cv) * 4
     result = {
         "metric": "Fourier decode attn HBM GB/s (% peak) + tok/s, Llama-3.1-8B geometry, 32k ctx",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -450,7 +473,8 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "batch": w["B"], "context": w["ctx"], "q_heads": Hq, "kv_heads": Hkv,
                    "head_dim": w["D"], "sink": w["I"], "window": w["W"], "coeff_rows": w["M"],
-                   "compressed_dims_per_head": w["cper"], "coeff_dtype": "f32"},
+                   "compressed_dims_per_head": w["cper"] if w["cper"] else {"k": w["kc_heads"], "v": w["vc_heads"]},
+                   "coeff_dtype": "f32"},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "attn_only_tok_s": round(w["B"] / (args.layers * ms * 1e-3), 1),
         "kv_bytes_per_layer_per_seq": {"full_bf16": full, "fourier": fourier, "reduction": round(full / fourier, 3)},
@@ -490,7 +514,7 @@ def main():
         cache.update(kn, vn, 0)
     torch.cuda.synchronize()
     upd_wall = (time.perf_counter() - t0) / 50
-    upd_bytes = w["B"] * 2 * 2 * w["M"] * ck * 4
+    upd_bytes = w["B"] * 2 * w["M"] * (ck + cv) * 4
     # a decode step in use: the streaming update, then the attention over the updated cache
     for _ in range(5):
         cache.update(kn, vn, 0)

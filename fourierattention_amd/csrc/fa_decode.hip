@@ -1036,8 +1036,8 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
   const int NSL = table_slices(N), KS = N / (16 * NSL);
   half8* tabE = (half8*)tables;
   half8* tabET = tabE + NSL * 2 * KS * 64;
-  float2v* rot = (float2v*)(tabET + 2 * NSL * 2 * KS * 64);
-  const int total = 3 * NSL * 2 * KS * 64 + 2 * N;
+  float2v* rot = (float2v*)(tabET + NSL * 2 * KS * 64);
+  const int total = tables_entries(N) + N;
   decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N, NSL);
 }
 
@@ -1116,7 +1116,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.tabE = (const half8*)tables;
         const int NSL = table_slices(a.N);
         mp.tabET = mp.tabE + NSL * 2 * KS * 64;
-        mp.rot = (const float2v*)(mp.tabET + 2 * NSL * 2 * KS * 64);
+        mp.rot = (const float2v*)(mp.tabET + NSL * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.scores = (float*)(ws + p.off_scores);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;

@@ -5,12 +5,21 @@
 // range of 32-token pages.  Per page:
 //
 //   scores  S[32 x 16] = E[32 x 2N] . W'[2N x 16]      (f16 MFMA; E = cos/sin of the token offset
-//                        + K_mn[32 x dims] . Q_n        inside the page, W' = coefficient-domain
-//                                                        query rotated to the page start)
+//                        + K_mn[32 x dims] . Q_n        from the centre of the frame, W' = coefficient-domain
+//                                                        query rotated to that centre)
 //   softmax P = exp2(S - m)                              (online, base 2)
 //   g'[2N x 16] += E^T[2N x 32] . P                      (f16 MFMA, accumulated in the frame of the
-//                                                        current page: rotated by one page step first)
+//                                                        current pair of pages)
 //   o_n[dims x 16] += V_mn^T[dims x 32] . P              (bf16 / f16 MFMA on the stored dims)
+//
+// Frames.  Two pages share one frame whose centre lies half a token before the first token of the second
+// page: its tokens sit at the offsets +(i + 1/2), those of the first page at -(i + 1/2), i = 0 .. 31.  Cosine is
+// even and sine is odd, so ONE constant operand E (offsets i + 1/2) serves both pages: on the first ("mirrored")
+// page the sine rows of W' enter negated and row i of the product is token 31 - i; for g the sine tiles take
+// -P.  W' and the g history are rotated once per frame (64 tokens), not once per page.  On a mirrored page every
+// position-indexed quantity (score partials in LDS, probabilities) is held in the mirrored order; the K and V
+// pages come into LDS through per-lane addresses, so fetching a K fragment with its 16 rows reversed (and the two
+// 16-token blocks exchanged) or a V fragment with its four groups of 8 tokens exchanged costs nothing.
 //
 // The 2N coefficient rows are split four ways; slice i belongs to score wave i (E, W') and to
 // value wave i (E^T, g'), which share a SIMD.  The score waves work one page ahead of the value
@@ -35,16 +44,17 @@ constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one 
 
 // ---------------------------------------------------------------------------
 // constant operand tables (depend on T and N only); KS = N / (16 * slices) ksteps per frequency slice
-//   tabE  [slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM
-//   tabET [2 pages][slices][2*KS row tiles][64 lanes] x half8 : A operand of the g GEMM for the tokens of
-//         a page (0) and for the tokens of the page after it seen from the same page start (1)
-//   rot   [2][N] float2 : (cos, sin)(2 pi f 32 / T) and (cos, sin)(2 pi f 64 / T), the frame rotation of one
-//         page step and of two
+//   tabE  [slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM, row i = offset i + 1/2
+//   tabET [slices][2*KS tiles][64 lanes] x half8 : A operand of the g GEMM; tile 2j holds the cosines and tile
+//         2j + 1 the sines of the 16 frequencies 16j .. 16j + 15 of the slice (row = frequency), columns = the
+//         offsets i + 1/2
+//   rot   [N] float2 : (cos, sin)(2 pi f 64 / T), the rotation from one frame to the next
+// Half-token offsets: phase f (2i + 1) / (2T), reduced exactly in integers.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ tabE, half8* __restrict__ tabET,
                                                             float2v* __restrict__ rot, int KS, int T, int N, int NSL) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  const int nE = NSL * 2 * KS * 64, nET = 2 * NSL * 2 * KS * 64;
+  const int nE = NSL * 2 * KS * 64, nET = NSL * 2 * KS * 64;
   if (idx < nE) {
     const int lane = idx & 63, s = (idx >> 6) % KS, rb = ((idx >> 6) / KS) & 1, w = (idx >> 6) / (2 * KS);
     const int lg = lane >> 4, lc = lane & 15;
@@ -55,40 +65,40 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
       const int v = e >> 1, cs = e & 1;
       const int f = w * 16 * KS + freq_of(2 * s + (v >> 1), lg, v & 1);
       float sn, co;
-      fa_sincos_phase(f, i, T, &sn, &co);
+      fa_sincos_phase(f, 2 * i + 1, 2 * T, &sn, &co);
       out[e] = (_Float16)(cs ? sn : co);
     }
     tabE[idx] = out;
   } else if (idx < nE + nET) {
     const int k = idx - nE;
-    const int lane = k & 63, rt = (k >> 6) % (2 * KS), w = ((k >> 6) / (2 * KS)) % NSL;
-    const int page = (k >> 6) / (2 * KS * NSL);
-    const int lg = lane >> 4, rho = lane & 15;
-    const int f = w * 16 * KS + freq_of(rt, rho >> 2, (rho & 3) >> 1);
-    const int cs = rho & 1;
+    const int lane = k & 63, tile = (k >> 6) % (2 * KS), w = (k >> 6) / (2 * KS);
+    const int lg = lane >> 4;
+    const int f = w * 16 * KS + 16 * (tile >> 1) + (lane & 15);
+    const int cs = tile & 1;
     half8 out;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float sn, co;
-      fa_sincos_phase(f, 32 * page + 8 * lg + e, T, &sn, &co);
+      fa_sincos_phase(f, 2 * (8 * lg + e) + 1, 2 * T, &sn, &co);
       out[e] = (_Float16)(cs ? sn : co);
     }
     tabET[k] = out;
-  } else if (idx < nE + nET + 2 * N) {
-    const int f = (idx - nE - nET) % N, two = (idx - nE - nET) / N;
+  } else if (idx < nE + nET + N) {
+    const int f = idx - nE - nET;
     float sn, co;
-    fa_sincos_phase(f, 32 * (1 + two), T, &sn, &co);
-    rot[two * N + f] = float2v{co, sn};
+    fa_sincos_phase(f, 64, T, &sn, &co);
+    rot[f] = float2v{co, sn};
   }
 }
 
 // frequency slices: four (one per SIMD, score and value wave of a slice side by side) up to N = 512; eight for
 // N = 1024, whose per-wave state only fits when a pass runs one role on all eight waves
 static inline int table_slices(int N) { return N > 512 ? 8 : 4; }
-static inline size_t tables_bytes(int N) {
+static inline int tables_entries(int N) {
   const int NSL = table_slices(N), KS = N / (16 * NSL);
-  return (size_t)(3 * NSL * 2 * KS * 64) * 16 + (size_t)2 * N * 8;
+  return 2 * NSL * 2 * KS * 64;   // half8 operands of tabE and tabET together
 }
+static inline size_t tables_bytes(int N) { return (size_t)tables_entries(N) * 16 + (size_t)N * 8; }
 
 
 // ---- page-step rotation of coefficient-domain state ---------------------------------------------------
@@ -181,20 +191,17 @@ __device__ __forceinline__ void rot_apply(unsigned lane_base, uint4v (&rc)[NBUF]
   rot_apply_from<NT, NBUF, 0>(lane_base, rc, pair, pin);
 }
 
-// hacc[rt] += A[rt] . pf for the second page of a frame: the A operands (E^T of token offsets 32..63) come from
-// LDS four row tiles at a time (1 KiB apart per row tile)
-template <int NT, int RT0>
-__device__ __forceinline__ void et1_accumulate(unsigned lane_base, half8 pf, float4v (&hacc)[NT], uint4v (&a)[4]) {
-  if constexpr (RT0 < NT) {
-    a[0] = lds_read_b128_async_at<(RT0 + 0) * 1024>(lane_base);
-    a[1] = lds_read_b128_async_at<(RT0 + 1) * 1024>(lane_base);
-    a[2] = lds_read_b128_async_at<(RT0 + 2) * 1024>(lane_base);
-    a[3] = lds_read_b128_async_at<(RT0 + 3) * 1024>(lane_base);
-    lds_wait_for4<0>(a);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      hacc[RT0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a[j]), pf, hacc[RT0 + j], 0, 0, 0);
-    et1_accumulate<NT, RT0 + 4>(lane_base, pf, hacc, a);
+// Wait until at most AHEAD pages of PER * n fragment loads each are still in flight (n is uniform over the wave,
+// 1 .. NMAX; the count of the wait instruction is an immediate, hence one branch per possible value).
+template <int AHEAD, int NMAX, int PER, int F = 1>
+__device__ __forceinline__ void wait_pages_in_flight(int n) {
+  if constexpr (AHEAD == 0) {
+    wait_vmcnt<0>();
+  } else if constexpr (F >= NMAX) {
+    wait_vmcnt<AHEAD * PER * NMAX>();
+  } else {
+    if (n == F) wait_vmcnt<AHEAD * PER * F>();
+    else wait_pages_in_flight<AHEAD, NMAX, PER, F + 1>(n);
   }
 }
 
@@ -227,9 +234,11 @@ struct MidParams {
 
 // The workgroup is a two-stage pipeline over the pages of its split, one barrier per page:
 //   waves 0-3 ("score waves")  page t+1: S partial = E . W' (their frequency slice) + K_mn . Q_n (their batch
-//                              element) -> LDS; then advance W' by one page step
-//   waves 4-7 ("value waves")  page t  : sum the four partials, online softmax, rotate/rescale the g history,
-//                              g' += E^T . P (their frequency slice), o_n += V_mn^T . P (their batch element)
+//                              element) -> LDS; after the second page of a frame, W' moves on to the next frame
+//   waves 4-7 ("value waves")  page t  : sum the four partials, online softmax, before the first page of a frame
+//                              rotate the g history into it, rescale, g' += E^T . P (their frequency slice),
+//                              o_n += V_mn^T . P (their batch element)
+// Pages at an even distance from the first page of the split are the mirrored pages of their frames.
 // Score wave i and value wave i own the same frequencies and stream the same batch element of the group.
 // KS: ksteps (32 coefficient rows) per slice = N / (16 * slices).  KMAX: ksteps of stored K dims a head may have
 // (dp_k / 32).  VMAX: V dim groups of 16 (dp_v / 16).
@@ -252,12 +261,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // in the two-pass modes only waves 0-3 stream pages
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[MODE == 0 ? 8 : 4][NST][kFragsMax * 1024];
   __shared__ float s_part[MODE == 2 ? 1 : 2][MODE == 2 ? 1 : NSL][16 * kPart];
-  __shared__ float4v s_rot[NSL * 2 * KS * 4];  // [slice][row tile][lane group] = (c, s) pair 0, (c, s) pair 1
-  // Narrow pages leave LDS for a second g operand: the value waves then accumulate two pages per frame (the second
-  // through E^T of the token offsets 32..63, read from LDS) and rotate their history every other page only.
-  constexpr bool TWO = MODE == 0 && kFragsMax <= 4;
-  __shared__ float4v s_rot2[TWO ? kFreqWaves * 2 * KS * 4 : 1];   // the same for a step of two pages
-  __shared__ uint4v s_et1[TWO ? kFreqWaves * 2 * KS * 64 : 1];    // [slice][row tile][lane]
+  // frame-to-frame rotation constants, float4 = (c, s) of two neighbouring frequencies, [slice][unit][lane group]:
+  // for the score waves unit = row tile rt, frequencies freq_of(rt, lg, 0 / 1); for the value waves unit u covers
+  // the frequencies 16 (u / 2) + 4 lg + 2 (u % 2) + 0 / 1, the rows 4 lg + 2 (u % 2) + 0 / 1 of tile pair u / 2
+  __shared__ float4v s_rot[MODE == 2 ? 1 : NSL * 2 * KS * 4];
+  __shared__ float4v s_rotv[MODE == 1 ? 1 : NSL * 2 * KS * 4];
 
   const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
@@ -281,25 +289,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int t_end = min(n_tiles, t_beg + p.tiles_per_split);
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
 
-  // Rotation constants of slice sl into LDS: one entry (row tile, pair of frequencies) per lane, requested early and
-  // stored once the other loads of the prologue are on their way.  Every wave stores the constants it reads itself
-  // (score waves the step of one page, value waves the step of their frame), so no wave waits for another one here.
+  // Rotation constants of slice sl into LDS: one entry (unit, lane group) per lane, requested early and stored once
+  // the other loads of the prologue are on their way.  Every wave stores the constants it reads itself (in the
+  // order of its own role), so no wave waits for another one here.
   float4v rot_c = float4v{0.f, 0.f, 0.f, 0.f};
   const bool rot_lane_ok = lane < 2 * KS * 4;
-  const bool rot_of_two = TWO && !score_wave;
   auto rot_fetch = [&]() {
     if (rot_lane_ok) {
-      const int f = fbase + freq_of(lane >> 2, lane & 3, 0);   // even: (c, s)(f), (c, s)(f + 1) are 16 aligned bytes
-      rot_c = *(const float4v*)&p.rot[(rot_of_two ? N : 0) + f];
+      const int u = lane >> 2, ulg = lane & 3;
+      // even: (c, s)(f), (c, s)(f + 1) are 16 aligned bytes
+      const int f = fbase + (score_wave ? freq_of(u, ulg, 0) : 16 * (u >> 1) + 4 * ulg + 2 * (u & 1));
+      rot_c = *(const float4v*)&p.rot[f];
     }
   };
   auto rot_store = [&]() {
     if (rot_lane_ok) {
-      if (rot_of_two) s_rot2[(sl * 2 * KS) * 4 + lane] = rot_c;
-      else s_rot[(sl * 2 * KS) * 4 + lane] = rot_c;
+      if (score_wave) s_rot[(MODE == 2 ? 0 : sl * 2 * KS) * 4 + lane] = rot_c;
+      else s_rotv[(MODE == 1 ? 0 : sl * 2 * KS) * 4 + lane] = rot_c;
     }
     asm volatile("" ::: "memory");   // the reads of these constants are asm statements the compiler cannot order
   };
+  // per-lane element offsets of a fragment load: as stored, with the 16 rows of a K fragment reversed, with the four
+  // token groups of a V fragment exchanged
+  const int lane_nat = lane * 8, lane_krev = (lg * 16 + 15 - lc) * 8, lane_vrev = ((3 - lg) * 16 + lc) * 8;
 
   if (score_wave) {
     // =============================== score waves ===============================
@@ -310,20 +322,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int nks = dpk >> 5;
     const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
     const bool has_k = has_mn && nks > 0;
-    // a page moves the fragments the head really has (two stages: the page wait below is always "all landed")
-    auto issue_k = [&](int t) {            // page t -> stage (t - t_beg) % NST
-      const E* kp = kbase + (int64_t)t * dpk * 32;
+    // a page moves the fragments the head really has
+    // (mirrored page: token 31 - i becomes row i, i.e. the blocks change places and their rows are reversed)
+    auto issue_k = [&](int t, bool mir) {   // page t -> stage (t - t_beg) % NST
+      const E* kp = kbase + (int64_t)t * dpk * 32 + (mir ? lane_krev : lane_nat);
       unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
         for (int ks = 0; ks < KMAX; ++ks)
-          if (ks < nks) load_frag_to_lds<2>(kp + (tb * nks + ks) * 512 + lane * 8, st + (tb * KMAX + ks) * 1024);
+          if (ks < nks) load_frag_to_lds<2>(kp + ((mir ? 1 - tb : tb) * nks + ks) * 512, st + (tb * KMAX + ks) * 1024);
     };
     if (has_k) {
 #pragma unroll
       for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_k(t_beg + i);
+        if (i < n_it) issue_k(t_beg + i, (i & 1) == 0);
     }
     rot_fetch();
     // the index list of the gathered query dims is requested now: the query loads that depend on it then go out
@@ -339,7 +352,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     half8 Ea[2][KS];
 
     // coefficient-domain query: Wc/Ws[rt][f2] = (cos-row, sin-row) weights of frequency
-    // freq_of(rt, lg, f2) for column lc; normalised per column, rotated to the first page
+    // freq_of(rt, lg, f2) for column lc; normalised per column, rotated to the centre of the first frame
     float Wc[2 * KS][2], Ws[2 * KS][2];
     float wmax = 0.f;
     // the gathered query values: requested behind the weights, needed only once those have been processed
@@ -381,11 +394,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float colinv = 1.0f / colscale;
     const float c0col = (valid_r && sl == 0) ? p.c0[qrow] : 0.f;
     {
-      // phases of the first page: exact for row tile 0, then stepped by the (exact) phase of 8 frequencies
+      // phases of the first frame centre (token 32 (t_beg + 1) - 1/2, as a count of half tokens against 2T): exact
+      // for row tile 0, then stepped by the (exact) phase of 8 frequencies
+      const int64_t c2 = (int64_t)64 * (t_beg + 1) - 1;
       float sn[2], co[2], s8, c8;
-      fast_sincos_phase(8, (int64_t)32 * t_beg, p.T, &s8, &c8);
+      fast_sincos_phase(8, c2, 2 * p.T, &s8, &c8);
 #pragma unroll
-      for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), (int64_t)32 * t_beg, p.T, &sn[f2], &co[f2]);
+      for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), c2, 2 * p.T, &sn[f2], &co[f2]);
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt)
 #pragma unroll
@@ -421,7 +436,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
     rot_store();
-    const unsigned rot_lane = lds_addr_of(&s_rot[(sl * 2 * KS) * 4 + lg]);
+    const unsigned rot_lane = lds_addr_of(&s_rot[(MODE == 2 ? 0 : sl * 2 * KS) * 4 + lg]);
     // score pass: the complete scores of page pg of the split (sum of the eight partials; thread = (column,
     // token)) go to memory.  Called one page late, behind that page's barrier.
     auto flush_scores = [&](int pg) {
@@ -432,7 +447,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     };
 
-    for (int it = 0; it <= n_it; ++it) {
+    // one trip of the score pipeline: page `it` of the split (none on the trip after the last page)
+    auto score_trip = [&](int it, auto mirrored_tag) {
+      constexpr bool mirrored = decltype(mirrored_tag)::value;   // first page of its frame
       if (it < n_it) {
         const int t = t_beg + it;
         uint4v kraw[4];   // two ksteps of both token blocks at a time
@@ -440,9 +457,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         uint4v rc[2][4];
         if (has_k) {
           // pages t+1 .. t+NST-2 may still be in flight; page t has landed: start its LDS reads now
-          if (it + NST - 2 < n_it) wait_vmcnt<(NST - 2) * 2 * KMAX>();
+          if (it + NST - 2 < n_it) wait_pages_in_flight<NST - 2, KMAX, 2>(nks);   // (two fragments per kstep)
           else wait_vmcnt<0>();
-          if (it + NST - 1 < n_it) issue_k(t + NST - 1);   // refills the stage read one page ago
+          // refills the stage read one page ago
+          if (it + NST - 1 < n_it) issue_k(t + NST - 1, mirrored == (((NST - 1) & 1) == 0));
         }
         // The results of these reads arrive later (the wait is tied to them further down); until then no
         // instruction may touch their registers.  A read under a condition makes the compiler merge its result
@@ -456,22 +474,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           kraw[3] = lds_read_b128_async_at<(KMAX + 1) * 1024>(kst);
         }
         if (it > 0) flush_scores(it - 1);   // behind the page wait: the store has a whole page to complete
-        rot_issue<0>(rot_lane, rc[0]);
-        if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
+        if constexpr (!mirrored) {
+          rot_issue<0>(rot_lane, rc[0]);
+          if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
+        }
         float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
+        // The two pages of a frame convert the same W': without this the conversions of the second page are done
+        // together with those of the first and their results held across a whole page.
+#pragma unroll
+        for (int rt = 0; rt < 2 * KS; ++rt)
+          asm volatile("" : "+v"(Wc[rt][0]), "+v"(Wc[rt][1]), "+v"(Ws[rt][0]), "+v"(Ws[rt][1]));
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
           half8 wb;
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
+            const float ws = Ws[2 * s + (v >> 1)][v & 1];
             wb[2 * v] = (_Float16)Wc[2 * s + (v >> 1)][v & 1];
-            wb[2 * v + 1] = (_Float16)Ws[2 * s + (v >> 1)][v & 1];
+            wb[2 * v + 1] = (_Float16)(mirrored ? -ws : ws);   // offsets -(i + 1/2): the sines change sign
           }
           accf[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][s], wb, accf[0], 0, 0, 0);
           accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
         }
-        // advance W' by one page step
-        rot_apply_in_place_from<2 * KS, 0>(rot_lane, rc, Wc, Ws);
+        // behind the second page of a frame: W' moves on to the centre of the next frame
+        if constexpr (!mirrored) rot_apply_in_place_from<2 * KS, 0>(rot_lane, rc, Wc, Ws);
         float4v accm[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
         if (has_k) {
 #pragma unroll
@@ -503,6 +529,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         flush_scores(it - 1);
       }
       if (MODE == 0 || it < n_it) barrier_lds_only();
+    };
+    for (int it = 0; it <= n_it; it += 2) {
+      score_trip(it, std::true_type{});
+      if (it + 1 <= n_it) score_trip(it + 1, std::false_type{});
     }
   } else {
     // =============================== value waves ===============================
@@ -510,28 +540,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int ndg = dpv >> 4;
     const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
     const bool streams_v = has_mn && ndg > 0;
-    auto issue_v = [&](int t) {            // page t -> stage (t - t_beg) % NST
-      const E* vp = vbase + (int64_t)t * dpv * 32;
+    // (mirrored page: lane group lg takes the tokens of group 3 - lg; the probabilities follow, see below)
+    auto issue_v = [&](int t, bool mir) {   // page t -> stage (t - t_beg) % NST
+      const E* vp = vbase + (int64_t)t * dpv * 32 + (mir ? lane_vrev : lane_nat);
       unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
 #pragma unroll
       for (int f = 0; f < VMAX; ++f)
-        if (f < ndg) load_frag_to_lds<2>(vp + f * 512 + lane * 8, st + f * 1024);
+        if (f < ndg) load_frag_to_lds<2>(vp + f * 512, st + f * 1024);
     };
     if (streams_v) {   // first pages requested before the tables (see the score waves)
 #pragma unroll
       for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_v(t_beg + i);
+        if (i < n_it) issue_v(t_beg + i, (i & 1) == 0);
     }
     rot_fetch();
-    uint4v et1v[TWO ? 2 * KS : 1];   // E^T of the second page of a frame, on its way to LDS
-    half8 ETa[2 * KS];
+    half8 ETa[2 * KS];   // tile 2j: cosines, tile 2j + 1: sines of the frequencies 16j .. 16j + 15 of the slice
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
-    if (TWO) {
-      const uint4v* src = (const uint4v*)(p.tabET + (kFreqWaves + sl) * 2 * KS * 64) + lane;
-#pragma unroll
-      for (int rt = 0; rt < 2 * KS; ++rt) et1v[rt] = src[rt * 64];
-    }
     rot_store();
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
@@ -542,15 +567,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool ragged_tail = (p.L_m & 31) != 0;
     // This wave's own operands may arrive while the score waves work on the first page.  They must have landed
     // before the loop starts: inside it the only waits on vector memory are the explicit page waits.
-    if (TWO) {
-#pragma unroll
-      for (int rt = 0; rt < 2 * KS; ++rt) s_et1[(sl * 2 * KS + rt) * 64 + lane] = et1v[rt];
-      asm volatile("" ::: "memory");   // read back through asm statements
-    }
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
-    const unsigned rot_lane = lds_addr_of(TWO ? &s_rot2[(sl * 2 * KS) * 4 + lg] : &s_rot[(sl * 2 * KS) * 4 + lg]);
-    const unsigned et1_lane = lds_addr_of(&s_et1[TWO ? (sl * 2 * KS) * 64 + lane : 0]);
+    const unsigned rot_lane = lds_addr_of(&s_rotv[(MODE == 1 ? 0 : sl * 2 * KS) * 4 + lg]);
     // value pass: the scores of a page (column lc, tokens 8*lg .. 8*lg+7) are fetched one page ahead
     float4v sc_next[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
     const float* sc_src = nullptr;
@@ -569,7 +588,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int t = t_beg + it - 1, buf = (it - 1) & 1;
         const int pg = it - 1;   // page index within the split
         constexpr int RCB = VMAX > 4 ? 1 : 2;   // the wide variant has no registers to spare for a second batch
-        constexpr bool first_of_frame = decltype(first_tag)::value;   // first page of a frame (rotates), or second
+        constexpr bool first_of_frame = decltype(first_tag)::value;   // the mirrored page of a frame (rotates), or the second
         uint4v rc[RCB][4];
         if constexpr (first_of_frame) {
           rot_issue<0>(rot_lane, rc[0]);
@@ -586,27 +605,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           }
         }
         if constexpr (has_v) {
-          if (pg + NST - 2 < n_it) wait_vmcnt<(NST - 2) * VMAX>();
+          if (pg + NST - 2 < n_it) wait_pages_in_flight<NST - 2, VMAX, 1>(ndg);
           else wait_vmcnt<0>();
-          if (pg + NST - 1 < n_it) issue_v(t + NST - 1);   // refills the stage read one page ago
+          // refills the stage read one page ago
+          if (pg + NST - 1 < n_it) issue_v(t + NST - 1, first_of_frame == (((NST - 1) & 1) == 0));
         }
         if constexpr (MODE == 2) {
           const float* nx = sc_src + (int64_t)min(pg + 1, n_it - 1) * 512;   // clamped: the load is unconditional
           sc_next[0] = *(const float4v*)nx;
           sc_next[1] = *(const float4v*)(nx + 4);
         }
-        // the g history moves into the frame of this page (of this pair of pages)
+        // the g history moves into the frame of this pair of pages: unit u of the constants belongs to the rows
+        // 2 (u % 2) + f2 of the cosine tile 2 (u / 2) and of the sine tile behind it
         if constexpr (first_of_frame)
-        rot_apply<2 * KS, RCB>(rot_lane, rc, [&](int rt, int f2, float c, float sn) {
-          float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
+        rot_apply<2 * KS, RCB>(rot_lane, rc, [&](int u, int f2, float c, float sn) {
+          float x = hacc[2 * (u >> 1)][2 * (u & 1) + f2], y = hacc[2 * (u >> 1) + 1][2 * (u & 1) + f2];
           rot_pair(c, sn, x, y);
-          hacc[rt][2 * f2] = x;
-          hacc[rt][2 * f2 + 1] = y;
+          hacc[2 * (u >> 1)][2 * (u & 1) + f2] = x;
+          hacc[2 * (u >> 1) + 1][2 * (u & 1) + f2] = y;
           return y;
         }, [&](int b) {
           asm volatile("" : "+v"(hacc[4 * b]), "+v"(hacc[4 * b + 1]), "+v"(hacc[4 * b + 2]), "+v"(hacc[4 * b + 3]));
         });
-        // scores of the page in B-operand layout (column lc, tokens 8*lg + e): four partials to sum
+        // scores of the page in B-operand layout (column lc, positions 8*lg + e; on a mirrored page position i is
+        // token 31 - i): four partials to sum
         if constexpr (MODE == 0) {
           uint4v part[kFreqWaves][2];
           const unsigned pst = lds_addr_of(&s_part[buf][0][lc * kPart + 8 * lg]);
@@ -641,10 +663,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           vraw[3] = lds_read_b128_async_at<3072>(vst);
         }
         if (ragged_tail && t == n_tiles - 1) {
-          const int tok0 = t * 32 + 8 * lg;
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (tok0 + e >= p.L_m) sc[e] = -INFINITY;
+          for (int e = 0; e < 8; ++e) {
+            const int tok = t * 32 + (first_of_frame ? 31 - 8 * lg - e : 8 * lg + e);
+            if (tok >= p.L_m) sc[e] = -INFINITY;
+          }
         }
         float tmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
         tmax = fa_rows_max(tmax);
@@ -657,13 +680,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first page
         float psum = 0.f;
         half8 pf;
-        vec8 pe;
+        vec8 pe;   // for the V fragments, whose lane group lg holds the tokens of positions 8 lg + 7 - e on a mirrored page
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float pv = __builtin_amdgcn_exp2f(sc[e] - m_new);
           psum += pv;
           pf[e] = (_Float16)pv;
-          pe[e] = (typename M::elem)pv;
+          pe[first_of_frame ? 7 - e : e] = (typename M::elem)pv;
         }
         d_run = d_run * alpha + psum;
         m_run = m_new;
@@ -674,13 +697,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int f = 0; f < VMAX; ++f) oacc[f] *= alpha;
         }
-        if constexpr (first_of_frame) {
 #pragma unroll
-          for (int rt = 0; rt < 2 * KS; ++rt)
-            hacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[rt], pf, hacc[rt], 0, 0, 0);
-        } else {
-          et1_accumulate<2 * KS, 0>(et1_lane, pf, hacc, rc[0]);   // the constant buffer is idle on these pages
+        for (int j = 0; j < KS; ++j)
+          hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], pf, hacc[2 * j], 0, 0, 0);
+        if constexpr (first_of_frame) {
+          // offsets -(i + 1/2): the sine tiles take -P (the sign bits of the eight halves, flipped in place once
+          // the cosine tiles have been issued)
+          uint4v neg = __builtin_bit_cast(uint4v, pf);
+          asm volatile("" : "+v"(neg));
+          neg ^= uint4v{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+          pf = __builtin_bit_cast(half8, neg);
         }
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+          hacc[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j + 1], pf, hacc[2 * j + 1], 0, 0, 0);
         if constexpr (has_v) {
 #pragma unroll
           for (int f0 = 0; f0 < VMAX; f0 += 4) {
@@ -701,8 +731,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     };
     auto value_loop = [&](auto stream_tag) {
       if constexpr (MODE == 2) {
-        for (int it = 1; it <= n_it; ++it) value_page(it, std::true_type{}, stream_tag);
-      } else if constexpr (TWO) {
+        for (int it = 1; it <= n_it; it += 2) {
+          value_page(it, std::true_type{}, stream_tag);
+          if (it + 1 <= n_it) value_page(it + 1, std::false_type{}, stream_tag);
+        }
+      } else {
         barrier_lds_only();   // iteration 0: the score waves are one page ahead
         for (int it = 1; it <= n_it; it += 2) {
           value_page(it, std::true_type{}, stream_tag);
@@ -711,12 +744,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             value_page(it + 1, std::false_type{}, stream_tag);
             barrier_lds_only();
           }
-        }
-      } else {
-        barrier_lds_only();   // iteration 0: the score waves are one page ahead
-        for (int it = 1; it <= n_it; ++it) {
-          value_page(it, std::true_type{}, stream_tag);
-          barrier_lds_only();
         }
       }
     };
@@ -733,29 +760,38 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
     {
-      // g of this split, back from the page frame (rotation by +phi), in the layout it is held in:
-      // [batch group][KV head][split][slice][row tile][column][pair of frequencies] x {cos f, sin f, cos f+1,
-      // sin f+1}: every store is one contiguous KiB (the columns of one batch element lie side by side for the
-      // merge); lanes of columns past the group store values that nobody reads
-      float4v* gl = (float4v*)p.pg + ((((int64_t)(grp * p.Hkv + h) * p.n_split + split) * NSL + sl) * 2 * KS) * 64 + (lc * 4 + lg);
-      const int64_t last = (int64_t)32 * (t_end > t_beg ? t_beg + (TWO ? ((n_it - 1) & ~1) : n_it - 1) : t_beg);
-      float sn[2], co[2], s8, c8;   // stepped phases, as for the first page
-      fast_sincos_phase(8, last, p.T, &s8, &c8);
+      // g of this split, back from its last frame (rotation by +phi of the frame centre), in the layout the merge
+      // reads: [batch group][KV head][split][slice][row tile rt][column][lane group lg'] x {cos f, sin f, cos f+1,
+      // sin f+1} with f = 8 rt + 2 lg' (the layout of the weights W).  This lane holds the frequencies
+      // 16 j + 4 lg + v, v = 0 .. 3, of tile pair j: rt = 2 j + lg / 2, lg' = 2 (lg % 2) + v / 2.  Lanes of columns
+      // past the group store values that nobody reads.
+      float4v* gl = (float4v*)p.pg + ((((int64_t)(grp * p.Hkv + h) * p.n_split + split) * NSL + sl) * 2 * KS) * 64 + lc * 4;
+      // twice the centre of the last frame, in half tokens
+      const int64_t c2 = (int64_t)64 * (t_beg + (n_it > 0 ? ((n_it - 1) & ~1) : 0) + 1) - 1;
+      float sn[4], co[4], s16, c16;   // stepped phases, as for the first frame of the score waves
+      fast_sincos_phase(16, c2, 2 * p.T, &s16, &c16);
 #pragma unroll
-      for (int f2 = 0; f2 < 2; ++f2) fast_sincos_phase(fbase + freq_of(0, lg, f2), last, p.T, &sn[f2], &co[f2]);
+      for (int v = 0; v < 4; ++v) fast_sincos_phase(fbase + 4 * lg + v, c2, 2 * p.T, &sn[v], &co[v]);
 #pragma unroll
-      for (int rt = 0; rt < 2 * KS; ++rt) {
-        float4v o;
+      for (int j = 0; j < KS; ++j) {
 #pragma unroll
-        for (int f2 = 0; f2 < 2; ++f2) {
-          const float x = hacc[rt][2 * f2], y = hacc[rt][2 * f2 + 1];
-          o[2 * f2] = co[f2] * x - sn[f2] * y;
-          o[2 * f2 + 1] = sn[f2] * x + co[f2] * y;
-          const float cn = co[f2] * c8 - sn[f2] * s8;
-          sn[f2] = sn[f2] * c8 + co[f2] * s8;
-          co[f2] = cn;
+        for (int h2 = 0; h2 < 2; ++h2) {
+          float4v o;
+#pragma unroll
+          for (int f2 = 0; f2 < 2; ++f2) {
+            const int v = 2 * h2 + f2;
+            const float x = hacc[2 * j][v], y = hacc[2 * j + 1][v];
+            o[2 * f2] = co[v] * x - sn[v] * y;
+            o[2 * f2 + 1] = sn[v] * x + co[v] * y;
+          }
+          gl[(2 * j + (lg >> 1)) * 64 + 2 * (lg & 1) + h2] = o;
         }
-        gl[rt * 64] = o;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float cn = co[v] * c16 - sn[v] * s16;
+          sn[v] = sn[v] * c16 + co[v] * s16;
+          co[v] = cn;
+        }
       }
     }
     if (valid_r) {

@@ -64,17 +64,21 @@ def splithead_from_raw(raw: Dict[str, Dict[str, List[int]]], num_kv_heads: int, 
     return out
 
 
-def synthetic_masks(num_layers: int, num_kv_heads: int, head_dim: int, k_per_head: int, v_per_head: int = None,
-                    seed: int = 0):
-    """Seeded masks compressing exactly ``k_per_head`` / ``v_per_head`` dims of every head."""
+def synthetic_masks(num_layers: int, num_kv_heads: int, head_dim: int, k_per_head, v_per_head=None, seed: int = 0):
+    """Seeded masks compressing exactly ``k_per_head`` / ``v_per_head`` dims of every head (an int, or one count per
+    head for masks whose heads differ)."""
     v_per_head = k_per_head if v_per_head is None else v_per_head
+    per = lambda c: [int(c)] * num_kv_heads if np.isscalar(c) else [int(x) for x in c]
+    k_cnt, v_cnt = per(k_per_head), per(v_per_head)
+    if len(k_cnt) != num_kv_heads or len(v_cnt) != num_kv_heads:
+        raise ValueError(f"one count per KV head expected ({num_kv_heads})")
     rng = np.random.default_rng(seed)
     out = {}
     for i in range(num_layers):
         kc, vc = [], []
         for h in range(num_kv_heads):
-            kc += (h * head_dim + np.sort(rng.choice(head_dim, k_per_head, replace=False))).tolist()
-            vc += (h * head_dim + np.sort(rng.choice(head_dim, v_per_head, replace=False))).tolist()
+            kc += (h * head_dim + np.sort(rng.choice(head_dim, k_cnt[h], replace=False))).tolist()
+            vc += (h * head_dim + np.sort(rng.choice(head_dim, v_cnt[h], replace=False))).tolist()
         out[f"Layer_{i}"] = layer_from_compressed(kc, vc, num_kv_heads, head_dim)
     return out
 
