@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void prefill_vt_kernel(const E* __restrict__ v
 }
 
 template <typename E, int D, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void prefill_attn_kernel(const PrefillParams<E> p) {
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) void prefill_attn_kernel(const PrefillParams<E> p) {
   using M = Mma<E>;
   using vec8 = typename M::vec8;
   constexpr int KS = D / 32, DG = D / 16;
@@ -89,17 +89,31 @@ __global__ __launch_bounds__(64 * WAVES) void prefill_attn_kernel(const PrefillP
   // this wave's share of a tile: fragments w, w + WAVES, ... (clamped to the last one: every wave issues OPS loads)
   const E* kb_base = p.k + (int64_t)b * p.k_bs + (int64_t)kvh * D + 8 * lg;
   const E* vt_base = p.vt + ((int64_t)b * p.Hkv + kvh) * p.n_tiles * (int64_t)(kTileKeys * D) + lane * 8;
+  // The tiles are requested in order, so every load keeps a running pointer that moves on by one tile; only a last
+  // tile that reaches past the keys computes its (clamped) rows afresh.
+  const E* run[OPS];
+#pragma unroll
+  for (int i = 0; i < OPS; ++i) {
+    const int f = min(w + i * WAVES, NF - 1);
+    if (f < 2 * KS) run[i] = kb_base + (int64_t)(16 * (f / KS) + lc) * p.k_rs + 32 * (f % KS);
+    else run[i] = vt_base + (int64_t)(f - 2 * KS) * 512;
+  }
+  const int64_t k_step = (int64_t)kTileKeys * p.k_rs;
+  const bool ragged_keys = (p.S % kTileKeys) != 0;
   auto issue = [&](int t, int buf) {
+    const bool clamp = ragged_keys && t == p.n_tiles - 1;   // wave-uniform
 #pragma unroll
     for (int i = 0; i < OPS; ++i) {
       const int f = min(w + i * WAVES, NF - 1);
-      const E* src;
+      const E* src = run[i];
       if (f < 2 * KS) {
-        const int kb = f / KS, ks = f - kb * KS;
-        const int key = min(t * kTileKeys + 16 * kb + lc, p.S - 1);
-        src = kb_base + (int64_t)key * p.k_rs + 32 * ks;
+        if (clamp) {
+          const int key = min(t * kTileKeys + 16 * (f / KS) + lc, p.S - 1);
+          src = kb_base + (int64_t)key * p.k_rs + 32 * (f % KS);
+        }
+        run[i] += k_step;
       } else {
-        src = vt_base + ((int64_t)t * DG + (f - 2 * KS)) * 512;
+        run[i] += DG * 512;
       }
       load_frag_to_lds(src, &s_tile[buf][f * 1024]);
     }
@@ -190,10 +204,11 @@ __global__ __launch_bounds__(64 * WAVES) void prefill_attn_kernel(const PrefillP
     float alpha[2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
-      float s[8];
+      float s[8];   // raw products: the softmax scale rides in the instruction that subtracts the reference
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s[e] = sacc[e >> 2][rb][e & 3] * p.sm_log2e;
+      for (int e = 0; e < 8; ++e) s[e] = sacc[e >> 2][rb][e & 3];
       if (edge) {
+        asm volatile("");   // a real branch: as selects these masks would run on every tile
         const int row_lim = r0 + 16 * rb + lc + offset;   // last key this row may see
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -202,14 +217,14 @@ __global__ __launch_bounds__(64 * WAVES) void prefill_attn_kernel(const PrefillP
         }
       }
       float tmax = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-      tmax = fa_rows_max(tmax);
+      tmax = fa_rows_max(tmax) * p.sm_log2e;   // (the scale is positive)
       const float m_new = fmaxf(m_run[rb], tmax);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a row that has seen no key yet
       alpha[rb] = __builtin_amdgcn_exp2f(m_run[rb] - m_use);   // 0 on the row's first tile
       float psum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float pv = __builtin_amdgcn_exp2f(s[e] - m_use);
+        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], p.sm_log2e, -m_use));
         psum += pv;
         pb[rb][e] = (typename M::elem)pv;
       }
