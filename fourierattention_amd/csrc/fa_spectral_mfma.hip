@@ -216,8 +216,11 @@ __global__ __launch_bounds__(256) void spectral_reduce_kernel(const float* __res
 //   r[k, m] = (1/N) sum_n cos(theta k n) c[n, m] + sin(theta k n) c[N + n, m] = (1/N) Re sum_n e^{i theta k n} (c - i s)
 // is the compression GEMM with the roles of position and frequency exchanged: the rows are the positions k,
 // the "tokens" are the N coefficient indices.  A workgroup owns 128 positions, keeps their basis rows in
-// registers, and walks over every block of 64 columns: one pass over the cos coefficients (keeps the real part),
-// one over the sin coefficients (adds the imaginary part), then folds its positions into sum / max / min.
+// registers, and walks over every block of 64 columns: one pass over the cos coefficients (keeps the real part A_k),
+// one over the sin coefficients (keeps the imaginary part B_k), then folds its positions into sum / max / min.
+// Position k gives r[k] = A_k + B_k and, because the period is a whole number of positions, also its mirror image
+// r[T - k] = A_k - B_k: only the positions up to T / 2 are computed, each standing for two where the sequence
+// reaches past T / 2.
 // The coefficients travel as f16 scaled by a power of two per column (their range is not bounded).
 // ---------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void coef_colscale_kernel(const float* __restrict__ c, float* __restrict__ scale,
@@ -255,6 +258,9 @@ struct ReconStatsParams {
   float* pmax;
   float* pmin;             // [B][RB][Mc]
   int B, N, Mc, CT, KS32, K, T, n_steps, RB;
+  int Kd;     // positions computed directly: min(K, T / 2 + 1)
+  int half;   // T / 2: mirror images beyond it count as positions of their own (a value no position exceeds
+              // when the sequence is longer than the period and every position is computed directly)
 };
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void spectral_recon_stats_kernel(
@@ -266,7 +272,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb = blockIdx.x, b = blockIdx.y;
   const int rt0 = (rb * 4 + w) * 4;
-  const int n_rt = (p.K + 7) / 8;
+  const int n_rt = (p.Kd + 7) / 8;
   const int S = p.n_steps;
   const int n_cb = (p.Mc + kWgCols - 1) / kWgCols;
   const int Q = n_cb * 2 * S;   // steps of this workgroup: column block, pass (cos, sin), step (last to first)
@@ -350,7 +356,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
       continue;
     }
-    // both passes done for this column block: r = (re + im) * scale / N at this lane's 8 positions per column
+    // both passes done for this column block: r = (re +- im) * scale / N at this lane's 8 positions per column and
+    // at their mirror images
+    const int half = p.half;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int m = (cb * 4 + j) * 16 + lc;
@@ -362,10 +370,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int f2 = 0; f2 < 2; ++f2) {
           const int k = (rt0 + i) * 8 + lg * 2 + f2;
           const float r = (re[i][j][f2] + acc[i][j][2 * f2 + 1]) * sc;
-          if (k < p.K) {
+          if (k < p.Kd) {
             sum += r;
             mx = fmaxf(mx, r);
             mn = fminf(mn, r);
+          }
+          const int km = p.T - k;   // the mirror image counts where it is a position of its own beyond T / 2
+          const float r2 = (re[i][j][f2] - acc[i][j][2 * f2 + 1]) * sc;
+          if (k < p.Kd && km > half && km < p.K) {
+            sum += r2;
+            mx = fmaxf(mx, r2);
+            mn = fminf(mn, r2);
           }
         }
       sum = fa_rows_sum(sum);
@@ -498,7 +513,11 @@ int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int 
   *psum = (float*)(ws + pl.off_sum);
   *pmax = (float*)(ws + pl.off_max);
   *pmin = (float*)(ws + pl.off_min);
-  const int kp8 = fa_cdiv(K, 8) * 8;
+  // positions 0 .. T / 2 stand for their mirror images as well (unless the sequence is longer than the period)
+  const bool mirror = K <= T + 1;
+  const int Kd = mirror && T / 2 + 1 < K ? T / 2 + 1 : K;
+  const int RBd = fa_cdiv(Kd, kWgFreqs);
+  const int kp8 = fa_cdiv(Kd, 8) * 8;
   spectral_table_kernel<<<fa_cdiv((kp8 / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, kp8, T);
   coef_colscale_kernel<<<dim3(fa_cdiv(Mc, 64), B), 1024, 0, st>>>(c, scale, inv, 2 * N, Mc);
   dim3 pgrid(pl.KS32, fa_cdiv(Mc, 256), B);
@@ -508,7 +527,9 @@ int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int 
   ReconStatsParams rp{};
   rp.tab = tab; rp.packed[0] = pc; rp.packed[1] = ps; rp.scale = scale;
   rp.psum = *psum; rp.pmax = *pmax; rp.pmin = *pmin;
-  rp.B = B; rp.N = N; rp.Mc = Mc; rp.CT = pl.CT; rp.KS32 = pl.KS32; rp.K = K; rp.T = T; rp.n_steps = pl.n_steps; rp.RB = pl.RB;
-  spectral_recon_stats_kernel<<<dim3(pl.RB, B), 256, 0, st>>>(rp);
-  return pl.RB;
+  rp.B = B; rp.N = N; rp.Mc = Mc; rp.CT = pl.CT; rp.KS32 = pl.KS32; rp.K = K; rp.T = T; rp.n_steps = pl.n_steps; rp.RB = RBd;
+  rp.Kd = Kd;
+  rp.half = mirror ? T / 2 : 0x7fffffff;
+  spectral_recon_stats_kernel<<<dim3(RBd, B), 256, 0, st>>>(rp);
+  return RBd;
 }

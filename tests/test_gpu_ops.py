@@ -199,7 +199,13 @@ def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
     assert rel_err(got2.cpu().numpy(), 2 * got.cpu().numpy()) <= 1e-6
 
 
-@pytest.mark.parametrize("B,L,C,N,T", [(2, 1500, 70, 40, 1533), (1, 4100, 128, 128, 4100), (1, 1100, 16, 200, 5000)])
+@pytest.mark.parametrize("B,L,C,N,T", [
+    (2, 1500, 70, 40, 1533),     # most positions beyond T / 2 are taken as mirror images, odd period
+    (1, 4100, 128, 128, 4100),   # a whole even period: position T / 2 is its own image, position 0 has none
+    (1, 1100, 16, 200, 5000),    # nothing beyond T / 2
+    (1, 1202, 16, 64, 1201),     # one position more than the period: position T is the image of position 0
+    (1, 1300, 16, 64, 1201),     # longer than the period: every position is computed directly
+])
 def test_stats_reconstructed_matrix_cores(B, L, C, N, T):
     """Long reconstructions take the matrix-core kernel (fp16 basis and per-column scaled fp16 coefficients, fp32
     accumulation): statistics against the oracle and against the fp32 vector kernel.  Bound: each operand carries
