@@ -93,6 +93,41 @@ def audit_async_lds_reads(asm_text: str):
     return found
 
 
+# sources whose kernels issue LDS reads from inline asm (directly or through fa_decode_mfma.h): their assembly must
+# show such reads, or the audit above has looked at nothing
+ASYNC_LDS_SOURCES = ("fa_decode", "fa_prefill", "fa_spectral_mfma")
+
+
+def count_async_lds_reads(asm_text: str) -> int:
+    """Inline-asm ``ds_read`` instructions in a gfx950 assembly listing (what ``audit_async_lds_reads`` follows)."""
+    n, in_asm = 0, False
+    for line in asm_text.split("\n"):
+        s = line.strip()
+        if "ASMSTART" in s:
+            in_asm = True
+        elif "ASMEND" in s:
+            in_asm = False
+        elif in_asm and s.startswith("ds_read"):
+            n += 1
+    return n
+
+
+def audit_listings(base: str, listings) -> list:
+    """The audit of one source file, failing closed: ``listings`` are the texts of the gfx950 assembly files the
+    compile left behind.  None at all, or none of the expected inline-asm reads in a source that uses them, is
+    reported like a violation (the scan would otherwise pass by not seeing anything)."""
+    if not listings:
+        return [f"{base}: the compile left no gfx950 assembly listing to audit"]
+    found, reads = [], 0
+    for text in listings:
+        found += audit_async_lds_reads(text)
+        reads += count_async_lds_reads(text)
+    if base in ASYNC_LDS_SOURCES and reads == 0:
+        found.append(f"{base}: no inline-asm LDS read found in the assembly of a source that issues them "
+                     "(markers or spellings the scan relies on have changed)")
+    return found
+
+
 def _compile(src: str, obj_dir: str, extra) -> str:
     base = os.path.basename(src)[:-4]
     obj = os.path.join(obj_dir, base + ".o")
@@ -100,12 +135,13 @@ def _compile(src: str, obj_dir: str, extra) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
-    found = []
+    listings = []
     for tmp in glob.glob(os.path.join(obj_dir, base + "-*")) + glob.glob(os.path.join(obj_dir, base + ".hip-*")):
         if tmp.endswith("gfx950.s"):
             with open(tmp) as f:
-                found = audit_async_lds_reads(f.read())
+                listings.append(f.read())
         os.remove(tmp)   # intermediate files of the compile
+    found = audit_listings(base, listings)
     if found:
         raise RuntimeError(f"{src}: results of asynchronous LDS reads are used before their wait:\n" + "\n".join(found))
     return obj

@@ -95,3 +95,17 @@ def test_scan_restarts_behind_an_unconditional_branch_only():
     assert audit_async_lds_reads(LOOP_EXIT_BEHIND_BODY) == []
     found = audit_async_lds_reads(FALLS_THROUGH_A_CONDITIONAL_BRANCH)
     assert len(found) == 1 and "v_mov_b32_e32 v5, v30" in found[0]
+
+
+def test_audit_fails_closed():
+    """No assembly listing at all, or none of the inline-asm reads in a source that issues them, is a failure of
+    the audit, not a pass."""
+    from fourierattention_amd.build import ASYNC_LDS_SOURCES, audit_listings, count_async_lds_reads
+    assert count_async_lds_reads(GOOD) == 1 and count_async_lds_reads(PARTIAL) >= 2
+    assert audit_listings("fa_decode", [GOOD]) == []
+    assert any("no gfx950 assembly" in m for m in audit_listings("fa_decode", []))
+    plain = "_Zkernel_z:\n\tv_add_f32_e32 v1, v2, v3\n\ts_endpgm\n"
+    assert "fa_decode" in ASYNC_LDS_SOURCES and "fa_stream" not in ASYNC_LDS_SOURCES
+    assert any("no inline-asm LDS read" in m for m in audit_listings("fa_decode", [plain]))
+    assert audit_listings("fa_stream", [plain]) == []          # a source without such reads passes on a plain listing
+    assert audit_listings("fa_stream", [BAD_COPY]) != []       # but a violation is reported wherever it shows up
