@@ -71,10 +71,10 @@ MFMA_CASES = [
     (torch.bfloat16, 2, 32, 8, 128, 4, 64, 1024, 2200, 2, [64] * 8, [64] * 8),       # the benchmark's geometry, short
     (torch.bfloat16, 3, 16, 2, 128, 4, 200, 256, 900, 3, [64, 40], [64, 96]),        # 8:1 grouping, window of several tiles
     # the remaining instances of the mid-row kernel (256 frequencies with narrow pages, 512 with wide ones), an odd
-    # number of pages per split and a single page
+    # number of pages per split and splits of a single page (nine pages, the last one ragged)
     (torch.bfloat16, 2, 8, 2, 128, 4, 32, 512, 1000, 2, [64, 70], [80, 64]),
     (torch.bfloat16, 2, 16, 4, 128, 4, 32, 1024, 2300, 2, [30, 64, 0, 100], [128, 3, 64, 20]),
-    (torch.bfloat16, 1, 8, 2, 128, 4, 32, 256, 60, 2, [64, 64], [64, 64]),
+    (torch.bfloat16, 1, 8, 2, 128, 4, 32, 256, 300, 2, [64, 64], [64, 64]),
     # 1024 frequencies: the mid rows run as a score pass and a value pass
     (torch.bfloat16, 5, 16, 4, 128, 4, 32, 2048, 4500, 2, [64] * 4, [64] * 4),
     (torch.float16, 2, 8, 2, 128, 4, 32, 2048, 4200, 2, [0, 128], [120, 7]),
