@@ -378,6 +378,9 @@ def main():
                          "CPU baseline after it (for profiler runs)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decodes of configs 4 and 5 in the default run")
     ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
+    ap.add_argument("--even-splits", action="store_true",
+                    help="give every KV head the same number of splits of the mid rows (default: heads that store more dims "
+                         "get more; no difference with a uniform mask)")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
                     help="run the end-to-end decode of a random-init model instead (its own JSON line); --steps caps the "
                          "number of timed tokens per sequence")
@@ -424,6 +427,7 @@ def main():
             print(f"bench.py: parity check failed (max abs err {parity})", file=sys.stderr)
             sys.exit(1)
     cache, q, kn, vn = build_cache(w, dtype, device)
+    cache.balance_heads = not args.even_splits
     Hq, Hkv = w["Hq"], w["Hkv"]
     for _ in range(args.warmup):
         out = cache.decode_attention(q, 0, Hq, Hkv)

@@ -44,6 +44,7 @@ class DecodeArgs(ctypes.Structure):
         ("mid_layout", c_int32), ("mid_cap_pages", c_int32),
         ("k_pad_h_list", c_void_p), ("v_pad_h_list", c_void_p),
         ("mid_max_k_pad", c_int32), ("mid_max_v_pad", c_int32),
+        ("k_pad_h_host", c_void_p), ("v_pad_h_host", c_void_p),
         ("tables", c_void_p), ("force_generic", c_int32),
         ("avg_k_u", c_void_p), ("avg_k_d", c_void_p), ("scale_k", c_void_p),
         ("avg_v_u", c_void_p), ("avg_v_d", c_void_p), ("scale_v", c_void_p),

@@ -202,6 +202,7 @@ class DynamicCache(Cache):
                             for i in range(self._num_layers)]
         self._tables: Optional[torch.Tensor] = None   # constant operands of the MFMA decode kernels
         self.force_generic = False                     # testing: keep decode attention off the MFMA kernels
+        self.balance_heads = True                      # mid rows: more splits for heads that store more dims
         self._book = CacheBook(self._num_layers, self.numinittokens, self.maxlocallen, self.maxmidstates,
                                self.maxnewtokens, self.maxtokens)
         self._layers: List[_Layer] = [_Layer() for _ in range(self._num_layers)]
@@ -452,4 +453,4 @@ class DynamicCache(Cache):
         return ops.decode_attn_raw(q, segs, layer.k.coef, layer.v.coef, layer.k.mid, layer.v.mid, layer.k.stats32,
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
                                    sm_scale, tables=self._tables, force_generic=self.force_generic, timings=timings,
-                                   out_dtype=out_dtype, out=out, no_alloc=no_alloc)
+                                   out_dtype=out_dtype, out=out, no_alloc=no_alloc, balance_heads=self.balance_heads)

@@ -491,10 +491,12 @@ __device__ __forceinline__ float weighted_sum(const float* __restrict__ ptr, int
 
 constexpr int kMergeChunksMax = 8;  // blocks per (b, KV head): each applies the V coefficients of its share of the dims
 
+// n_mid_stride: splits the partial buffers of the mid rows have room for per query head; the head's own number of
+// splits comes from the table (heads that store more dims are cut into more splits)
 __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const float* __restrict__ il_m, const float* __restrict__ il_d, const float* __restrict__ il_o, int n_il_split,
     const float* __restrict__ md_m, const float* __restrict__ md_d, const float* __restrict__ md_g,
-    const float* __restrict__ md_on, int n_mid_split, const float* __restrict__ v_mc,
+    const float* __restrict__ md_on, int n_mid_stride, const fa_mfma::SplitTable st, const float* __restrict__ v_mc,
     const float* __restrict__ avg_u, const float* __restrict__ avg_d, const float* __restrict__ scale,
     const int32_t* __restrict__ vc_list, const int32_t* __restrict__ vc_h, const int32_t* __restrict__ vn_list,
     const int32_t* __restrict__ vn_h, float* __restrict__ out, void* __restrict__ out_cast, int cast_dtype, int Hq, int Hkv,
@@ -514,6 +516,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   // (query head, split)
   extern __shared__ float smem[];
   const int G = Hq / Hkv;
+  const int n_mid_split = (int)blockIdx.x < fa_mfma::kSplitHeads ? min(st.n[blockIdx.x], n_mid_stride) : n_mid_stride;
   const int n_all = n_il_split + n_mid_split;
   float* s_g = smem;                     // [G][2N]
   float* s_w = s_g + G * 2 * N;          // [G][n_all]
@@ -543,8 +546,8 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     const int g = tid / n_all, s_ = tid - g * n_all;
     const int64_t r = r0 + g;
     const bool il = s_ < n_il_split;
-    m_raw = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
-    d_raw = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
+    m_raw = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_stride + (s_ - n_il_split)];
+    d_raw = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_stride + (s_ - n_il_split)];
   }
   // g partials: two neighbouring threads share four consecutive coefficient rows of one head, one takes the even
   // splits, the other the odd ones (16-byte loads: a quarter of the load instructions of a row-per-thread map)
@@ -561,11 +564,11 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
       g = (item >> 2) % G;
       n4 = (item / (4 * G)) * 4 + (item & 3);
       const int grp = b / g_nbpg, lc = (b - grp * g_nbpg) * G + g;
-      return md_g + (int64_t)(grp * Hkv + h) * n_mid_split * g_split_stride + (int64_t)(n4 >> 2) * 256 + (lc * 4 + (n4 & 3)) * 4;
+      return md_g + (int64_t)(grp * Hkv + h) * n_mid_stride * g_split_stride + (int64_t)(n4 >> 2) * 256 + (lc * 4 + (n4 & 3)) * 4;
     }
     g = item / (2 * N / E4);
     n4 = item - g * (2 * N / E4);
-    return md_g + (r0 + g) * n_mid_split * 2 * N + E4 * n4;
+    return md_g + (r0 + g) * n_mid_stride * 2 * N + E4 * n4;
   };
   float4 g_pre[kGPre];
   if (has_coef && g_item < g_items) {
@@ -585,7 +588,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
   float n_pre[kMergePre];                           // stored-dim outputs of the mid rows
   if (n_mid_split > 0 && tid < G * nn) {
     const int g = tid / nn, jj = n_lo + (tid - g * nn);
-    prefetch_strided(n_pre, md_on + (r0 + g) * n_mid_split * D + jj, D, n_mid_split);
+    prefetch_strided(n_pre, md_on + (r0 + g) * n_mid_stride * D + jj, D, n_mid_split);
   }
   float il_pre[kMergeIl];                           // sink/window outputs of element tid
   if (n_il_split > 0 && tid < G * D) {
@@ -602,8 +605,8 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
       const int g = idx / n_all, s_ = idx - g * n_all;
       const int64_t r = r0 + g;
       const bool il = s_ < n_il_split;
-      s_w[idx] = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_split + (s_ - n_il_split)];
-      s_d[idx] = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_split + (s_ - n_il_split)];
+      s_w[idx] = il ? il_m[r * n_il_split + s_] : md_m[r * n_mid_stride + (s_ - n_il_split)];
+      s_d[idx] = il ? il_d[r * n_il_split + s_] : md_d[r * n_mid_stride + (s_ - n_il_split)];
     }
   }
   for (int idx = tid; idx < G * D; idx += 1024) s_o[idx] = 0.f;
@@ -732,13 +735,13 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
     }
     if (tid < G * nn) {
       const int g = tid / nn, jj = n_lo + (tid - g * nn);
-      s_o[g * D + (vn_list[vn0 + jj] - h * D)] = weighted_sum_pre(n_pre, md_on + (r0 + g) * n_mid_split * D + jj, D,
+      s_o[g * D + (vn_list[vn0 + jj] - h * D)] = weighted_sum_pre(n_pre, md_on + (r0 + g) * n_mid_stride * D + jj, D,
                                                                   s_w + g * n_all + n_il_split, n_mid_split);
     }
     for (int idx = tid + 1024; idx < G * nn; idx += 1024) {
       const int g = idx / nn, jj = n_lo + (idx - g * nn);
       s_o[g * D + (vn_list[vn0 + jj] - h * D)] =
-          weighted_sum(md_on + (r0 + g) * n_mid_split * D + jj, D, s_w + g * n_all + n_il_split, n_mid_split);
+          weighted_sum(md_on + (r0 + g) * n_mid_stride * D + jj, D, s_w + g * n_all + n_il_split, n_mid_split);
     }
   }
   __syncthreads();
@@ -956,7 +959,11 @@ enum class Path { Generic, Mfma };
 
 struct Plan {
   Path path;
+  // n_mid_split: splits the partial buffers of the mid rows have room for per head (with the matrix-core kernels the
+  // heads may differ, see st; tiles_per_split then belongs to the generic kernels only)
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
+  int n_wg;   // matrix-core mid rows: workgroups per batch group
+  fa_mfma::SplitTable st;
   int n_merge_chunks;
   size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_scores, total;
 };
@@ -967,7 +974,54 @@ bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
          (N == 128 || N == 256 || N == 512 || N == 1024);
 }
 
-Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma, bool il_fast) {
+// Splits per head of the matrix-core mid rows.  Without the per-head padded dim counts (kpad / vpad, host copies of the
+// cumulative lists) every head gets the same number.  With them the same total is shared out so that the slowest
+// workgroup is as fast as possible: a page of a head costs a fixed part for the coefficient-domain arithmetic (54) plus
+// 1 per 1 KiB fragment of stored K dims and 3 per fragment of stored V dims (the value waves are the slower role;
+// weights fitted on the kernel's time with the per-head counts of three layers of the reference's mask for
+// Llama-3.1-8B), a workgroup takes ceil(pages / splits) pages, and single splits move from the head that finishes first to
+// the head that finishes last while that shortens the longest time.  No head gets more than `room` splits (half as
+// many again as the even share: the partial buffers are sized for that).  Returns the largest count.
+int share_out_splits(fa_mfma::SplitTable& st, int Hkv, int tiles, int ns, int room, const int32_t* kpad, const int32_t* vpad) {
+  using fa_mfma::kSplitHeads;
+  for (int h = 0; h < kSplitHeads; ++h) st.n[h] = ns;
+  if (kpad && vpad && ns > 1 && Hkv > 1 && Hkv <= kSplitHeads) {
+    int cost[kSplitHeads];
+    for (int h = 0; h < Hkv; ++h) cost[h] = 54 + 2 * ((kpad[h + 1] - kpad[h]) / 32) + 3 * ((vpad[h + 1] - vpad[h]) / 16);
+    auto time_of = [&](int h, int n) { return (int64_t)cost[h] * fa_cdiv(tiles, n); };
+    for (int moves = 0; moves < ns * Hkv; ++moves) {
+      int slow = 0;
+      for (int h = 1; h < Hkv; ++h)
+        if (time_of(h, st.n[h]) > time_of(slow, st.n[slow])) slow = h;
+      if (st.n[slow] >= room) break;
+      const int64_t worst = time_of(slow, st.n[slow]);
+      int donor = -1;   // the head that is fastest even with one split fewer
+      for (int h = 0; h < Hkv; ++h)
+        if (h != slow && st.n[h] > 1 && (donor < 0 || time_of(h, st.n[h] - 1) < time_of(donor, st.n[donor] - 1))) donor = h;
+      if (donor < 0 || time_of(donor, st.n[donor] - 1) >= worst) break;   // nothing gained: the donor would be as slow
+      // the step must shorten the longest time or leave it to another head that is no slower than before
+      --st.n[donor];
+      ++st.n[slow];
+    }
+  }
+  int largest = 0;
+  st.first[0] = 0;
+  for (int h = 0; h < kSplitHeads; ++h) {
+    if (h < Hkv) {
+      // (as many splits as pages of the resulting length really fill)
+      const int per = fa_cdiv(tiles, st.n[h] > 0 ? st.n[h] : 1);
+      st.n[h] = st.n[h] > 0 ? fa_cdiv(tiles, per) : 0;
+      if (st.n[h] > largest) largest = st.n[h];
+    }
+    st.first[h + 1] = st.first[h] + (h < Hkv ? st.n[h] : 0);
+  }
+  return largest;
+}
+
+// kpad / vpad: see share_out_splits.  full_room: size the partial buffers for the most uneven share a call with those
+// lists could ask for (the workspace query, which does not see them).
+Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma, bool il_fast,
+               const int32_t* kpad = nullptr, const int32_t* vpad = nullptr, bool full_room = false) {
   Plan p{};
   p.path = mfma ? Path::Mfma : Path::Generic;
   p.n_il_split = fa_cdiv(n_il, il_fast ? kIlFastTile : kTile);
@@ -982,7 +1036,12 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     if (want < 1) want = 1;
     int ns = tiles < want ? tiles : want;
     p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
-    p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+    const int even = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+    int room = fa_cdiv(3 * even, 2);
+    if (room > tiles) room = tiles;
+    const int largest = share_out_splits(p.st, Hkv, tiles, even, room, kpad, vpad);
+    p.n_mid_split = full_room && Hkv > 1 && Hkv <= fa_mfma::kSplitHeads ? room : largest;
+    p.n_wg = p.st.first[Hkv <= fa_mfma::kSplitHeads ? Hkv : fa_mfma::kSplitHeads];
   } else {
     const int tiles = fa_cdiv(L_m, kTile);
     int want = fa_cdiv(1024, (int64_t)B * Hkv);
@@ -991,6 +1050,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     if (ns > 64) ns = 64;
     p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
     p.n_mid_split = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
+    for (int h = 0; h < fa_mfma::kSplitHeads; ++h) p.st.n[h] = p.n_mid_split;
   }
   const size_t rows = (size_t)B * Hq;
   size_t o = 0;
@@ -1044,7 +1104,7 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
 // eight frequency slices: a score pass, then a value pass over the same pages
 template <typename E>
 void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
-  dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
+  dim3 grid(p.n_wg, p.n_groups);
   if (wide) {
     fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
     fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 2><<<grid, 512, 0, st>>>(mp);
@@ -1056,7 +1116,7 @@ void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bo
 
 template <typename E, int KS>
 void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
-  dim3 grid(p.n_mid_split, mp.Hkv, p.n_groups);
+  dim3 grid(p.n_wg, p.n_groups);
   if (wide)
     fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2><<<grid, 512, 0, st>>>(mp);
   else
@@ -1120,7 +1180,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.scores = (float*)(ws + p.off_scores);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
-        mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.tiles_per_split = p.tiles_per_split;
+        mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.st = p.st;
         mp.sm_log2e = sm_log2e;
         if (ev) hipEventRecord(ev[1], st);
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
@@ -1182,7 +1242,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
       FA_REQUIRE(e == hipSuccess, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS refused", lds);
     }
     decode_merge_kernel<<<dim3(a.Hkv, a.B, p.n_merge_chunks), 1024, lds, st>>>(
-        ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
+        ilm, ild, ilo, p.n_il_split, mm, md, mg, mon, p.n_mid_split, p.st, a.v_mc, a.avg_v_u, a.avg_v_d, a.scale_v,
         a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list, a.out, a.out_cast, a.dtype, a.Hq, a.Hkv, a.D, a.N, a.Cv,
         p.path == Path::Mfma ? p.nbpg : 0);
   }
@@ -1192,12 +1252,13 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
 
 bool use_mfma(const fa_decode_args& a) {
   return a.L_m > 0 && !a.force_generic && mfma_shape_ok(a.Hq, a.Hkv, a.D, a.N, a.dtype, a.mid_layout) &&
-         a.Hq / a.Hkv <= kGMax && a.mid_max_k_pad <= 128 && a.mid_max_v_pad <= 128;
+         a.Hq / a.Hkv <= kGMax && a.mid_max_k_pad <= 128 && a.mid_max_v_pad <= 128 && a.Hkv <= fa_mfma::kSplitHeads;
 }
 
 }  // namespace
 
-extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m) {
+// full_room: room for the uneven shares that a call with the per-head lists on the host side may ask for
+static size_t workspace_bytes_for(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m, bool full_room) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || N < 0 || il_rows_total < 0 || L_m < 0 || Hq % Hkv) return 0;
   const int n = N > 0 ? N : 1;
   // large enough for either path
@@ -1206,11 +1267,15 @@ extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, 
     size_t b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, false, il_fast != 0).total;
     if (b > a) a = b;
     if (mfma_shape_ok(Hq, Hkv, D, n, FA_BF16, FA_MID_PAGED)) {
-      b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, true, il_fast != 0).total;
+      b = make_plan(B, Hq, Hkv, D, n, il_rows_total, L_m, true, il_fast != 0, nullptr, nullptr, full_room).total;
       if (b > a) a = b;
     }
   }
   return a;
+}
+
+extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m) {
+  return workspace_bytes_for(B, Hq, Hkv, D, N, il_rows_total, L_m, true);
 }
 
 extern "C" size_t fa_decode_tables_bytes(int N) { return (N > 0 && N % 64 == 0) ? fa_mfma::tables_bytes(N) : 0; }
@@ -1267,7 +1332,7 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
   const bool mfma = use_mfma(*a);
   const bool il_fast = il_fast_ok(*a);
   const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma,
-                           il_fast);
+                           il_fast, a->k_pad_h_host, a->v_pad_h_host);
   FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
              a->workspace_bytes, p.total);
   FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");
@@ -1317,7 +1382,8 @@ int scratch_on_current_device(void** out) {
 
 extern "C" int fa_decode_attn_noalloc(const fa_decode_args* a, fa_stream_t stream) {
   FA_REQUIRE(a, FA_ERR_NULL_POINTER, "fa_decode_attn_noalloc: null argument block");
-  const size_t need = fa_decode_attn_workspace_bytes(a->B, a->Hq, a->Hkv, a->D, a->N, a->il_rows[0] + a->il_rows[1], a->L_m);
+  // (every head the same number of splits here: the built-in buffer is not sized for uneven shares)
+  const size_t need = workspace_bytes_for(a->B, a->Hq, a->Hkv, a->D, a->N, a->il_rows[0] + a->il_rows[1], a->L_m, false);
   FA_REQUIRE(need > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn_noalloc: bad B/Hq/Hkv/D/N/row counts");
   FA_REQUIRE(need <= (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES, FA_ERR_WORKSPACE,
              "fa_decode_attn_noalloc: this shape needs %zu bytes of scratch, the built-in buffer holds %zu; use "
@@ -1326,6 +1392,7 @@ extern "C" int fa_decode_attn_noalloc(const fa_decode_args* a, fa_stream_t strea
   int rc = scratch_on_current_device(&ptr);
   if (rc != FA_OK) return rc;
   fa_decode_args b = *a;
+  b.k_pad_h_host = b.v_pad_h_host = nullptr;
   b.workspace = ptr;
   b.workspace_bytes = (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES;
   return decode_attn_impl(&b, stream, nullptr);

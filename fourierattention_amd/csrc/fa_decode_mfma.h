@@ -205,6 +205,14 @@ __device__ __forceinline__ void wait_pages_in_flight(int n) {
   }
 }
 
+// The mid rows of KV head h are cut into n[h] splits (heads that store more dims take longer per page and get more);
+// the workgroups of one batch group are numbered head by head, first[h] being the first one of head h.
+constexpr int kSplitHeads = 64;
+struct SplitTable {
+  int n[kSplitHeads];
+  int first[kSplitHeads + 1];
+};
+
 template <typename E>
 struct MidParams {
   const E* q;
@@ -228,8 +236,10 @@ struct MidParams {
   float* pg;
   float* pon;
   float* scores;   // two-pass mode: [groups][Hkv][pages][16 columns][32 tokens] fp32
-  int B, Hq, Hkv, D, G, nbpg, N, L_m, T, n_split, tiles_per_split;
+  int B, Hq, Hkv, D, G, nbpg, N, L_m, T;
+  int n_split;   // splits the partial buffers have room for per head (the largest n[h])
   float sm_log2e;
+  SplitTable st;
 };
 
 // The workgroup is a two-stage pipeline over the pages of its split, one barrier per page:
@@ -271,7 +281,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
   const bool score_wave = MODE == 0 ? w < kFreqWaves : MODE == 1;
   const int sl = MODE == 0 ? (w & 3) : w;  // frequency slice; below 4 also the batch element of the group
-  const int split = blockIdx.x, h = blockIdx.y, grp = blockIdx.z;
+  // workgroup -> (KV head, split of that head)
+  const int grp = blockIdx.y;
+  int h = 0;
+  while (h + 1 < p.Hkv && (int)blockIdx.x >= p.st.first[h + 1]) ++h;
+  const int split = blockIdx.x - p.st.first[h];
   const int G = p.G, N = p.N;
   const int b0 = grp * p.nbpg;
   const int nb = min(p.nbpg, p.B - b0);
@@ -285,8 +299,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int stw = has_mn ? w & 3 : 0;   // page stage of this wave
 
   const int n_tiles = (p.L_m + 31) >> 5;
-  const int t_beg = split * p.tiles_per_split;
-  const int t_end = min(n_tiles, t_beg + p.tiles_per_split);
+  const int tiles_per_split = (n_tiles + p.st.n[h] - 1) / p.st.n[h];
+  const int t_beg = split * tiles_per_split;
+  const int t_end = min(n_tiles, t_beg + tiles_per_split);
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
 
   // Rotation constants of slice sl into LDS: one entry (unit, lane group) per lane, requested early and stored once

@@ -6,6 +6,8 @@ from __future__ import annotations
 
 from typing import List
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -25,6 +27,7 @@ class MidStore:
             n = n_h_host[h + 1] - n_h_host[h]
             pad.append(pad[-1] + (n + unit - 1) // unit * unit)
         self.pad_h_host = pad
+        self.pad_h_c = (ctypes.c_int32 * len(pad))(*pad)   # the same for the C side (kept alive with the store)
         self.max_pad = max([pad[h + 1] - pad[h] for h in range(num_kv_heads)] + [0])
         self.pad_h32 = torch.tensor(pad, dtype=torch.int32, device=device)
         self.dtype, self.device = dtype, torch.device(device)

@@ -347,7 +347,7 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
                     T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None,
-                    no_alloc=False):
+                    no_alloc=False, balance_heads=True):
     """Thin call into ``fa_decode_attn``.  The result is float32 like the reference's (TRI:779) unless ``out_dtype``
     names the dtype of ``q``: then the merge launch rounds it to that type itself (the caller's ``.to(dtype)``).
 
@@ -356,7 +356,9 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     ``stats_*``: ``(avg_u, avg_d, scale)`` fp32 ``(B, C)``.  ``lists``: the eight int32 tensors
     ``kc, kc_h, kn, kn_h, vc, vc_h, vn, vn_h`` (``*_h`` with the leading 0).
     ``no_alloc``: call ``fa_decode_attn_noalloc`` (partial results in the library's own fixed buffer, no workspace
-    tensor; pass ``out`` as well and nothing is allocated on the device at all)."""
+    tensor; pass ``out`` as well and nothing is allocated on the device at all).
+    ``balance_heads``: hand the per-head padded dim counts of a paged store over on the host side too, so that heads
+    that store more dims get more splits (``False``: every head the same number, for comparison)."""
     from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
@@ -388,6 +390,9 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
             a.k_mn_batch_stride, a.v_mn_batch_stride = k_mn.batch_stride, v_mn.batch_stride
             a.k_pad_h_list, a.v_pad_h_list = k_mn.pad_h32.data_ptr(), v_mn.pad_h32.data_ptr()
             a.mid_max_k_pad, a.mid_max_v_pad = k_mn.max_pad, v_mn.max_pad
+            if balance_heads:
+                a.k_pad_h_host = ctypes.cast(k_mn.pad_h_c, ctypes.c_void_p)
+                a.v_pad_h_host = ctypes.cast(v_mn.pad_h_c, ctypes.c_void_p)
         else:
             for t in (k_mn, v_mn):
                 assert t.stride(2) == 1 and t.dtype == q.dtype

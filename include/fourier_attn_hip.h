@@ -177,6 +177,11 @@ typedef struct fa_decode_args {
   const int32_t* v_pad_h_list;
   int32_t mid_max_k_pad;   /* largest per-head padded dim count of K / V (host copies of */
   int32_t mid_max_v_pad;   /* max_h(pad_h[h+1] - pad_h[h]); select the kernel instance)   */
+  /* optional HOST copies of k_pad_h_list / v_pad_h_list (Hkv + 1 entries each), or NULL: with them the mid rows
+   * of a head that stores more dims are cut into more splits than those of a head that stores few (the
+   * reference's masks differ head by head), so that all workgroups finish together */
+  const int32_t* k_pad_h_host;
+  const int32_t* v_pad_h_host;
   /* optional constant operand tables built by fa_decode_tables_build for this (N, T);
    * NULL lets the call build them in its workspace */
   const void* tables;
@@ -281,8 +286,10 @@ int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
  * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  `args->workspace` and
  * `args->workspace_bytes` are ignored; the partial results live in a buffer of FA_DECODE_NOALLOC_SCRATCH_BYTES
  * that is part of the library image on every GPU it runs on (held until the process ends).  Nothing is allocated
- * or freed, by this call or by anything it calls.  Shapes for which fa_decode_attn_workspace_bytes(...) exceeds
- * that size are refused with FA_ERR_WORKSPACE.  Every call on one GPU shares that GPU's buffer: calls that may
+ * or freed, by this call or by anything it calls.  k_pad_h_host / v_pad_h_host are ignored as well: every KV head
+ * gets the same number of splits, and shapes whose partial results then exceed that size (at most what
+ * fa_decode_attn_workspace_bytes(...) reports, which leaves room for uneven shares) are refused with
+ * FA_ERR_WORKSPACE.  Every call on one GPU shares that GPU's buffer: calls that may
  * overlap on one GPU (two streams, two threads) race and must be serialised by the caller; consecutive calls on
  * one stream are fine (every kernel writes what it later reads, nothing needs clearing).  The first call on a
  * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture. */

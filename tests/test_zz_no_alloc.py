@@ -1,7 +1,8 @@
 """``fa_decode_attn_noalloc``: the decode-attention entry point that keeps its partial results in a buffer built into
 the library instead of a caller's workspace.  Called through the C ABI on the same operands as ``fa_decode_attn``,
 twice in a row with the second call on a smaller input (the buffer keeps the first call's contents), it must give
-the same result bit for bit: both run the same kernels with the same split of the work."""
+the same result bit for bit: both run the same kernels with the same split of the work (the cache's default, more
+splits for heads that store more dims, is switched off for the comparison)."""
 import ctypes
 
 import numpy as np
@@ -34,7 +35,12 @@ def test_oversized_shape_is_refused_before_anything_is_touched():
     assert need > _lib.DECODE_NOALLOC_SCRATCH_BYTES
     assert lib.fa_decode_attn_noalloc(ctypes.byref(a), None) == -4          # FA_ERR_WORKSPACE
     msg = lib.fa_last_error_string().decode()
-    assert str(need) in msg and str(_lib.DECODE_NOALLOC_SCRATCH_BYTES) in msg
+    # the size it names is that of a call with the same number of splits for every head (what this entry point
+    # runs): above the buffer, and no more than the general workspace query, which leaves room for uneven shares
+    import re
+    sizes = [int(x) for x in re.findall(r"\d{6,}", msg)]
+    assert _lib.DECODE_NOALLOC_SCRATCH_BYTES in sizes
+    assert any(_lib.DECODE_NOALLOC_SCRATCH_BYTES < x <= need for x in sizes)
     assert lib.fa_decode_attn_noalloc(None, None) == -1                     # FA_ERR_NULL_POINTER
 
 
@@ -69,7 +75,12 @@ def test_two_calls_in_a_row_match_the_entry_point_with_a_workspace(dtype, tol):
     big = _cache_case(dtype, 5, Hq, Hkv, D, 64, 512, 3000, [64, 40], [64, 96], seed=1)
     small = _cache_case(dtype, 2, Hq, Hkv, D, 32, 256, 700, [64, 64], [30, 64], seed=2)
     for gpu, q, want in (big, small):
+        # the entry point under test gives every head the same number of splits; so does the reference call here
+        # (with its default, shares by stored dims, the sums run in another order: checked to rounding below)
+        shared = gpu.decode_attention(q, 0, Hq, Hkv)
+        gpu.balance_heads = False
         ref = gpu.decode_attention(q, 0, Hq, Hkv)                               # fa_decode_attn, caller's workspace
+        assert (shared - ref).abs().max().item() <= 1e-3 * max(1.0, ref.abs().max().item())
         out = torch.full_like(ref, float("nan"))
         got = gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True)       # fa_decode_attn_noalloc
         assert got is out and torch.equal(got, ref)
