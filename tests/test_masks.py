@@ -66,6 +66,12 @@ def test_synthetic_masks_are_valid_and_seeded():
         assert len(entry["kc_list"]) == 512 and len(entry["vn_list"]) == 512
     r = pm.synthetic_masks(1, 4, 16, 0, 16)["Layer_0"]
     assert r["kc_list"] == [] and r["kn_h_list"] == [16, 32, 48, 64] and r["vn_list"] == []
+    # one count per head (masks whose heads differ, like the reference's own)
+    e = pm.synthetic_masks(1, 4, 16, [3, 0, 16, 7], [16, 1, 2, 0], seed=2)["Layer_0"]
+    pm.validate_layer(e, 4, 16)
+    assert e["kc_h_list"] == [3, 3, 19, 26] and e["vc_h_list"] == [16, 17, 19, 19]
+    with pytest.raises(ValueError):
+        pm.synthetic_masks(1, 4, 16, [3, 0, 16])
 
 
 def test_validate_rejects_inconsistent():
