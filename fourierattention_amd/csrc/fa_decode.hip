@@ -1278,6 +1278,20 @@ extern "C" size_t fa_decode_attn_workspace_bytes(int B, int Hq, int Hkv, int D, 
   return workspace_bytes_for(B, Hq, Hkv, D, N, il_rows_total, L_m, true);
 }
 
+extern "C" int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m,
+                                    const int32_t* k_pad_h_host, const int32_t* v_pad_h_host, int32_t* splits_out,
+                                    int32_t* room_out) {
+  FA_REQUIRE(splits_out, FA_ERR_NULL_POINTER, "fa_decode_split_plan: null pointer");
+  FA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && D > 0 && N > 0 && il_rows_total >= 0 && L_m > 0 && Hq % Hkv == 0, FA_ERR_BAD_SHAPE,
+             "fa_decode_split_plan: bad shape");
+  FA_REQUIRE(mfma_shape_ok(Hq, Hkv, D, N, FA_BF16, FA_MID_PAGED) && Hq / Hkv <= kGMax && Hkv <= fa_mfma::kSplitHeads,
+             FA_ERR_UNSUPPORTED, "fa_decode_split_plan: this shape does not take the matrix-core kernels");
+  const Plan p = make_plan(B, Hq, Hkv, D, N, il_rows_total, L_m, true, true, k_pad_h_host, v_pad_h_host);
+  for (int h = 0; h < Hkv; ++h) splits_out[h] = p.st.n[h];
+  if (room_out) *room_out = make_plan(B, Hq, Hkv, D, N, il_rows_total, L_m, true, true, nullptr, nullptr, true).n_mid_split;
+  return FA_OK;
+}
+
 extern "C" size_t fa_decode_tables_bytes(int N) { return (N > 0 && N % 64 == 0) ? fa_mfma::tables_bytes(N) : 0; }
 
 extern "C" int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_stream_t stream) {

@@ -293,6 +293,15 @@ int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
  * overlap on one GPU (two streams, two threads) race and must be serialised by the caller; consecutive calls on
  * one stream are fine (every kernel writes what it later reads, nothing needs clearing).  The first call on a
  * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture. */
+/* How fa_decode_attn would cut the mid rows of each KV head into splits on the matrix-core kernels (host-side
+ * arithmetic only, no GPU work; no counterpart in the reference): splits_out[h] for h < Hkv, given the host copies of
+ * the per-head padded dim counts (or NULL for both: every head the same), and in *room_out (optional) the number of
+ * splits per head that fa_decode_attn_workspace_bytes leaves room for.  FA_ERR_UNSUPPORTED for shapes that take the
+ * generic kernels. */
+int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m,
+                         const int32_t* k_pad_h_host, const int32_t* v_pad_h_host, int32_t* splits_out,
+                         int32_t* room_out);
+
 #define FA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
 int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
 

@@ -253,3 +253,41 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_stream_update(ctypes.byref(sa), None) == -2                  # empty shape
     assert lib.fa_stats_workspace_bytes(2, 10, 1000) == 3 * 2 * 4 * 10 * 4
     assert lib.fa_decode_attn_workspace_bytes(8, 32, 8, 128, 512, 1028, 31740) > 0
+
+
+def test_split_plan_of_the_mid_rows():
+    """``fa_decode_split_plan`` (host-side arithmetic of the launch, runs without a GPU): how the mid rows of each KV
+    head are cut into splits.  Same count for every head without the per-head lists or with a uniform mask; with a
+    ragged mask the total stays the same, nobody gets more than the workspace query leaves room for, nobody gets
+    none, and a head that stores more dims never gets fewer splits (beyond one of rounding) than one that stores fewer
+    of both K and V."""
+    import ctypes
+    from fourierattention_amd import _lib
+    lib = _lib.load()
+
+    def plan(L_m, kpads, vpads, B=8, Hq=32, Hkv=8, N=512):
+        out, room = (ctypes.c_int32 * Hkv)(), ctypes.c_int32()
+        cum = lambda p: (ctypes.c_int32 * (Hkv + 1))(*([0] + list(np.cumsum(p)))) if p is not None else None
+        k, v = cum(kpads), cum(vpads)
+        rc = lib.fa_decode_split_plan(B, Hq, Hkv, 128, N, 1028, L_m, k, v, out, ctypes.byref(room))
+        assert rc == 0, lib.fa_last_error_string()
+        return list(out), room.value
+
+    even, room = plan(31740, None, None)
+    assert len(set(even)) == 1 and even[0] >= 1 and room == -(-3 * even[0] // 2)
+    assert plan(31740, [64] * 8, [64] * 8)[0] == even                    # a uniform mask changes nothing
+    # padded per-head counts of layers 15 and 31 of the reference's Llama-3.1-8B mask
+    for kp, vp in (([64, 32, 32, 32, 32, 64, 32, 64], [16, 0, 32, 32, 128, 16, 0, 48]),
+                   ([96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16])):
+        got, room2 = plan(31740, kp, vp)
+        assert room2 == room and sum(got) <= sum(even) and sum(got) >= sum(even) - len(got)
+        assert min(got) >= 1 and max(got) <= room
+        for a in range(8):
+            for b in range(8):
+                if kp[a] >= kp[b] and vp[a] >= vp[b]:
+                    assert got[a] + 1 >= got[b], (a, b, got)             # (single splits move: equal heads may differ by one)
+        assert got[vp.index(max(vp))] > even[0]                          # the head with the widest V pages gets more
+    # fewer pages than workgroups: one page per split for everybody
+    short, _ = plan(200, [96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16])
+    assert short == [7] * 8
+    assert lib.fa_decode_split_plan(8, 32, 8, 128, 100, 0, 5000, None, None, (ctypes.c_int32 * 8)(), None) == -5   # N not covered
