@@ -104,7 +104,52 @@ __global__ void rope_qk_kernel(const E* q_in, int64_t q_stride, E* q_out, E* k, 
   x[i + half] = Rounder<E>::put(rnd<E>(x2 * c2) + rnd<E>(x1 * s2));
 }
 
+// The same on 16 bytes per thread (16-bit storage, D a multiple of 16, rows and pointers 16-byte aligned): one block
+// per row walks over every (head, pair of 8-element pieces i / i + D/2); long prompts are bound by memory here.
+template <typename E>
+__global__ __launch_bounds__(256) void rope_qk_vec_kernel(const E* q_in, int64_t q_stride, E* q_out, E* k, int64_t k_stride,
+                                                          const E* __restrict__ cs, const E* __restrict__ sn, int Hq, int Hkv,
+                                                          int D) {
+  struct alignas(16) Pack { E e[8]; };
+  const int64_t row = blockIdx.x;
+  const int half = D >> 1, per_head = half >> 3;
+  for (int item = threadIdx.x; item < (Hq + Hkv) * per_head; item += 256) {
+    const int head = item / per_head, i = (item - head * per_head) * 8;
+    const E* src = head < Hq ? q_in + row * q_stride + head * D : k + row * k_stride + (head - Hq) * D;
+    E* x = head < Hq ? q_out + (row * Hq + head) * D : k + row * k_stride + (head - Hq) * D;
+    const Pack a1 = *(const Pack*)(src + i), a2 = *(const Pack*)(src + i + half);
+    const Pack c1 = *(const Pack*)(cs + row * D + i), c2 = *(const Pack*)(cs + row * D + i + half);
+    const Pack s1 = *(const Pack*)(sn + row * D + i), s2 = *(const Pack*)(sn + row * D + i + half);
+    Pack o1, o2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float x1 = fa_to_float(a1.e[e]), x2 = fa_to_float(a2.e[e]);
+      o1.e[e] = Rounder<E>::put(rnd<E>(x1 * fa_to_float(c1.e[e])) + rnd<E>(-x2 * fa_to_float(s1.e[e])));
+      o2.e[e] = Rounder<E>::put(rnd<E>(x2 * fa_to_float(c2.e[e])) + rnd<E>(x1 * fa_to_float(s2.e[e])));
+    }
+    *(Pack*)(x + i) = o1;
+    *(Pack*)(x + i + half) = o2;
+  }
+}
+
 // grid (column blocks, rows): gate and up rows may be slices of wider rows (a fused projection output)
+template <typename E>
+__global__ __launch_bounds__(256) void silu_mul_vec_kernel(const E* __restrict__ gate, const E* __restrict__ up,
+                                                            E* __restrict__ out, int cols, int64_t in_stride) {
+  struct alignas(16) Pack { E e[8]; };   // (16-bit storage: 16 bytes per thread)
+  const int i = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i >= cols) return;
+  const int64_t row = blockIdx.y;
+  const Pack g8 = *(const Pack*)(gate + row * in_stride + i), u8 = *(const Pack*)(up + row * in_stride + i);
+  Pack o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float g = fa_to_float(g8.e[e]);
+    o.e[e] = Rounder<E>::put(rnd<E>(g / (1.0f + expf(-g))) * fa_to_float(u8.e[e]));
+  }
+  *(Pack*)(out + row * cols + i) = o;
+}
+
 template <typename E>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const E* __restrict__ gate, const E* __restrict__ up,
                                                         E* __restrict__ out, int cols, int64_t in_stride) {
@@ -157,6 +202,14 @@ extern "C" int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, vo
   hipStream_t st = fa_hip_stream(stream);
   int rc = by_dtype(dtype, "fa_rope_qk", [&](auto tag) {
     using E = decltype(tag);
+    if constexpr (sizeof(E) == 2) {
+      const uintptr_t ptrs = (uintptr_t)q_in | (uintptr_t)q_out | (uintptr_t)k | (uintptr_t)cos | (uintptr_t)sin;
+      if (D % 16 == 0 && (ptrs & 15) == 0 && q_in_stride % 8 == 0 && k_stride % 8 == 0) {
+        rope_qk_vec_kernel<E><<<rows, 256, 0, st>>>((const E*)q_in, q_in_stride, (E*)q_out, (E*)k, k_stride, (const E*)cos,
+                                                    (const E*)sin, Hq, Hkv, D);
+        return;
+      }
+    }
     rope_qk_kernel<E><<<dim3(rows, Hq + Hkv), D / 2, 0, st>>>((const E*)q_in, q_in_stride, (E*)q_out, (E*)k, k_stride,
                                                               (const E*)cos, (const E*)sin, Hq, Hkv, D);
   });
@@ -172,6 +225,13 @@ extern "C" int fa_silu_mul(const void* gate, const void* up, void* out, int rows
   hipStream_t st = fa_hip_stream(stream);
   int rc = by_dtype(dtype, "fa_silu_mul", [&](auto tag) {
     using E = decltype(tag);
+    if constexpr (sizeof(E) == 2) {
+      if (cols % 8 == 0 && in_stride % 8 == 0 && (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)out) & 15) == 0) {
+        silu_mul_vec_kernel<E><<<dim3(fa_cdiv(cols / 8, 256), rows), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out,
+                                                                                cols, in_stride);
+        return;
+      }
+    }
     silu_mul_kernel<E><<<dim3(fa_cdiv(cols, 256), rows), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out, cols, in_stride);
   });
   return rc != FA_OK ? rc : fa_check_launch("fa_silu_mul");

@@ -182,29 +182,32 @@ def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
         torch.testing.assert_close(y.float(), want_y.float(), rtol=ulp, atol=ulp)   # reduction order: last place only
         y0 = ops.add_rmsnorm(h2, None, norm.weight, 1e-5)                 # no delta: h untouched
         assert torch.equal(h2, want_h) and torch.equal(y0, y)
-    # rotary embedding: no reduction anywhere, so bit for bit
-    B, q_len, Hq, Hkv, D = 3, 2, 6, 2, 64
-    q, k = rn(B, q_len, Hq * D).to(dtype), rn(B, q_len, Hkv * D).to(dtype)
-    ang = rn(B, q_len, D) * 3
-    cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
-    wq, wk = apply_rotary_pos_emb(q.view(B, q_len, Hq, D).transpose(1, 2), k.view(B, q_len, Hkv, D).transpose(1, 2), cos, sin)
-    q2, k2 = q.clone(), k.clone()
-    ops.rope_qk_(q2, k2, cos, sin, D)
-    assert torch.equal(q2.view(B, q_len, Hq, D).transpose(1, 2), wq) and torch.equal(k2.view(B, q_len, Hkv, D).transpose(1, 2), wk)
-    # the same on column slices of one fused projection output: q comes back densely packed, k is rotated where it lies
-    qkv = torch.cat([q, k, rn(B, q_len, Hkv * D).to(dtype)], dim=-1)
-    qs, ks, vs = qkv.split((Hq * D, Hkv * D, Hkv * D), dim=-1)
-    v_before = vs.clone()
-    q3 = ops.rope_qk(qs, ks, cos, sin, D)
-    assert q3.is_contiguous() and torch.equal(q3, q2) and torch.equal(ks, k2) and torch.equal(vs, v_before)
-    # SwiGLU gate: the exponential may differ in the last place
-    gate, up = (rn(7, 1, 1111) * 3).to(dtype), rn(7, 1, 1111).to(dtype)
-    want = torch.nn.functional.silu(gate) * up
-    got = ops.silu_mul(gate, up)
-    torch.testing.assert_close(got.float(), want.float(), rtol=2 * ulp, atol=2 * ulp)
-    g2, u2 = torch.cat([gate, up], dim=-1).chunk(2, dim=-1)              # column slices of one wider row
-    got2 = ops.silu_mul(g2, u2)
-    assert got2.is_contiguous() and torch.equal(got2, got)
+    # rotary embedding: no reduction anywhere, so bit for bit (head dims of 64: 16 bytes per thread with 16-bit
+    # storage; of 40: the element-wise variant)
+    for D in (64, 40):
+        B, q_len, Hq, Hkv = 3, 2, 6, 2
+        q, k = rn(B, q_len, Hq * D).to(dtype), rn(B, q_len, Hkv * D).to(dtype)
+        ang = rn(B, q_len, D) * 3
+        cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
+        wq, wk = apply_rotary_pos_emb(q.view(B, q_len, Hq, D).transpose(1, 2), k.view(B, q_len, Hkv, D).transpose(1, 2), cos, sin)
+        q2, k2 = q.clone(), k.clone()
+        ops.rope_qk_(q2, k2, cos, sin, D)
+        assert torch.equal(q2.view(B, q_len, Hq, D).transpose(1, 2), wq) and torch.equal(k2.view(B, q_len, Hkv, D).transpose(1, 2), wk)
+        # the same on column slices of one fused projection output: q comes back densely packed, k is rotated where it lies
+        qkv = torch.cat([q, k, rn(B, q_len, Hkv * D).to(dtype)], dim=-1)
+        qs, ks, vs = qkv.split((Hq * D, Hkv * D, Hkv * D), dim=-1)
+        v_before = vs.clone()
+        q3 = ops.rope_qk(qs, ks, cos, sin, D)
+        assert q3.is_contiguous() and torch.equal(q3, q2) and torch.equal(ks, k2) and torch.equal(vs, v_before)
+    # SwiGLU gate: the exponential may differ in the last place (1111 columns: element-wise; 2048: 16 bytes per thread)
+    for cols in (1111, 2048):
+        gate, up = (rn(7, 1, cols) * 3).to(dtype), rn(7, 1, cols).to(dtype)
+        want = torch.nn.functional.silu(gate) * up
+        got = ops.silu_mul(gate, up)
+        torch.testing.assert_close(got.float(), want.float(), rtol=2 * ulp, atol=2 * ulp)
+        g2, u2 = torch.cat([gate, up], dim=-1).chunk(2, dim=-1)              # column slices of one wider row
+        got2 = ops.silu_mul(g2, u2)
+        assert got2.is_contiguous() and torch.equal(got2, got)
 
 
 @pytest.mark.gpu
