@@ -204,7 +204,8 @@ extern "C" int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, vo
     using E = decltype(tag);
     if constexpr (sizeof(E) == 2) {
       const uintptr_t ptrs = (uintptr_t)q_in | (uintptr_t)q_out | (uintptr_t)k | (uintptr_t)cos | (uintptr_t)sin;
-      if (D % 16 == 0 && (ptrs & 15) == 0 && q_in_stride % 8 == 0 && k_stride % 8 == 0) {
+      // (a decode step has too few rows to fill the device with one block per row: those keep one block per head)
+      if (rows >= 64 && D % 16 == 0 && (ptrs & 15) == 0 && q_in_stride % 8 == 0 && k_stride % 8 == 0) {
         rope_qk_vec_kernel<E><<<rows, 256, 0, st>>>((const E*)q_in, q_in_stride, (E*)q_out, (E*)k, k_stride, (const E*)cos,
                                                     (const E*)sin, Hq, Hkv, D);
         return;

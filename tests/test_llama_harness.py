@@ -182,10 +182,10 @@ def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
         torch.testing.assert_close(y.float(), want_y.float(), rtol=ulp, atol=ulp)   # reduction order: last place only
         y0 = ops.add_rmsnorm(h2, None, norm.weight, 1e-5)                 # no delta: h untouched
         assert torch.equal(h2, want_h) and torch.equal(y0, y)
-    # rotary embedding: no reduction anywhere, so bit for bit (head dims of 64: 16 bytes per thread with 16-bit
-    # storage; of 40: the element-wise variant)
-    for D in (64, 40):
-        B, q_len, Hq, Hkv = 3, 2, 6, 2
+    # rotary embedding: no reduction anywhere, so bit for bit (head dims of 64 and at least 64 rows: 16 bytes per
+    # thread with 16-bit storage; otherwise the element-wise variant)
+    for D, q_len in ((64, 40), (64, 2), (40, 2)):   # 120 rows; a few rows (one block per head); odd head dim
+        B, Hq, Hkv = 3, 6, 2
         q, k = rn(B, q_len, Hq * D).to(dtype), rn(B, q_len, Hkv * D).to(dtype)
         ang = rn(B, q_len, D) * 3
         cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
