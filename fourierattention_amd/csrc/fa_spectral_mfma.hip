@@ -90,7 +90,8 @@ __global__ __launch_bounds__(256) void spectral_pack_kernel(
 struct SpectralGemmParams {
   const half8* tab;      // basis table
   const half8* packed;   // [B][CT][KS32][64] fragments
-  float* part;           // [S][B][2N][Mc]
+  float* part;           // [S][B][2N][Mc]; with a single chunk: the result c itself (no reduction launch)
+  int add_to_part;       // single chunk only: add to what part holds instead of overwriting it
   int B, N, Mc, CT, KS32, T;
   int n_steps, steps_per_chunk, n_chunks;
   int64_t k_start;
@@ -191,8 +192,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int m = (ct0 + j) * 16 + lc;
         if (m < p.Mc) {
           const float c = acc[i][j][2 * f2], s_ = acc[i][j][2 * f2 + 1];
-          out[(int64_t)n * p.Mc + m] = co * c - sn * s_;
-          out[(int64_t)(p.N + n) * p.Mc + m] = sn * c + co * s_;
+          float* oc = out + (int64_t)n * p.Mc + m;
+          float* os = out + (int64_t)(p.N + n) * p.Mc + m;
+          const float vc = co * c - sn * s_, vs = sn * c + co * s_;
+          *oc = p.add_to_part ? *oc + vc : vc;
+          *os = p.add_to_part ? *os + vs : vs;
         }
       }
     }
@@ -458,14 +462,16 @@ int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_
   else
     spectral_pack_kernel<f16_t><<<pgrid, 256, 0, st>>>((const f16_t*)a, a_bs, a_rs, cols, nullptr, packed, K, Mc, pl.CT, pl.KS32);
   SpectralGemmParams gp{};
-  gp.tab = tab; gp.packed = packed; gp.part = part;
+  const bool direct = pl.n_chunks == 1;   // nothing to sum: the GEMM writes (or adds to) c itself
+  gp.tab = tab; gp.packed = packed; gp.part = direct ? c : part;
+  gp.add_to_part = direct && accumulate;
   gp.B = B; gp.N = N; gp.Mc = Mc; gp.CT = pl.CT; gp.KS32 = pl.KS32; gp.T = T;
   gp.n_steps = pl.n_steps; gp.steps_per_chunk = pl.steps_per_chunk; gp.n_chunks = pl.n_chunks;
   gp.k_start = k_start;
   dim3 ggrid(fa_cdiv(Mc, kWgCols), fa_cdiv(N, kWgFreqs), B * pl.n_chunks);
   spectral_gemm_kernel<<<ggrid, 256, 0, st>>>(gp);
   const int64_t total = (int64_t)B * 2 * N * Mc;
-  spectral_reduce_kernel<<<fa_cdiv(total / 4, 256), 256, 0, st>>>(part, c, total, pl.n_chunks, accumulate);
+  if (!direct) spectral_reduce_kernel<<<fa_cdiv(total / 4, 256), 256, 0, st>>>(part, c, total, pl.n_chunks, accumulate);
   return fa_check_launch("fa_mat_fourier");
 }
 
