@@ -98,6 +98,9 @@ _SIGNATURES = {
     "fa_decode_attn": (c_int, [POINTER(DecodeArgs), c_void_p]),
     "fa_decode_attn_noalloc": (c_int, [POINTER(DecodeArgs), c_void_p]),
     "fa_decode_attn_timed": (c_int, [POINTER(DecodeArgs), c_void_p, POINTER(c_float)]),
+    "fa_linear_pack": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "fa_linear_packed_ok": (c_int, [c_int, c_int, c_int]),
+    "fa_linear_packed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "fa_decode_split_plan": (c_int, [c_int] * 7 + [c_void_p, c_void_p, c_void_p, c_void_p]),
     "fa_decode_tables_bytes": (c_size_t, [c_int]),
     "fa_decode_tables_build": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),

@@ -4,6 +4,7 @@
 // of a 16-bit model rounds its result to that type), so the results agree with that chain to the last bit
 // except where a reduction order or an exponential differs in the last place.
 #include "fa_common.h"
+#include "fa_mfma_util.h"
 
 namespace {
 
@@ -160,6 +161,84 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const E* __restrict__ gat
   out[row * cols + i] = Rounder<E>::put(rnd<E>(g / (1.0f + expf(-g))) * fa_to_float(up[row * in_stride + i]));
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Projections of a decode step: out[rows <= 16][n_out] = x[rows][K] . W[n_out][K]^T (nn.Linear without bias,
+// modeling_llama_fourier.py:283, 597-599, 665).  With a handful of rows the product is a stream over the weights,
+// so they are kept in the order the matrix cores take them: fragment (tile of 16 output features, step of 32 input
+// features) = 64 lanes x 8 elements, lane (lg, lc) holding W[16 tile + lc][32 step + 8 lg ..] - every load is one
+// contiguous KiB and goes straight into an MFMA as the A operand.  A workgroup owns one tile of 16 output features;
+// its eight waves share the input features, keep two groups of four fragments in flight each, and meet in LDS.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kLinWaves = 8, kLinGroup = 4;
+
+template <typename E>
+__global__ __launch_bounds__(256) void linear_pack_kernel(const E* __restrict__ w, E* __restrict__ packed, int n_out, int K) {
+  struct alignas(16) Pack { E e[8]; };
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one 16-byte piece: (tile, step, lane)
+  const int KS = K >> 5;
+  if (idx >= (int64_t)(n_out >> 4) * KS * 64) return;
+  const int lane = (int)(idx & 63), lg = lane >> 4, lc = lane & 15;
+  const int64_t frag = idx >> 6;
+  const int ks = (int)(frag % KS);
+  const int64_t tile = frag / KS;
+  *(Pack*)(packed + idx * 8) = *(const Pack*)(w + (tile * 16 + lc) * K + ks * 32 + 8 * lg);
+}
+
+template <typename E>
+__global__ __launch_bounds__(64 * kLinWaves) void linear_packed_kernel(const E* __restrict__ x, int64_t x_rs,
+                                                                        const E* __restrict__ wp, E* __restrict__ out,
+                                                                        int rows, int K, int n_out) {
+  using M = fa_mfma::Mma<E>;
+  using vec8 = typename M::vec8;
+  using fa_mfma::float4v;
+  using fa_mfma::uint4v;
+  __shared__ float4v s_part[kLinWaves][64];
+  const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tile = blockIdx.x;
+  const int KS = K >> 5, per_wave = KS / kLinWaves, n_groups = per_wave / kLinGroup;
+  const bool row_ok = lc < rows;
+  const uint4v* a_ptr = (const uint4v*)wp + ((int64_t)tile * KS + w * per_wave) * 64 + lane;
+  const E* b_row = x + (int64_t)(row_ok ? lc : 0) * x_rs + w * per_wave * 32 + 8 * lg;
+  float4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  uint4v A0[kLinGroup], B0[kLinGroup], A1[kLinGroup], B1[kLinGroup];
+  auto load = [&](int g, uint4v (&A)[kLinGroup], uint4v (&B)[kLinGroup]) {
+#pragma unroll
+    for (int i = 0; i < kLinGroup; ++i) {
+      A[i] = __builtin_nontemporal_load(a_ptr + (int64_t)(g * kLinGroup + i) * 64);   // read once: keep it out of the caches
+      B[i] = *(const uint4v*)(b_row + (g * kLinGroup + i) * 32);
+    }
+  };
+  auto compute = [&](uint4v (&A)[kLinGroup], uint4v (&B)[kLinGroup]) {
+#pragma unroll
+    for (int i = 0; i < kLinGroup; ++i) {
+      uint4v b = B[i];
+      if (!row_ok) b = uint4v{0u, 0u, 0u, 0u};   // columns past the rows: the clamped row must not reach the result
+      if (i & 1) acc1 = M::mma(__builtin_bit_cast(vec8, A[i]), __builtin_bit_cast(vec8, b), acc1);
+      else acc0 = M::mma(__builtin_bit_cast(vec8, A[i]), __builtin_bit_cast(vec8, b), acc0);
+    }
+  };
+  load(0, A0, B0);
+  for (int g = 0; g < n_groups; g += 2) {
+    if (g + 1 < n_groups) load(g + 1, A1, B1);
+    compute(A0, B0);
+    if (g + 2 < n_groups) load(g + 2, A0, B0);
+    if (g + 1 < n_groups) compute(A1, B1);
+  }
+  s_part[w][lane] = acc0 + acc1;
+  __syncthreads();
+  if (w == 0 && row_ok) {
+    float4v s = s_part[0][lane];
+#pragma unroll
+    for (int i = 1; i < kLinWaves; ++i) s += s_part[i][lane];
+    // lane (lg, lc) holds the output features 4 lg .. 4 lg + 3 of the tile for row lc
+    struct alignas(sizeof(E) * 4) Quad { E e[4]; } o;
+    o.e[0] = Rounder<E>::put(s.x); o.e[1] = Rounder<E>::put(s.y);
+    o.e[2] = Rounder<E>::put(s.z); o.e[3] = Rounder<E>::put(s.w);
+    *(Quad*)(out + (int64_t)lc * n_out + tile * 16 + 4 * lg) = o;
+  }
+}
+
 template <typename F>
 int by_dtype(int dtype, const char* what, F&& f) {
   switch (dtype) {
@@ -236,4 +315,43 @@ extern "C" int fa_silu_mul(const void* gate, const void* up, void* out, int rows
     silu_mul_kernel<E><<<dim3(fa_cdiv(cols, 256), rows), 256, 0, st>>>((const E*)gate, (const E*)up, (E*)out, cols, in_stride);
   });
   return rc != FA_OK ? rc : fa_check_launch("fa_silu_mul");
+}
+
+extern "C" int fa_linear_pack(const void* w, void* packed, int n_out, int K, int dtype, fa_stream_t stream) {
+  FA_REQUIRE(w && packed, FA_ERR_NULL_POINTER, "fa_linear_pack: null pointer");
+  FA_REQUIRE(n_out > 0 && K > 0 && n_out % 16 == 0 && K % 32 == 0, FA_ERR_BAD_SHAPE,
+             "fa_linear_pack: n_out=%d (multiple of 16) K=%d (multiple of 32)", n_out, K);
+  FA_REQUIRE(dtype == FA_BF16 || dtype == FA_FP16, FA_ERR_BAD_DTYPE, "fa_linear_pack: dtype %d (16-bit storage only)", dtype);
+  FA_REQUIRE((((uintptr_t)w | (uintptr_t)packed) & 15) == 0, FA_ERR_MISALIGNED, "fa_linear_pack: pointers not 16-byte aligned");
+  hipStream_t st = fa_hip_stream(stream);
+  const int64_t pieces = (int64_t)(n_out / 16) * (K / 32) * 64;
+  by_dtype(dtype, "fa_linear_pack", [&](auto tag) {
+    using E = decltype(tag);
+    if constexpr (sizeof(E) == 2)
+      linear_pack_kernel<E><<<(unsigned)fa_cdiv(pieces, (int64_t)256), 256, 0, st>>>((const E*)w, (E*)packed, n_out, K);
+  });
+  return fa_check_launch("fa_linear_pack");
+}
+
+extern "C" int fa_linear_packed_ok(int rows, int K, int n_out) {
+  return rows >= 1 && rows <= 16 && n_out > 0 && n_out % 16 == 0 && K > 0 && K % (32 * kLinWaves * kLinGroup) == 0;
+}
+
+extern "C" int fa_linear_packed(const void* x, int64_t x_row_stride, const void* w_packed, void* out, int rows, int K,
+                                int n_out, int dtype, fa_stream_t stream) {
+  FA_REQUIRE(x && w_packed && out, FA_ERR_NULL_POINTER, "fa_linear_packed: null pointer");
+  FA_REQUIRE(fa_linear_packed_ok(rows, K, n_out), FA_ERR_UNSUPPORTED,
+             "fa_linear_packed: rows=%d (1..16) K=%d (multiple of %d) n_out=%d (multiple of 16)", rows, K,
+             32 * kLinWaves * kLinGroup, n_out);
+  FA_REQUIRE(dtype == FA_BF16 || dtype == FA_FP16, FA_ERR_BAD_DTYPE, "fa_linear_packed: dtype %d (16-bit storage only)", dtype);
+  FA_REQUIRE(x_row_stride >= K && x_row_stride % 8 == 0 && (((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)out) & 15) == 0,
+             FA_ERR_MISALIGNED, "fa_linear_packed: rows of x / pointers not 16-byte aligned");
+  hipStream_t st = fa_hip_stream(stream);
+  by_dtype(dtype, "fa_linear_packed", [&](auto tag) {
+    using E = decltype(tag);
+    if constexpr (sizeof(E) == 2)
+      linear_packed_kernel<E><<<n_out / 16, 64 * kLinWaves, 0, st>>>((const E*)x, x_row_stride, (const E*)w_packed, (E*)out,
+                                                                    rows, K, n_out);
+  });
+  return fa_check_launch("fa_linear_packed");
 }

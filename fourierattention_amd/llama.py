@@ -86,6 +86,28 @@ class LlamaDecoderLayer(nn.Module):
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self._qkv_weight = self._gate_up_weight = None
+        self._packed = {}   # "qkv", "o", "gate_up", "down" -> ops.PackedLinearWeight (decode steps of at most 16 rows)
+
+    def pack_projections(self):
+        """Keeps a second copy of the four weight groups in the order ``ops.linear_packed`` streams them (16-bit GPU
+        weights without bias).  A decode step of at most 16 rows then runs its projections on those copies; prompts
+        keep using the row-major weights through the GEMM library.  Doubles the memory of the layer's weights."""
+        at, mlp = self.self_attn, self.mlp
+        w = at.q_proj.weight
+        if at.q_proj.bias is not None or mlp.gate_proj.bias is not None or not w.is_cuda or w.dtype not in (torch.bfloat16, torch.float16):
+            return
+        groups = {"qkv": (at.q_proj, at.k_proj, at.v_proj), "o": (at.o_proj,), "gate_up": (mlp.gate_proj, mlp.up_proj),
+                  "down": (mlp.down_proj,)}
+        for name, mods in groups.items():
+            n_out, k = sum(m.weight.shape[0] for m in mods), mods[0].weight.shape[1]
+            if n_out % 16 or k % 1024:
+                continue
+            fused = mods[0].weight.data if len(mods) == 1 else torch.cat([m.weight.data for m in mods], dim=0)
+            self._packed[name] = ops.PackedLinearWeight(fused.contiguous())
+
+    def _linear(self, name, x, fallback):
+        w = self._packed.get(name)
+        return ops.linear_packed(x, w) if w is not None and w.covers(x) else fallback(x)
 
     def fuse_projections(self, max_rows: int = 16384):
         """Moves the q/k/v weights into one tensor and the gate/up weights into another; the five modules keep
@@ -121,8 +143,11 @@ class LlamaDecoderLayer(nn.Module):
         at = self.self_attn
         y = ops.add_rmsnorm(h, delta, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
         bsz, q_len, _ = y.shape
-        if self._qkv_weight is not None:
-            nq, nk = at.num_heads * at.head_dim, at.num_key_value_heads * at.head_dim
+        nq, nk = at.num_heads * at.head_dim, at.num_key_value_heads * at.head_dim
+        pk = self._packed.get("qkv")
+        if pk is not None and pk.covers(y):
+            q, k, v = ops.linear_packed(y, pk).split((nq, nk, nk), dim=-1)
+        elif self._qkv_weight is not None:
             q, k, v = F.linear(y, self._qkv_weight).split((nq, nk, nk), dim=-1)
         else:
             q, k, v = at.q_proj(y), at.k_proj(y), at.v_proj(y)
@@ -132,13 +157,16 @@ class LlamaDecoderLayer(nn.Module):
         o = fourier_attention(split(q, at.num_heads), split(k, at.num_key_value_heads), split(v, at.num_key_value_heads),
                               past_key_value, at.layer_idx, at.num_heads, at.num_key_value_heads,
                               {"sin": sin, "cos": cos, "cache_position": cache_position})
-        y = ops.add_rmsnorm(h, at.o_proj(o), self.post_attention_layernorm.weight,
+        y = ops.add_rmsnorm(h, self._linear("o", o, at.o_proj), self.post_attention_layernorm.weight,
                             self.post_attention_layernorm.variance_epsilon)
-        if self._gate_up_weight is not None:
+        pk = self._packed.get("gate_up")
+        if pk is not None and pk.covers(y):
+            gate, up = ops.linear_packed(y, pk).chunk(2, dim=-1)
+        elif self._gate_up_weight is not None:
             gate, up = F.linear(y, self._gate_up_weight).chunk(2, dim=-1)
         else:
             gate, up = self.mlp.gate_proj(y), self.mlp.up_proj(y)
-        return self.mlp.down_proj(ops.silu_mul(gate, up))
+        return self._linear("down", ops.silu_mul(gate, up), self.mlp.down_proj)
 
 
 class LlamaModel(nn.Module):
@@ -156,6 +184,11 @@ class LlamaModel(nn.Module):
     def fuse_projections(self, max_rows: int = 16384):
         for layer in self.layers:
             layer.fuse_projections(max_rows)
+        return self
+
+    def pack_projections(self):
+        for layer in self.layers:
+            layer.pack_projections()
         return self
 
     def forward(self, input_ids, past_key_values: DynamicCache, position_ids=None):

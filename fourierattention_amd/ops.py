@@ -281,6 +281,39 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+class PackedLinearWeight:
+    """A bias-free ``nn.Linear`` weight ``(n_out, K)`` re-laid for ``linear_packed``: the order in which the matrix
+    cores take it, so that a decode step (a handful of rows) streams it in contiguous KiB pieces."""
+
+    def __init__(self, weight: torch.Tensor):
+        _require_gpu(weight, "weight")
+        assert weight.dim() == 2 and weight.is_contiguous() and weight.dtype in (torch.bfloat16, torch.float16)
+        self.n_out, self.k = int(weight.shape[0]), int(weight.shape[1])
+        self.dtype = weight.dtype
+        self.data = torch.empty_like(weight)
+        check(_lib.load().fa_linear_pack(weight.data_ptr(), self.data.data_ptr(), self.n_out, self.k, dtype_code(weight.dtype),
+                                         _stream(weight.device)))
+
+    def covers(self, x: torch.Tensor) -> bool:
+        rows = x.numel() // max(x.shape[-1], 1)
+        return (x.is_cuda and x.dtype == self.dtype and x.shape[-1] == self.k and x.stride(-1) == 1
+                and bool(_lib.load().fa_linear_packed_ok(rows, self.k, self.n_out)))
+
+
+def linear_packed(x: torch.Tensor, w: PackedLinearWeight) -> torch.Tensor:
+    """``F.linear(x, weight)`` for ``x (..., K)`` of at most 16 rows (fp32 accumulation, result in the storage type)
+    on the packed weight; rows must be evenly spaced (dense, or slices of wider rows)."""
+    assert w.covers(x), "shape not covered: at most 16 rows, K a multiple of 1024, n_out of 16"
+    rows = x.numel() // w.k
+    stride = x.stride(-2) if x.dim() >= 2 and rows > 1 else w.k
+    assert all(x.shape[d] == 1 or x.stride(d) == x.stride(d + 1) * x.shape[d + 1] for d in range(x.dim() - 2)), \
+        "rows are not evenly spaced"
+    out = torch.empty(x.shape[:-1] + (w.n_out,), dtype=x.dtype, device=x.device)
+    check(_lib.load().fa_linear_packed(x.data_ptr(), stride, w.data.data_ptr(), out.data_ptr(), rows, w.k, w.n_out,
+                                       dtype_code(x.dtype), _stream(x.device)))
+    return out
+
+
 def prefill_attention_supported(q: torch.Tensor, k: torch.Tensor, head_dim: int) -> bool:
     """Shapes the matrix-core prompt attention covers: 16-bit GPU tensors, heads of 64 or 128 dims, 16-byte rows."""
     return (q.is_cuda and q.dtype in (torch.bfloat16, torch.float16) and k.dtype == q.dtype and head_dim in (64, 128)

@@ -359,6 +359,19 @@ int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, void* k, int6
 int fa_silu_mul(const void* gate, const void* up, void* out, int rows, int cols, int64_t in_stride,
                 int dtype, fa_stream_t stream);
 
+/* The projections of a decode step, nn.Linear without bias (q/k/v_proj MODEL:597-599, o_proj MODEL:665, the MLP
+ * MODEL:283): out[r][n] = sum_k x[r][k] * w[n][k] for a handful of rows, where the product is one pass over the
+ * weights.  fa_linear_pack re-lays a row-major weight (n_out, K) once, in the order the matrix cores take it
+ * (tile of 16 output features x step of 32 input features = 64 lanes x 8 elements, lane 16 g + c holding
+ * w[16 tile + c][32 step + 8 g ..]); fa_linear_packed multiplies: x (rows, K) with rows x_row_stride elements apart,
+ * out (rows, n_out) densely packed, fp32 accumulation, result rounded to `dtype`.  16-bit storage only;
+ * fa_linear_packed_ok says whether a shape is covered (1 <= rows <= 16, n_out a multiple of 16, K of 1024): other
+ * shapes belong to a GEMM library. */
+int fa_linear_pack(const void* w, void* packed, int n_out, int K, int dtype, fa_stream_t stream);
+int fa_linear_packed_ok(int rows, int K, int n_out);
+int fa_linear_packed(const void* x, int64_t x_row_stride, const void* w_packed, void* out, int rows, int K,
+                     int n_out, int dtype, fa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

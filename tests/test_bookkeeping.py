@@ -248,6 +248,14 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_silu_mul(p, p, None, 1, 8, 8, 0, None) == -1
     assert lib.fa_silu_mul(p, p, p, -1, 8, 8, 0, None) == -2
     assert lib.fa_silu_mul(p, p, p, 2, 8, 4, 0, None) == -2                        # stride shorter than a row
+    assert lib.fa_linear_pack(None, p, 16, 1024, 0, None) == -1
+    assert lib.fa_linear_pack(p, p, 24, 1024, 0, None) == -2                       # output features not a multiple of 16
+    assert lib.fa_linear_pack(p, p, 16, 1024, 2, None) == -3                       # float32 storage
+    assert lib.fa_linear_packed(p, 1024, p, None, 1, 1024, 16, 0, None) == -1
+    assert lib.fa_linear_packed(p, 1024, p, p, 17, 1024, 16, 0, None) == -5        # more than 16 rows: the GEMM library's
+    assert lib.fa_linear_packed(p, 1536, p, p, 1, 1536, 16, 0, None) == -5         # K not a multiple of 1024
+    assert lib.fa_linear_packed(p, 1000, p, p, 2, 1024, 16, 0, None) == -7         # rows of x closer than K
+    assert lib.fa_linear_packed_ok(16, 4096, 6144) == 1 and lib.fa_linear_packed_ok(0, 4096, 6144) == 0
     assert lib.fa_stream_update(None, None) == -1
     sa = _lib.StreamArgs()
     assert lib.fa_stream_update(ctypes.byref(sa), None) == -2                  # empty shape

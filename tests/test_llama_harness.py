@@ -245,3 +245,62 @@ def test_fused_decoder_path_matches_the_module_chain():
     # a wider GEMM may pick another tiling, hence another summation order inside the dot products
     torch.testing.assert_close(outs[2], outs[0], rtol=3e-2, atol=3e-2)
     assert (outs[2] - outs[0]).abs().mean().item() < 3e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_packed_linear_matches_the_library_product(dtype):
+    """``fa_linear_packed`` (projections of a decode step on weights re-laid for the matrix cores) against the fp32
+    product of the same 16-bit operands: fp32 accumulation either way, so what is left is the rounding of the result
+    (half a unit in the last place of the storage type) plus the order of the sums."""
+    from fourierattention_amd import ops
+    g = torch.Generator(device="cuda").manual_seed(5)
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    for rows, K, n_out in ((16, 4096, 6144), (4, 3072, 5120), (1, 1024, 16), (7, 14336, 4096), (16, 2048, 28672)):
+        w = (torch.randn(n_out, K, generator=g, device="cuda") * 0.05).to(dtype)
+        x = torch.randn(rows, 1, K, generator=g, device="cuda").to(dtype)
+        pw = ops.PackedLinearWeight(w)
+        assert pw.covers(x)
+        got = ops.linear_packed(x, pw)
+        want = torch.nn.functional.linear(x.float(), w.float())
+        assert got.shape == (rows, 1, n_out) and got.dtype == dtype
+        bound = 0.75 * ulp * want.abs().max().item() + 1e-6
+        assert (got.float() - want).abs().max().item() <= bound
+        # rows that are slices of wider rows (a fused projection output, as the decoder hands them over)
+        wide = torch.cat([x, torch.randn(rows, 1, 64, generator=g, device="cuda").to(dtype)], dim=-1)
+        assert torch.equal(ops.linear_packed(wide[..., :K], pw), got)
+    # shapes outside the kernel are for the GEMM library
+    assert not pw.covers(torch.zeros(17, 2048, dtype=dtype, device="cuda"))
+    assert not ops.PackedLinearWeight(torch.zeros(16, 1536, dtype=dtype, device="cuda")).covers(torch.zeros(1, 1536, dtype=dtype, device="cuda"))
+
+
+@pytest.mark.gpu
+def test_decoder_steps_on_packed_projections():
+    """The same bf16 model stepped with the projections of its decode steps on the packed weights and through the
+    GEMM library (the prompt goes through the library either way)."""
+    from fourierattention_amd import DynamicCache
+    from fourierattention_amd.llama import LlamaConfig, random_init
+    cfg = LlamaConfig(hidden_size=1024, intermediate_size=2048, num_hidden_layers=2, num_attention_heads=8,
+                      num_key_value_heads=2, head_dim=128, vocab_size=301)
+    model = random_init(cfg, dtype=torch.bfloat16, device="cuda:0", seed=7, std=0.03)
+    model.model.fuse_projections()
+    masks = _masks(2, 2, 128, [64, 64], [64, 64], seed=4)
+    ec = lambda: _cfg(masks, numinittokens=4, maxlocallen=32, maxmidstates=64, num_key_value_heads=2, max_new_tokens=8,
+                      max_position_embeddings=1024)
+    ids = torch.randint(0, cfg.vocab_size, (3, 200), generator=torch.Generator().manual_seed(3)).cuda()
+    outs = []
+    with torch.no_grad():
+        for packed in (False, True):
+            if packed:
+                model.model.pack_projections()
+                assert set(model.model.layers[0]._packed) == {"qkv", "o", "gate_up", "down"}
+            cache = DynamicCache(ec())
+            logits = [model(input_ids=ids, past_key_values=cache, num_logits_to_keep=1).logits[:, -1]]
+            tok = logits[0].argmax(-1, keepdim=True)
+            for _ in range(3):
+                logits.append(model(input_ids=tok, past_key_values=cache, num_logits_to_keep=1).logits[:, -1])
+                tok = logits[-1].argmax(-1, keepdim=True)
+            outs.append(torch.stack(logits))
+    assert torch.equal(outs[0][0], outs[1][0])                     # the prompt pass does not touch the packed weights
+    torch.testing.assert_close(outs[1], outs[0], rtol=3e-2, atol=3e-2)   # another summation order inside the dot products
+    assert (outs[1] - outs[0]).abs().mean().item() < 3e-3
