@@ -101,8 +101,8 @@ static inline int tables_entries(int N) {
 static inline size_t tables_bytes(int N) { return (size_t)tables_entries(N) * 16 + (size_t)N * 8; }
 
 
-// ---- page-step rotation of coefficient-domain state ---------------------------------------------------
-// Both wave roles turn 2*KS row tiles of (cos, sin) pairs by the per-frequency angle of one page.  The
+// ---- frame-to-frame rotation of coefficient-domain state ---------------------------------------------------
+// Both wave roles turn 2*KS row tiles of (cos, sin) pairs by the per-frequency angle of one frame (64 tokens).  The
 // constants sit in LDS as float4 {c, s, c', s'} per (row tile, lane group), 64 bytes between row tiles.
 // They are fetched in batches of four tiles, two batches in flight, so that the LDS latency hides behind
 // the arithmetic of the previous batch instead of being paid once per tile.
@@ -585,7 +585,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
     const unsigned rot_lane = lds_addr_of(&s_rotv[(MODE == 1 ? 0 : sl * 2 * KS) * 4 + lg]);
-    // value pass: the scores of a page (column lc, tokens 8*lg .. 8*lg+7) are fetched one page ahead
+    // value pass: the scores of a page (column lc, positions 8*lg .. 8*lg+7) are fetched one page ahead
     float4v sc_next[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
     const float* sc_src = nullptr;
     if constexpr (MODE == 2) {
