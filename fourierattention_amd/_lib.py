@@ -106,6 +106,11 @@ _SIGNATURES = {
     "fa_decode_tables_build": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),
     "fa_mid_pack": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p,
                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "fa_prefill_compress_ok": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "fa_prefill_compress_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "fa_prefill_compress": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_int64, c_int,
+                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "fa_mid_append": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_void_p]),
     "fa_mid_unpack": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,

@@ -203,6 +203,7 @@ class DynamicCache(Cache):
         self._tables: Optional[torch.Tensor] = None   # constant operands of the MFMA decode kernels
         self.force_generic = False                     # testing: keep decode attention off the MFMA kernels
         self.balance_heads = True                      # mid rows: more splits for heads that store more dims
+        self.fuse_prefill = True                       # prefill: pages, coefficients and statistics from one read
         self._book = CacheBook(self._num_layers, self.numinittokens, self.maxlocallen, self.maxmidstates,
                                self.maxnewtokens, self.maxtokens)
         self._layers: List[_Layer] = [_Layer() for _ in range(self._num_layers)]
@@ -277,8 +278,8 @@ class DynamicCache(Cache):
         cut = self.numinittokens + layer.spare
         return [(layer.k.il[:, :cut, :], layer.v.il[:, :cut, :]), (layer.k.il[:, cut + 1:, :], layer.v.il[:, cut + 1:, :])]
 
-    def _compress_tensor(self, t: _Tensor, states: torch.Tensor, c32: torch.Tensor, n32: torch.Tensor, nh32: torch.Tensor,
-                         nh_host, is_v: bool, L: int, fft_rows: int, n_f: int):
+    def _compress_tensor(self, t: _Tensor, states: torch.Tensor, c32: torch.Tensor, ch32: torch.Tensor, n32: torch.Tensor,
+                         nh32: torch.Tensor, nh_host, is_v: bool, L: int, fft_rows: int, n_f: int):
         I, W = self.numinittokens, self.maxlocallen
         B, S, HD = states.shape
         mid = states[:, I: S - W, :]
@@ -289,10 +290,15 @@ class DynamicCache(Cache):
         t.ring[:, W, :].zero_()
         cap = max(self._book.t_x, L + int(self.maxnewtokens)) + 1     # room for every row the decode will evict
         t.mid = MidStore(B, n32, nh32, nh_host, self.heads, self.head_dim, cap, states.dtype, states.device, is_v)
-        t.mid.pack(states, I, L, head_dims=True)
-        # spectral compression of the selected columns (gather fused into the kernel)
-        t.coef = ops.mat_fourier(mid, n_f, self._book.t_c, 0, cols=c32, K=fft_rows)
-        u_avg, u_std = ops.mat_avg_std(mid, cols=c32, round_dtype=states.dtype)
+        fused = t.mid.pack_and_compress(states, I, L, fft_rows, c32, ch32, n_f, self._book.t_c, states.dtype) \
+            if self.fuse_prefill else None
+        if fused is not None:   # pages, coefficients and column statistics from one read of the rows
+            t.coef, u_avg, u_std = fused
+        else:
+            t.mid.pack(states, I, L, head_dims=True)
+            # spectral compression of the selected columns (gather fused into the kernel)
+            t.coef = ops.mat_fourier(mid, n_f, self._book.t_c, 0, cols=c32, K=fft_rows)
+            u_avg, u_std = ops.mat_avg_std(mid, cols=c32, round_dtype=states.dtype)
         i_avg, i_std = ops.mat_fourier_avg_std(t.coef, L, self._book.t_x, torch.float16)
         # dtypes as the reference leaves them: u_* in the model dtype, i_* in fp16, quotient promoted
         u_avg_m, u_std_m = u_avg.to(states.dtype), u_std.to(states.dtype)
@@ -335,9 +341,9 @@ class DynamicCache(Cache):
                 l32 = self._lists32[layer_idx]
                 n_f = self.maxmidstates // 2
                 hl = self._head_lists[layer_idx]
-                ks, ku, kd = self._compress_tensor(layer.k, k, l32[0], l32[2], l32[3], hl[0], False, step.mid_rows,
+                ks, ku, kd = self._compress_tensor(layer.k, k, l32[0], l32[1], l32[2], l32[3], hl[0], False, step.mid_rows,
                                                    step.fft_rows, n_f)
-                vs, vu, vd = self._compress_tensor(layer.v, v, l32[4], l32[6], l32[7], hl[1], True, step.mid_rows,
+                vs, vu, vd = self._compress_tensor(layer.v, v, l32[4], l32[5], l32[6], l32[7], hl[1], True, step.mid_rows,
                                                    step.fft_rows, n_f)
                 if self._tables is None and layer_idx == 0:
                     self._tables = ops.decode_tables(n_f, self.period_reconstruct, self.device)

@@ -31,6 +31,9 @@ size_t fa_recon_stats_mfma_workspace(int B, int N, int Mc, int K);
 // partial sums / maxima / minima of the reconstruction, [B][row blocks][Mc] each; returns the number of row blocks
 int fa_recon_stats_mfma_launch(const float* c, int B, int N, int Mc, int K, int T, void* workspace, float** psum,
                                float** pmax, float** pmin, hipStream_t st);
+// the last launch of the column statistics (fa_spectral.hip): partials [B][nsplit][Mc] -> mean and maximum deviation
+void fa_stats_finalize_launch(const float* psum, const float* pmax, const float* pmin, float* avg, float* dev, int B, int K,
+                              int Mc, int nsplit, int round_dtype, hipStream_t st);
 size_t fa_spectral_mfma_workspace(int B, int K, int Mc, int N);
 int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols, float* c, int B,
                             int K, int Mc, int N, int T, int64_t k_start, int accumulate, void* workspace,

@@ -320,6 +320,11 @@ int stats_splits(int K) { return K <= 0 ? 1 : fa_cdiv(K, 256); }
 
 }  // namespace
 
+void fa_stats_finalize_launch(const float* psum, const float* pmax, const float* pmin, float* avg, float* dev, int B, int K,
+                              int Mc, int nsplit, int round_dtype, hipStream_t st) {
+  stats_finalize_kernel<<<dim3(fa_cdiv(Mc, 64), B), 256, 0, st>>>(psum, pmax, pmin, avg, dev, K, Mc, nsplit, round_dtype);
+}
+
 // ---------------------------------------------------------------------------
 // C ABI
 // ---------------------------------------------------------------------------
@@ -336,7 +341,8 @@ extern "C" int fa_mat_fourier(const void* a, int a_dtype, int64_t a_bs, int64_t 
              "fa_mat_fourier: bad shape B=%d K=%d Mc=%d N=%d T=%d", B, K, Mc, N, T);
   FA_REQUIRE(a_dtype == FA_BF16 || a_dtype == FA_FP16 || a_dtype == FA_FP32, FA_ERR_BAD_DTYPE, "fa_mat_fourier: dtype %d",
              a_dtype);
-  if (workspace && fa_spectral_mfma_ok(a_dtype, K, Mc, N) && workspace_bytes >= fa_spectral_mfma_workspace(B, K, Mc, N)) {
+  if (workspace && ((uintptr_t)c & 15) == 0 && fa_spectral_mfma_ok(a_dtype, K, Mc, N) &&
+      workspace_bytes >= fa_spectral_mfma_workspace(B, K, Mc, N)) {
     FA_REQUIRE(((uintptr_t)workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_mat_fourier: workspace not 256-byte aligned");
     return fa_spectral_mfma_launch(a, a_dtype, a_bs, a_rs, cols, c, B, K, Mc, N, T, k_start, accumulate, workspace,
                                    fa_hip_stream(stream));

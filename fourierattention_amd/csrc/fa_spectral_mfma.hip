@@ -87,6 +87,126 @@ __global__ __launch_bounds__(256) void spectral_pack_kernel(
   }
 }
 
+// ---- one pass over the prompt's K (or V) rows for everything the cache's prefill needs from them -------------------
+// block = (PPB consecutive pages of 32 tokens, KV head, batch element); the head's slice of the rows goes through LDS
+// once and leaves as
+//   pages      the stored dims in the page layout of the decode kernels (what fa_mid_pack writes),
+//   fragments  the compressed dims as f16 B operands of the compression GEMM (what spectral_pack_kernel writes; a
+//              column tile that two heads share is written by both, each its own 16-byte pieces),
+//   partials   sum / max / min of every compressed column over the block's tokens (what col_stats_partial_kernel
+//              leaves, finished by the same final launch).
+constexpr int kPackPages = 4;   // pages per block
+
+template <typename E>
+struct PrefillPackParams {
+  const E* src;
+  int64_t src_bs, src_rs, row0;
+  int L, K_fft;                 // mid rows; rows that enter the transform (K_fft <= L)
+  E* store;                     // paged store of the stored dims
+  int64_t st_bs;
+  int cap_pages;
+  const int32_t* n_list; const int32_t* n_h; const int32_t* pad_h;   // stored dims: flat h*D + d, per-head offsets
+  const int32_t* c_list; const int32_t* c_h;                         // compressed dims, likewise
+  half8* packed;                // [B][CT][KS32][64]
+  float* psum; float* pmax; float* pmin;   // [B][n_blocks][Mc]
+  int Mc, CT, KS32, n_pages, n_blocks, Hkv, D, is_v;
+};
+
+template <typename E>
+__global__ __launch_bounds__(256) void prefill_pack_kernel(const PrefillPackParams<E> p) {
+  constexpr int kMaxD = 256;
+  constexpr int kPitch = kMaxD + 8;                 // elements; keeps rows 16-byte aligned
+  struct alignas(sizeof(E) * 8) Piece { E v[8]; };
+  __shared__ __attribute__((aligned(32))) E tile[32][kPitch];
+  __shared__ int s_col[kMaxD];                      // dim within the head of every stored position
+  __shared__ int s_ccol[kMaxD];                     // ... of every compressed position
+  const int h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x, D = p.D;
+  const int n0 = p.n_h[h], n_len = p.n_h[h + 1] - n0;
+  const int p0 = p.pad_h[h], dp = p.pad_h[h + 1] - p0;
+  const int c0 = p.c_h[h], c_len = p.c_h[h + 1] - c0;
+  for (int j = tid; j < dp; j += 256) s_col[j] = n_len > 0 ? min(max(p.n_list[n0 + min(j, n_len - 1)] - h * D, 0), D - 1) : 0;
+  for (int j = tid; j < c_len; j += 256) s_ccol[j] = min(max(p.c_list[c0 + j] - h * D, 0), D - 1);
+  const E* sb = p.src + (int64_t)b * p.src_bs + p.row0 * p.src_rs + (int64_t)h * D;
+  const int ppr = D >> 3;                           // 16-byte pieces per row of the head
+  const int pages_of_rows = (p.L + 31) >> 5;
+  // columns past the last compressed dim in the last column tile belong to nobody: the last head clears them
+  const int c_extra = h == p.Hkv - 1 ? p.CT * 16 - p.Mc : 0;
+  float sum = 0.f, mx = -INFINITY, mn = INFINITY;   // thread j < c_len: statistics of its column
+  for (int pp = 0; pp < kPackPages; ++pp) {
+    const int page = blockIdx.x * kPackPages + pp;
+    if (page >= p.n_pages) break;
+    __syncthreads();                                // the tile of the page before has been read (and the lists stored)
+    if (page < pages_of_rows) {
+      const int64_t last = (int64_t)p.L - 1;
+      for (int q = tid; q < 32 * ppr; q += 256) {
+        const int t = q / ppr, c = q - t * ppr;
+        const int64_t token = (int64_t)page * 32 + t;
+        *(Piece*)&tile[t][c * 8] = *(const Piece*)(sb + (token < last ? token : last) * p.src_rs + c * 8);
+      }
+    }
+    __syncthreads();
+    // ---- pages of the stored dims
+    if (page < pages_of_rows && n_len > 0) {
+      Piece* out = (Piece*)(p.store + (int64_t)b * p.st_bs + (int64_t)p0 * 32 * p.cap_pages + (int64_t)page * dp * 32);
+      const int n_pieces = dp * 32 / 8;
+      for (int piece = tid; piece < n_pieces; piece += 256) {
+        const int frag = piece >> 6, lane = piece & 63;
+        Piece o;
+        if (!p.is_v) {
+          const int nks = dp >> 5;
+          const int tb = frag / nks, s_ = frag - tb * nks;
+          const int t = tb * 16 + (lane & 15), j0 = s_ * 32 + 8 * (lane >> 4);
+          const bool row_ok = (int64_t)page * 32 + t < p.L;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o.v[e] = (row_ok && j0 + e < n_len) ? tile[t][s_col[j0 + e]] : E{};
+        } else {
+          const int j = frag * 16 + (lane & 15);
+          const int col = s_col[j];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int t = 8 * (lane >> 4) + i;
+            o.v[i] = (j < n_len && (int64_t)page * 32 + t < p.L) ? tile[t][col] : E{};
+          }
+        }
+        out[piece] = o;
+      }
+    }
+    // ---- f16 fragments of the compressed dims (tokens past the transform's rows are zero)
+    if (page < p.KS32) {
+      for (int idx = tid; idx < (c_len + c_extra) * 4; idx += 256) {
+        const int j = idx >> 2, lg = idx & 3;
+        const int m = c0 + j;                       // column of the compressed matrix
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int t = 8 * lg + e;
+          float x = 0.f;
+          if (j < c_len && (int64_t)page * 32 + t < p.K_fft) x = fminf(fmaxf(fa_to_float(tile[t][s_ccol[j]]), -65504.f), 65504.f);
+          o[e] = (_Float16)x;
+        }
+        p.packed[(((int64_t)b * p.CT + (m >> 4)) * p.KS32 + page) * 64 + lg * 16 + (m & 15)] = o;
+      }
+    }
+    // ---- column statistics over the mid rows
+    if (tid < c_len && page < pages_of_rows) {
+      const int col = s_ccol[tid];
+      const int n_t = min(32, p.L - page * 32);
+      for (int t = 0; t < n_t; ++t) {
+        const float v = fa_to_float(tile[t][col]);
+        sum += v;
+        mx = fmaxf(mx, v);
+        mn = fminf(mn, v);
+      }
+    }
+  }
+  if (tid < c_len) {
+    const int64_t o = ((int64_t)b * p.n_blocks + blockIdx.x) * p.Mc + c0 + tid;
+    p.psum[o] = sum;
+    p.pmax[o] = mx;
+    p.pmin[o] = mn;
+  }
+}
+
 struct SpectralGemmParams {
   const half8* tab;      // basis table
   const half8* packed;   // [B][CT][KS32][64] fragments
@@ -206,7 +326,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 __global__ __launch_bounds__(256) void spectral_reduce_kernel(const float* __restrict__ part, float* __restrict__ c,
                                                               int64_t total, int n_chunks, int accumulate) {
   const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-  if (i >= total) return;   // total is a multiple of 4 (Mc is even and 2N a multiple of 16)
+  if (i >= total) return;   // total is a multiple of 16 whatever Mc is: 2N is one
   float4 a = accumulate ? *(const float4*)(c + i) : make_float4(0.f, 0.f, 0.f, 0.f);
   for (int s = 0; s < n_chunks; ++s) {
     const float4 v = *(const float4*)(part + (int64_t)s * total + i);
@@ -441,26 +561,40 @@ SpectralPlan spectral_plan(int B, int K, int Mc, int N) {
 }  // namespace
 
 bool fa_spectral_mfma_ok(int a_dtype, int K, int Mc, int N) {
-  return (a_dtype == FA_BF16 || a_dtype == FA_FP16) && N % 8 == 0 && Mc % 2 == 0 && K >= 4 * fa_mfma::kStepTokens;
+  return (a_dtype == FA_BF16 || a_dtype == FA_FP16) && N % 8 == 0 && K >= 4 * fa_mfma::kStepTokens;
 }
 
 size_t fa_spectral_mfma_workspace(int B, int K, int Mc, int N) { return spectral_plan(B, K, Mc, N).total; }
+
+namespace {
+// table, GEMM and chunk reduction on fragments that are already in the workspace
+int spectral_after_pack(const SpectralPlan& pl, float* c, int B, int Mc, int N, int T, int64_t k_start, int accumulate,
+                        void* workspace, hipStream_t st);
+}  // namespace
 
 int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_rs, const int32_t* cols, float* c, int B,
                             int K, int Mc, int N, int T, int64_t k_start, int accumulate, void* workspace,
                             hipStream_t st) {
   using namespace fa_mfma;
   const SpectralPlan pl = spectral_plan(B, K, Mc, N);
-  char* ws = (char*)workspace;
-  half8* tab = (half8*)(ws + pl.off_tab);
-  half8* packed = (half8*)(ws + pl.off_packed);
-  float* part = (float*)(ws + pl.off_part);
-  spectral_table_kernel<<<fa_cdiv((N / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, N, T);
+  half8* packed = (half8*)((char*)workspace + pl.off_packed);
   dim3 pgrid(pl.KS32, fa_cdiv(Mc, 256), B);
   if (a_dtype == FA_BF16)
     spectral_pack_kernel<bf16_t><<<pgrid, 256, 0, st>>>((const bf16_t*)a, a_bs, a_rs, cols, nullptr, packed, K, Mc, pl.CT, pl.KS32);
   else
     spectral_pack_kernel<f16_t><<<pgrid, 256, 0, st>>>((const f16_t*)a, a_bs, a_rs, cols, nullptr, packed, K, Mc, pl.CT, pl.KS32);
+  return spectral_after_pack(pl, c, B, Mc, N, T, k_start, accumulate, workspace, st);
+}
+
+namespace {
+int spectral_after_pack(const SpectralPlan& pl, float* c, int B, int Mc, int N, int T, int64_t k_start, int accumulate,
+                        void* workspace, hipStream_t st) {
+  using namespace fa_mfma;
+  char* ws = (char*)workspace;
+  half8* tab = (half8*)(ws + pl.off_tab);
+  half8* packed = (half8*)(ws + pl.off_packed);
+  float* part = (float*)(ws + pl.off_part);
+  spectral_table_kernel<<<fa_cdiv((N / 8) * kStepK * 64, 256), 256, 0, st>>>(tab, N, T);
   SpectralGemmParams gp{};
   const bool direct = pl.n_chunks == 1;   // nothing to sum: the GEMM writes (or adds to) c itself
   gp.tab = tab; gp.packed = packed; gp.part = direct ? c : part;
@@ -473,6 +607,79 @@ int fa_spectral_mfma_launch(const void* a, int a_dtype, int64_t a_bs, int64_t a_
   const int64_t total = (int64_t)B * 2 * N * Mc;
   if (!direct) spectral_reduce_kernel<<<fa_cdiv(total / 4, 256), 256, 0, st>>>(part, c, total, pl.n_chunks, accumulate);
   return fa_check_launch("fa_mat_fourier");
+}
+
+struct PrefillPlan {
+  SpectralPlan sp;
+  int n_pages, n_blocks;
+  size_t off_sum, off_max, off_min, total;
+};
+PrefillPlan prefill_plan(int B, int L, int K_fft, int Mc, int N) {
+  PrefillPlan p{};
+  p.sp = spectral_plan(B, K_fft, Mc, N);
+  const int pages_of_rows = fa_cdiv(L, 32);
+  p.n_pages = pages_of_rows > p.sp.KS32 ? pages_of_rows : p.sp.KS32;
+  p.n_blocks = fa_cdiv(p.n_pages, fa_mfma::kPackPages);
+  size_t o = p.sp.total;
+  auto take = [&](size_t bytes) { size_t at = o; o += fa_align_up(bytes, 256); return at; };
+  p.off_sum = take((size_t)B * p.n_blocks * Mc * 4);
+  p.off_max = take((size_t)B * p.n_blocks * Mc * 4);
+  p.off_min = take((size_t)B * p.n_blocks * Mc * 4);
+  p.total = o;
+  return p;
+}
+}  // namespace
+
+extern "C" int fa_prefill_compress_ok(int dtype, int L, int K_fft, int Mc, int N, int D) {
+  return fa_spectral_mfma_ok(dtype, K_fft, Mc, N) && L >= K_fft && K_fft > 0 && D % 8 == 0 && D <= 256;
+}
+
+extern "C" size_t fa_prefill_compress_workspace_bytes(int B, int L, int K_fft, int Mc, int N) {
+  if (B <= 0 || L <= 0 || K_fft <= 0 || Mc <= 0 || N <= 0) return 0;
+  return prefill_plan(B, L, K_fft, Mc, N).total;
+}
+
+extern "C" int fa_prefill_compress(const void* src, int dtype, int64_t src_bs, int64_t src_rs, int64_t row0, int L, int K_fft,
+                                   void* store, int64_t st_bs, int cap_pages, const int32_t* n_list, const int32_t* n_h,
+                                   const int32_t* pad_h, const int32_t* c_list, const int32_t* c_h, int Mc, float* coef,
+                                   float* avg, float* max_dev, int stats_round_dtype, int B, int Hkv, int D, int N, int T,
+                                   int is_v, void* workspace, size_t workspace_bytes, fa_stream_t stream) {
+  using namespace fa_mfma;
+  FA_REQUIRE(src && store && n_h && pad_h && c_list && c_h && coef && avg && max_dev, FA_ERR_NULL_POINTER,
+             "fa_prefill_compress: null pointer");
+  FA_REQUIRE(B > 0 && Hkv > 0 && L > 0 && cap_pages > 0 && row0 >= 0 && T > 0, FA_ERR_BAD_SHAPE, "fa_prefill_compress: bad shape");
+  FA_REQUIRE((int64_t)cap_pages * 32 >= L, FA_ERR_BAD_SHAPE, "fa_prefill_compress: %d rows do not fit %d pages", L, cap_pages);
+  FA_REQUIRE(fa_prefill_compress_ok(dtype, L, K_fft, Mc, N, D), FA_ERR_UNSUPPORTED,
+             "fa_prefill_compress: dtype=%d L=%d K=%d Mc=%d N=%d D=%d is for the separate calls", dtype, L, K_fft, Mc, N, D);
+  FA_REQUIRE(src_rs >= (int64_t)Hkv * D && src_rs % 8 == 0 && src_bs % 8 == 0 && ((uintptr_t)src & 15) == 0,
+             FA_ERR_MISALIGNED, "fa_prefill_compress: rows of %lld elements (need %d, 16-byte aligned)", (long long)src_rs, Hkv * D);
+  const PrefillPlan pl = prefill_plan(B, L, K_fft, Mc, N);
+  FA_REQUIRE(workspace && workspace_bytes >= pl.total, FA_ERR_WORKSPACE, "fa_prefill_compress: workspace %zu < %zu",
+             workspace_bytes, pl.total);
+  FA_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)coef & 15) == 0, FA_ERR_MISALIGNED,
+             "fa_prefill_compress: workspace not 256-byte or coefficients not 16-byte aligned");
+  hipStream_t st = fa_hip_stream(stream);
+  char* ws = (char*)workspace;
+  float* psum = (float*)(ws + pl.off_sum);
+  float* pmax = (float*)(ws + pl.off_max);
+  float* pmin = (float*)(ws + pl.off_min);
+  auto launch = [&](auto tag) {
+    using E = decltype(tag);
+    PrefillPackParams<E> pp{};
+    pp.src = (const E*)src; pp.src_bs = src_bs; pp.src_rs = src_rs; pp.row0 = row0; pp.L = L; pp.K_fft = K_fft;
+    pp.store = (E*)store; pp.st_bs = st_bs; pp.cap_pages = cap_pages;
+    pp.n_list = n_list; pp.n_h = n_h; pp.pad_h = pad_h; pp.c_list = c_list; pp.c_h = c_h;
+    pp.packed = (half8*)(ws + pl.sp.off_packed);
+    pp.psum = psum; pp.pmax = pmax; pp.pmin = pmin;
+    pp.Mc = Mc; pp.CT = pl.sp.CT; pp.KS32 = pl.sp.KS32; pp.n_pages = pl.n_pages; pp.n_blocks = pl.n_blocks;
+    pp.Hkv = Hkv; pp.D = D; pp.is_v = is_v;
+    prefill_pack_kernel<E><<<dim3(pl.n_blocks, Hkv, B), 256, 0, st>>>(pp);
+  };
+  if (dtype == FA_BF16) launch(bf16_t{}); else launch(f16_t{});
+  int rc = spectral_after_pack(pl.sp, coef, B, Mc, N, T, 0, 0, workspace, st);
+  if (rc != FA_OK) return rc;
+  fa_stats_finalize_launch(psum, pmax, pmin, avg, max_dev, B, L, Mc, pl.n_blocks, stats_round_dtype, st);
+  return fa_check_launch("fa_prefill_compress");
 }
 
 namespace {

@@ -57,6 +57,34 @@ class MidStore:
                                       int(self.is_v), _lib.FA_COLS_HEAD_DIMS if head_dims else _lib.FA_COLS_ANY,
                                       _stream(self.device)))
 
+    def pack_and_compress(self, src: torch.Tensor, row0: int, rows: int, fft_rows: int, c_list32: torch.Tensor,
+                          c_h32: torch.Tensor, n_freq: int, period: int, round_dtype: torch.dtype):
+        """``pack(src, row0, rows, head_dims=True)`` together with, for the compressed dims ``c_list32`` (flat
+        ``h*D + d`` entries with per-head offsets ``c_h32``) of the same rows, ``ops.mat_fourier(..., K=fft_rows)``
+        and ``ops.mat_avg_std``: one read of the rows (cache_utils_fourier.py:560-565, 578-587).  Returns
+        ``(coef, avg, max_dev)``, or ``None`` with nothing written when the shape is for the separate calls."""
+        from .ops import workspace
+        lib = _lib.load()
+        Mc = int(c_list32.numel())
+        if (src.dim() != 3 or src.stride(2) != 1 or src.dtype != self.dtype or src.shape[2] != self.Hkv * self.D
+                or self.Cn == 0 or Mc == 0 or rows > self.cap_tokens or src.data_ptr() % 16 or src.stride(0) % 8
+                or src.stride(1) % 8
+                or not lib.fa_prefill_compress_ok(dtype_code(src.dtype), int(rows), int(fft_rows), Mc, int(n_freq), self.D)):
+            return None
+        B = self.B
+        coef = torch.empty((B, 2 * n_freq, Mc), device=self.device, dtype=torch.float32)
+        avg = torch.empty((B, Mc), device=self.device, dtype=torch.float32)
+        dev = torch.empty((B, Mc), device=self.device, dtype=torch.float32)
+        nbytes = int(lib.fa_prefill_compress_workspace_bytes(B, int(rows), int(fft_rows), Mc, int(n_freq)))
+        ws = workspace(self.device, nbytes, "spectral")
+        check(lib.fa_prefill_compress(src.data_ptr(), dtype_code(src.dtype), src.stride(0), src.stride(1), int(row0), int(rows),
+                                      int(fft_rows), self.data.data_ptr(), self.batch_stride, self.cap_pages,
+                                      self.n_list32.data_ptr(), self.n_h32.data_ptr(), self.pad_h32.data_ptr(),
+                                      c_list32.data_ptr(), c_h32.data_ptr(), Mc, coef.data_ptr(), avg.data_ptr(),
+                                      dev.data_ptr(), dtype_code(round_dtype), B, self.Hkv, self.D, int(n_freq), int(period),
+                                      int(self.is_v), ws.data_ptr(), ws.numel(), _stream(self.device)))
+        return coef, avg, dev
+
     def append(self, row: torch.Tensor, pos: int) -> None:
         """Store ``row[:, n_list]`` (``row (B, width)`` view) at token position ``pos``."""
         assert row.dim() == 2 and row.stride(1) == 1 and row.dtype == self.dtype

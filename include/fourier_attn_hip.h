@@ -262,6 +262,24 @@ int fa_mid_pack(const void* src, int dtype, int64_t src_batch_stride, int64_t sr
                 const int32_t* n_h_list, const int32_t* pad_h_list, int B, int Hkv, int D, int is_v,
                 int cols_kind, fa_stream_t stream);
 
+/* The prompt's mid rows of K (or V) in one pass: what the cache's prefill does with them in CACHE:560-565 (K) and
+ * CACHE:578-587 (V) -- keep the stored dims (fa_mid_pack with FA_COLS_HEAD_DIMS), transform the first K_fft rows of
+ * the compressed dims (fa_mat_fourier with k_start 0) and take the compressed dims' column statistics over all L rows
+ * (fa_mat_avg_std).  The rows [row0, row0 + L) of src (B, S, Hkv*D) are read once.  pages and coefficients equal
+ * those of the separate calls bit for bit; the statistics sum in another order (equal to rounding).
+ * c_list / c_h_list: the compressed dims as flat h*D + d entries, head by head, and their per-head offsets
+ * (Hkv + 1 entries), Mc = c_h_list[Hkv]; coef (B, 2N, Mc), avg and max_dev (B, Mc) fp32.
+ * Supported (fa_prefill_compress_ok) for 16-bit rows whose transform runs on the matrix cores, K_fft <= L, D a
+ * multiple of 8 up to 256; FA_ERR_UNSUPPORTED otherwise, and the caller makes the three calls. */
+int fa_prefill_compress_ok(int dtype, int L, int K_fft, int Mc, int N, int D);
+size_t fa_prefill_compress_workspace_bytes(int B, int L, int K_fft, int Mc, int N);
+int fa_prefill_compress(const void* src, int dtype, int64_t src_batch_stride, int64_t src_row_stride, int64_t row0,
+                        int L, int K_fft, void* store, int64_t store_batch_stride, int cap_pages,
+                        const int32_t* n_list, const int32_t* n_h_list, const int32_t* pad_h_list,
+                        const int32_t* c_list, const int32_t* c_h_list, int Mc, float* coef, float* avg,
+                        float* max_dev, int stats_round_dtype, int B, int Hkv, int D, int N, int T, int is_v,
+                        void* workspace, size_t workspace_bytes, fa_stream_t stream);
+
 /* Write one row (the evicted window row, CACHE:735, 741) at token position pos. */
 int fa_mid_append(const void* row, int dtype, int64_t row_batch_stride, int64_t pos, void* store,
                   int64_t store_batch_stride, int cap_pages, const int32_t* n_list, const int32_t* n_h_list,

@@ -266,3 +266,45 @@ def test_one_full_length_sequence_against_the_oracle(mask, dtype, Hq, S, states,
     got = gpu.decode_attention(H.to_gpu(q, dtype), 0, Hq, Hkv).cpu().numpy()
     err = np.abs(got - want).max()
     assert err <= 2e-2 and err <= 1e-3, err              # stated bound, and what fp32 accumulation really leaves
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,B,Hkv,D,W,M,prompt,t_c,kcounts,vcounts", [
+    (torch.bfloat16, 2, 2, 128, 32, 64, 1000, 4096, [64, 40], [64, 96]),        # ragged heads, rows not a page multiple
+    (torch.float16, 1, 4, 64, 16, 32, 700, 4096, [0, 64, 30, 2], [64, 0, 10, 32]),   # heads with nothing compressed / stored
+    (torch.bfloat16, 3, 2, 128, 32, 64, 2500, 1024, [100, 128], [128, 6]),      # transform over the first 1024 rows only
+    (torch.bfloat16, 1, 8, 128, 64, 256, 5000, 1 << 17, [64] * 8, [64] * 8),   # several chunks of the transform
+    (torch.bfloat16, 2, 8, 128, 64, 128, 3000, 1 << 17, [83, 116, 117, 96, 122, 88, 116, 81],
+     [120, 128, 110, 111, 8, 122, 128, 92]),                                   # head counts of a searched mask: odd totals
+])
+def test_prefill_in_one_pass_matches_the_separate_calls(dtype, B, Hkv, D, W, M, prompt, t_c, kcounts, vcounts):
+    """The cache's prefill reads the prompt's mid rows once for pages, coefficients and column statistics
+    (``fa_prefill_compress``); the same cache with ``fuse_prefill`` off makes the three calls.  Pages and coefficients
+    must agree bit for bit (same fragments into the same product), the statistics to fp32 rounding of a sum taken
+    in another order (they are then rounded to the model dtype: one unit there at most)."""
+    from fourierattention_amd import DynamicCache
+    masks = _masks(1, Hkv, D, kcounts, vcounts, seed=5)
+    cfg = _cfg(masks, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=16, max_position_embeddings=t_c)
+    r = np.random.default_rng(11)
+    k = H.to_gpu(H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)) + 0.3, dtype), dtype)
+    v = H.to_gpu(H.to_dtype_np(r.standard_normal((B, Hkv, prompt, D)) * 2.0, dtype), dtype)
+    one, three = DynamicCache(cfg), DynamicCache(cfg)
+    three.fuse_prefill = False
+    one.update(k, v, 0)
+    three.update(k, v, 0)
+    from fourierattention_amd import _lib
+    L = prompt - 4 - W
+    for tag in ("k", "v"):
+        a, b = getattr(one._layers[0], tag), getattr(three._layers[0], tag)
+        mc = a.coef.shape[2]
+        fused_ran = bool(a.mid.Cn and mc and _lib.load().fa_prefill_compress_ok(
+            _lib.FA_FP16 if dtype == torch.float16 else _lib.FA_BF16, L, min(L, one._book.t_c), mc, M // 2, D))
+        assert fused_ran == (mc > 0 and a.mid.Cn > 0), (tag, mc)
+        assert torch.equal(a.mid.data, b.mid.data), tag
+        assert torch.equal(a.coef, b.coef), tag
+        assert torch.equal(a.il, b.il), tag
+        eps = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        for x, y in zip(a.stats32, b.stats32):
+            assert x.shape == y.shape
+            if x.numel():
+                assert ((x - y).abs() <= 2 * eps * y.abs() + 1e-6).all(), (tag, (x - y).abs().max().item())

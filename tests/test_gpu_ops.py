@@ -174,6 +174,8 @@ def test_decode_attention_window_only_and_errors():
     (2, 1500, 96, 40, 1501, 0, True),       # ragged everything: last step partly empty, 5 row tiles, 6 column tiles
     (1, 4096, 512, 128, 4096, 0, True),     # whole tiles, several chunks
     (1, 700, 30, 8, 9000, 12345, False),    # phase offset, fewer columns than one workgroup tile
+    (2, 1100, 819, 16, 1100, 0, True),      # an odd number of columns (what a searched mask gives), last tile ragged
+    (1, 600, 33, 24, 777, 5, False),        # odd again, rows of the result not 16-byte aligned
 ])
 def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
     """Long 16-bit inputs take the matrix-core kernels (basis in fp16, fp32 accumulation): checked against the
@@ -187,6 +189,8 @@ def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
     xs = x[:, :, cols] if gather else x
     xg = H.to_gpu(x, dtype)
     cg = torch.from_numpy(cols).int().cuda() if gather else None
+    from fourierattention_amd import _lib
+    assert _lib.load().fa_mat_fourier_workspace_bytes(ops.dtype_code(dtype), B, K, Mc, N) > 0   # the shape is for the matrix cores
     got = ops.mat_fourier(xg, N, T, k0, cols=cg)
     ref = ops.mat_fourier(xg, N, T, k0, cols=cg, matrix_cores=False)
     assert rel_err(got.cpu().numpy(), ref.cpu().numpy()) <= 5e-4
@@ -205,6 +209,7 @@ def test_mat_fourier_matrix_cores(dtype, B, K, Mc, N, T, k0, gather):
     (1, 1100, 16, 200, 5000),    # nothing beyond T / 2
     (1, 1202, 16, 64, 1201),     # one position more than the period: position T is the image of position 0
     (1, 1300, 16, 64, 1201),     # longer than the period: every position is computed directly
+    (2, 1400, 819, 32, 1500),    # an odd number of columns
 ])
 def test_stats_reconstructed_matrix_cores(B, L, C, N, T):
     """Long reconstructions take the matrix-core kernel (fp16 basis and per-column scaled fp16 coefficients, fp32
