@@ -766,6 +766,317 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// merge after the matrix-core mid rows: the same result as decode_merge_kernel, cut along the coefficient rows.
+// Block (z, KV head, b) of 256 threads owns 64 frequencies = 128 coefficient rows: it folds the g partials of every
+// split for those rows (each read by exactly one block), multiplies them with its 128 rows of the V coefficients
+// (each read by exactly one block) and leaves the contribution to every compressed dim of the head in part_c.  It
+// also folds, for its share of the head's dims, the sink/window partial outputs (stage_il, by dim) and the
+// stored-dim partial outputs of the mid rows (stage_on, by position in the head's list).  The block that finishes
+// last for a (b, KV head) - a counter tells, cleared by the mid-row kernel in front - adds the row blocks up in a
+// fixed order, applies the column statistics, normalises and writes the G output rows.
+// Every load of the first phases is requested before the first barrier.
+// ---------------------------------------------------------------------------
+constexpr int kMrTiles = 8;               // g tiles of 8 frequencies per block
+constexpr int kMrRows = kMrTiles * 16;    // coefficient rows per block (cos and sin of 64 frequencies)
+constexpr int kMrGPre = 8;                // g partials (16 bytes each) a thread requests ahead
+constexpr int kMrVPre = 32;               // V-coefficient values a thread requests ahead
+constexpr int kMrSub = 4;                 // lanes that share one (query head, dim) of the staged sums
+constexpr int kMrIlPre = 6, kMrOnPre = 4; // sink/window and mid partial outputs requested ahead per lane
+
+// What the blocks of one launch hand to the block that finishes last goes through device-scope accesses: stores that
+// write through to memory, loads that do not stop at a cache another block's data has never been in.  The stores of a
+// block have completed when it counts itself (the barrier in front of the count waits for them), and the last block
+// loads after it has seen the count, so no cache write-back or invalidate is needed around the counter.
+__device__ __forceinline__ void st_device(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_device(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+struct MergeRowsArgs {
+  const float* il_m; const float* il_d; const float* il_o; int n_il_split;
+  const float* md_m; const float* md_d; const float* md_g; const float* md_on; int n_mid_stride;
+  const float* v_mc; const float* avg_u; const float* avg_d; const float* scale;
+  const int32_t* vc_list; const int32_t* vc_h; const int32_t* vn_list; const int32_t* vn_h;
+  float* out; void* out_cast; int cast_dtype;
+  float* part_c;      // [B][Hkv][row blocks][G][128]
+  float* stage_il;    // [B][Hq][D]
+  float* stage_on;    // [B][Hq][D]
+  unsigned* count;    // [B][Hkv]
+  int Hq, Hkv, D, N, Cv, nbpg;
+  fa_mfma::SplitTable st;
+};
+
+__global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsArgs a) {
+  extern __shared__ float smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int z = blockIdx.x, R = gridDim.x, h = blockIdx.y, b = blockIdx.z;
+  const int G = a.Hq / a.Hkv, D = a.D, N = a.N, Hkv = a.Hkv;
+  const int n_il = a.n_il_split, n_mid = min(a.st.n[h], a.n_mid_stride), n_all = n_il + n_mid;
+  const int64_t r0 = (int64_t)b * a.Hq + h * G;
+  float* s_w = smem;                        // [G][n_all]
+  float* s_d = s_w + G * n_all;             // [G][n_all]
+  float* s_sc = s_d + G * n_all;            // [2][kGMax]
+  float* s_g = s_sc + 2 * kGMax;            // [G][128]: cos rows of the block's 64 frequencies, then sin rows
+  float* s_x = s_g + G * kMrRows;           // max(1024, 256 * G): g per split class, then the row classes of the product
+  float* s_o = s_x + (256 * G > 1024 ? 256 * G : 1024);   // [G][D], last block
+  __shared__ int s_last;
+
+  // ---- requests: first those whose addresses do not wait for the head's entries of the index lists ------------
+  float m_raw = -INFINITY, d_raw = 0.f;
+  if (tid < G * n_all) {
+    const int g = tid / n_all, s_ = tid - g * n_all;
+    const bool il = s_ < n_il;
+    m_raw = il ? a.il_m[(r0 + g) * n_il + s_] : a.md_m[(r0 + g) * a.n_mid_stride + (s_ - n_il)];
+    d_raw = il ? a.il_d[(r0 + g) * n_il + s_] : a.md_d[(r0 + g) * a.n_mid_stride + (s_ - n_il)];
+  }
+  // g partials: item = (tile, query head, pair of frequencies) = 16 bytes {cos f, sin f, cos f+1, sin f+1};
+  // consecutive items walk through the 64 G contiguous bytes this (b, KV head) owns in a tile
+  const int n_items = kMrTiles * G * 4;                  // <= 256 (G <= kGMax)
+  const int n_cls = 256 / n_items;                       // split classes
+  const int item = tid % n_items, cls = tid / n_items;
+  const bool g_on = cls < n_cls;
+  const int64_t g_split_stride = (int64_t)16 * 2 * N;
+  const int it_g = (item >> 2) % G, it_t = item / (4 * G), it_q = item & 3;
+  const float* gp;
+  {
+    const int grp = b / a.nbpg, lc = (b - grp * a.nbpg) * G + it_g;
+    gp = a.md_g + (int64_t)(grp * Hkv + h) * a.n_mid_stride * g_split_stride + (int64_t)(z * kMrTiles + it_t) * 256 +
+         (lc * 4 + it_q) * 4;
+  }
+  float4 g_pre[kMrGPre];
+  if (g_on) {
+#pragma unroll
+    for (int u = 0; u < kMrGPre; ++u) g_pre[u] = *(const float4*)(gp + (int64_t)min(cls + u * n_cls, n_mid - 1) * g_split_stride);
+  }
+  const int dsh = (D + R - 1) / R, d_lo = min(D, z * dsh), d_n = min(D, d_lo + dsh) - d_lo;   // this block's dims
+  const int sub = tid & (kMrSub - 1), sit = tid / kMrSub;   // 64 (head, dim) items at a time
+  float il_pre[kMrIlPre], on_pre[kMrOnPre];
+  const bool il_on = n_il > 0 && sit < G * d_n;
+  if (il_on) {
+    const int g = sit / d_n, d = d_lo + (sit - g * d_n);
+#pragma unroll
+    for (int u = 0; u < kMrIlPre; ++u) il_pre[u] = a.il_o[((r0 + g) * n_il + min(sub + u * kMrSub, n_il - 1)) * D + d];
+  }
+  const int vc0 = a.vc_h[h], vc_len = a.vc_h[h + 1] - vc0;
+  const int vn0 = a.vn_h[h], vn_len = a.vn_h[h + 1] - vn0;
+  int cwp = 2;                              // power of two >= vc_len: threads = (dim, row class)
+  while (cwp < vc_len) cwp <<= 1;
+  const int parts = 256 / cwp;              // vc_len <= D <= 128: at least two row classes
+  const bool has_coef = vc_len > 0;
+  // V coefficients: local row rr < 64 is the cos row of frequency 64 z + rr, rr >= 64 the sin row of 64 z + rr - 64
+  const int j = tid & (cwp - 1), part = tid / cwp;
+  const int rows_per_thread = kMrRows / parts;           // parts divides 128
+  auto v_row = [&](int rr) { return rr < 64 ? 64 * z + rr : N + 64 * z + (rr - 64); };
+  const float* vp = a.v_mc + (int64_t)b * 2 * N * a.Cv + vc0 + j;
+  const bool v_on = has_coef && j < vc_len;
+  float v_pre[kMrVPre];
+  if (v_on) {
+#pragma unroll
+    for (int u = 0; u < kMrVPre; ++u) v_pre[u] = vp[(int64_t)v_row(min(part + u * parts, kMrRows - 1)) * a.Cv];
+  }
+  // this block's share of the stored positions of the mid rows
+  const int nsh = (vn_len + R - 1) / R, n_lo = min(vn_len, z * nsh), n_n = min(vn_len, n_lo + nsh) - n_lo;
+  const bool on_on = sit < G * n_n;
+  if (on_on) {
+    const int g = sit / n_n, jj = n_lo + (sit - g * n_n);
+#pragma unroll
+    for (int u = 0; u < kMrOnPre; ++u) on_pre[u] = a.md_on[((r0 + g) * a.n_mid_stride + min(sub + u * kMrSub, n_mid - 1)) * D + jj];
+  }
+
+  // ---- split weights: one wave per query head -----------------------------------------------------------
+  for (int idx = tid; idx < G * n_all; idx += 256) {
+    if (idx == tid) {
+      s_w[idx] = m_raw;
+      s_d[idx] = d_raw;
+    } else {
+      const int g = idx / n_all, s_ = idx - g * n_all;
+      const bool il = s_ < n_il;
+      s_w[idx] = il ? a.il_m[(r0 + g) * n_il + s_] : a.md_m[(r0 + g) * a.n_mid_stride + (s_ - n_il)];
+      s_d[idx] = il ? a.il_d[(r0 + g) * n_il + s_] : a.md_d[(r0 + g) * a.n_mid_stride + (s_ - n_il)];
+    }
+  }
+  __syncthreads();
+  for (int g = wv; g < G; g += 4) {
+    float mstar = -INFINITY;
+    for (int s_ = lane; s_ < n_all; s_ += 64) mstar = fmaxf(mstar, s_w[g * n_all + s_]);
+    mstar = fa_wave_max(mstar);
+    float dsum = 0.f, pmid = 0.f;
+    for (int s_ = lane; s_ < n_all; s_ += 64) {
+      const float m = s_w[g * n_all + s_];
+      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+      s_w[g * n_all + s_] = wgt;
+      if (s_ < n_il) dsum += wgt * s_d[g * n_all + s_]; else pmid += wgt * s_d[g * n_all + s_];
+    }
+    dsum = fa_wave_sum(dsum);
+    pmid = fa_wave_sum(pmid);
+    if (lane == 0) {
+      s_sc[g] = dsum + pmid;
+      s_sc[kGMax + g] = pmid;
+    }
+  }
+  __syncthreads();
+
+  // ---- g of the block's rows, summed over the splits ------------------------------------------------------
+  if (has_coef) {
+    if (g_on) {
+      const float* wg = s_w + it_g * n_all + n_il;
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      auto fold = [&](const float4& v, int sp) {
+        if (sp < n_mid) {
+          const float wt = wg[sp];
+          acc.x = fmaf(wt, v.x, acc.x); acc.y = fmaf(wt, v.y, acc.y);
+          acc.z = fmaf(wt, v.z, acc.z); acc.w = fmaf(wt, v.w, acc.w);
+        }
+      };
+#pragma unroll
+      for (int u = 0; u < kMrGPre; ++u) fold(g_pre[u], cls + u * n_cls);
+      for (int u0 = kMrGPre; cls + u0 * n_cls < n_mid; u0 += 4) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = *(const float4*)(gp + (int64_t)min(cls + (u0 + u) * n_cls, n_mid - 1) * g_split_stride);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) fold(v[u], cls + (u0 + u) * n_cls);
+      }
+      *(float4*)(s_x + (cls * n_items + item) * 4) = acc;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n_items * 4; idx += 256) {
+      float v = 0.f;
+      for (int c = 0; c < n_cls; ++c) v += s_x[c * n_items * 4 + idx];
+      const int it = idx >> 2, e = idx & 3;          // e: cos f, sin f, cos f + 1, sin f + 1 with f = 8 tile + 2 pair
+      const int g = (it >> 2) % G, t = it / (4 * G), q = it & 3;
+      s_g[g * kMrRows + (e & 1) * 64 + t * 8 + 2 * q + (e >> 1)] = v;
+    }
+    __syncthreads();
+    // ---- times the block's rows of the V coefficients
+    float acc[kGMax];
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
+    if (v_on) {
+#pragma unroll
+      for (int u = 0; u < kMrVPre; ++u) {
+        const int rr = part + u * parts;
+        if (u < rows_per_thread) {
+#pragma unroll
+          for (int g = 0; g < kGMax; ++g)
+            if (g < G) acc[g] = fmaf(s_g[g * kMrRows + rr], v_pre[u], acc[g]);
+        }
+      }
+      for (int u0 = kMrVPre; u0 < rows_per_thread; u0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = vp[(int64_t)v_row(min(part + (u0 + u) * parts, kMrRows - 1)) * a.Cv];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+          if (u0 + u < rows_per_thread) {
+#pragma unroll
+            for (int g = 0; g < kGMax; ++g)
+              if (g < G) acc[g] = fmaf(s_g[g * kMrRows + part + (u0 + u) * parts], v[u], acc[g]);
+          }
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < kGMax; ++g)
+      if (g < G) s_x[(part * G + g) * cwp + j] = acc[g];
+    __syncthreads();
+    float* pc = a.part_c + (((int64_t)b * Hkv + h) * R + z) * G * 128;
+    for (int idx = tid; idx < G * cwp; idx += 256) {
+      const int g = idx / cwp, jj = idx - g * cwp;
+      if (jj < vc_len) {
+        float v = 0.f;
+        for (int pp = 0; pp < parts; ++pp) v += s_x[(pp * G + g) * cwp + jj];
+        st_device(pc + g * 128 + jj, v);
+      }
+    }
+  }
+  // ---- staged sums of this block's share of the dims --------------------------------------------------
+  for (int it0 = 0; it0 < G * d_n && n_il > 0; it0 += 256 / kMrSub) {
+    const int it = it0 + sit;
+    float v = 0.f;
+    if (it < G * d_n) {
+      const int g = it / d_n, d = d_lo + (it - g * d_n);
+      const float* wg = s_w + g * n_all;
+      const float* src = a.il_o + (r0 + g) * n_il * D + d;
+      int u0 = 0;
+      if (it0 == 0) {
+#pragma unroll
+        for (int u = 0; u < kMrIlPre; ++u)
+          if (sub + u * kMrSub < n_il) v = fmaf(wg[sub + u * kMrSub], il_pre[u], v);
+        u0 = kMrIlPre;
+      }
+      for (int sp = sub + u0 * kMrSub; sp < n_il; sp += kMrSub) v = fmaf(wg[sp], src[(int64_t)sp * D], v);
+    }
+    v = fa_group_sum<kMrSub>(v);
+    if (it < G * d_n && sub == 0) {
+      const int g = it / d_n, d = d_lo + (it - g * d_n);
+      st_device(a.stage_il + (r0 + g) * D + d, v);
+    }
+  }
+  for (int it0 = 0; it0 < G * n_n; it0 += 256 / kMrSub) {
+    const int it = it0 + sit;
+    float v = 0.f;
+    if (it < G * n_n) {
+      const int g = it / n_n, jj = n_lo + (it - g * n_n);
+      const float* wg = s_w + g * n_all + n_il;
+      const float* src = a.md_on + (r0 + g) * a.n_mid_stride * D + jj;
+      int u0 = 0;
+      if (it0 == 0) {
+#pragma unroll
+        for (int u = 0; u < kMrOnPre; ++u)
+          if (sub + u * kMrSub < n_mid) v = fmaf(wg[sub + u * kMrSub], on_pre[u], v);
+        u0 = kMrOnPre;
+      }
+      for (int sp = sub + u0 * kMrSub; sp < n_mid; sp += kMrSub) v = fmaf(wg[sp], src[(int64_t)sp * D], v);
+    }
+    v = fa_group_sum<kMrSub>(v);
+    if (it < G * n_n && sub == 0) {
+      const int g = it / n_n, jj = n_lo + (it - g * n_n);
+      st_device(a.stage_on + (r0 + g) * D + jj, v);
+    }
+  }
+
+  // ---- the block that finishes last for this (b, KV head) puts the rows together ----------------------------
+  __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0) expcnt(0) lgkmcnt(0): this thread's stores have been acknowledged
+  __syncthreads();
+  if (tid == 0) s_last = atomicAdd(a.count + (int64_t)b * Hkv + h, 1u) == (unsigned)(R - 1);
+  __syncthreads();
+  if (!s_last) return;
+  for (int idx = tid; idx < G * D; idx += 256) s_o[idx] = n_il > 0 ? ld_device(a.stage_il + r0 * D + idx) : 0.f;
+  __syncthreads();
+  const float* pc0 = a.part_c + ((int64_t)b * Hkv + h) * R * G * 128;
+  for (int idx = tid; idx < G * vc_len; idx += 256) {
+    const int g = idx / vc_len, jj = idx - g * vc_len;
+    float v = 0.f;
+    for (int z0 = 0; z0 < R; z0 += 8) {       // eight loads in flight, added in the order of the row blocks
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] = ld_device(pc0 + ((int64_t)min(z0 + u, R - 1) * G + g) * 128 + jj);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (z0 + u < R) v += t[u];
+    }
+    v /= (float)N;
+    const int64_t o = (int64_t)b * a.Cv + vc0 + jj;
+    const float pmid = s_sc[kGMax + g];
+    s_o[g * D + (a.vc_list[vc0 + jj] - h * D)] += a.scale[o] * (v - a.avg_d[o] * pmid) + a.avg_u[o] * pmid;
+  }
+  for (int idx = tid; idx < G * vn_len; idx += 256) {
+    const int g = idx / vn_len, jj = idx - g * vn_len;
+    s_o[g * D + (a.vn_list[vn0 + jj] - h * D)] += ld_device(a.stage_on + (r0 + g) * D + jj);
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int g = idx / D;
+    const float v = s_o[idx] / s_sc[g];
+    const int64_t at = r0 * D + idx;
+    if (a.out) a.out[at] = v;
+    if (a.out_cast) {
+      if (a.cast_dtype == FA_BF16) ((bf16_t*)a.out_cast)[at] = bf16_t{fa_f32_to_bf16_bits(v)};
+      else if (a.cast_dtype == FA_FP16) ((f16_t*)a.out_cast)[at] = f16_t{(_Float16)v};
+      else ((float*)a.out_cast)[at] = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // sink + local window, vectorised (16-bit storage, head_dim 64 or 128, 16-byte aligned rows):
 // a block takes kIlFastTile rows; LPT = D/8 lanes share one row, each holding 8 dims; every wave
 // issues all of its loads first, then runs an online softmax of its own; the four waves of the
@@ -966,6 +1277,9 @@ struct Plan {
   fa_mfma::SplitTable st;
   int n_merge_chunks;
   size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_scores, total;
+  // merge after the matrix-core mid rows: contributions per block of coefficient rows, staged sums, counters
+  int n_row_blocks;
+  size_t off_pc, off_sil, off_son, off_cnt;
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
@@ -1076,6 +1390,11 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   while (p.n_merge_chunks > 1 && (int64_t)B * Hkv * p.n_merge_chunks > device_cu_count()) p.n_merge_chunks >>= 1;
   // two-pass mid rows (eight frequency slices): the scores of every page travel through memory
   p.off_scores = take(mfma && fa_mfma::table_slices(N) > 4 ? (size_t)p.n_groups * Hkv * fa_cdiv(L_m, 32) * 512 * 4 : 0);
+  p.n_row_blocks = mfma ? N / (kMrTiles * 8) : 0;
+  p.off_pc = take(mfma ? (size_t)B * Hkv * p.n_row_blocks * (Hq / Hkv) * 128 * 4 : 0);
+  p.off_sil = take(mfma ? rows * D * 4 : 0);
+  p.off_son = take(mfma ? rows * D * 4 : 0);
+  p.off_cnt = take(mfma ? (size_t)B * Hkv * 4 : 0);
   p.total = o;
   return p;
 }
@@ -1179,6 +1498,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.rot = (const float2v*)(mp.tabET + NSL * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.scores = (float*)(ws + p.off_scores);
+        mp.merge_count = (unsigned*)(ws + p.off_cnt);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.st = p.st;
         mp.sm_log2e = sm_log2e;
@@ -1233,7 +1553,24 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     }
   }
   if (ev) hipEventRecord(ev[3], st);
-  {
+  // 1024 frequencies: blocks per 128 coefficient rows read every partial once (26 against 35 us at B = 4, 130000 mid
+  // rows, 32 splits); up to 512 frequencies the blocks per share of dims below are as fast or 1 us faster
+  if (p.path == Path::Mfma && p.n_mid_split > 0 && a.N >= 1024) {
+    const int n_all = p.n_il_split + p.n_mid_split;
+    const size_t lds = (2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * kMrRows + (256 * (size_t)G > 1024 ? 256 * (size_t)G : 1024) +
+                        (size_t)G * a.D) * sizeof(float);
+    MergeRowsArgs ma{};
+    ma.il_m = ilm; ma.il_d = ild; ma.il_o = ilo; ma.n_il_split = p.n_il_split;
+    ma.md_m = mm; ma.md_d = md; ma.md_g = mg; ma.md_on = mon; ma.n_mid_stride = p.n_mid_split;
+    ma.v_mc = a.v_mc; ma.avg_u = a.avg_v_u; ma.avg_d = a.avg_v_d; ma.scale = a.scale_v;
+    ma.vc_list = a.vc_list; ma.vc_h = a.vc_h_list; ma.vn_list = a.vn_list; ma.vn_h = a.vn_h_list;
+    ma.out = a.out; ma.out_cast = a.out_cast; ma.cast_dtype = a.dtype;
+    ma.part_c = (float*)(ws + p.off_pc); ma.stage_il = (float*)(ws + p.off_sil); ma.stage_on = (float*)(ws + p.off_son);
+    ma.count = (unsigned*)(ws + p.off_cnt);
+    ma.Hq = a.Hq; ma.Hkv = a.Hkv; ma.D = a.D; ma.N = a.N; ma.Cv = a.Cv; ma.nbpg = p.nbpg;
+    ma.st = p.st;
+    decode_merge_rows_kernel<<<dim3(p.n_row_blocks, a.Hkv, a.B), 256, lds, st>>>(ma);
+  } else {
     const int n_all = p.n_il_split + p.n_mid_split;
     size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 1024 * (size_t)G + (size_t)G * a.D + a.D) * sizeof(float);
     if (lds > 64 * 1024) {

@@ -236,6 +236,7 @@ struct MidParams {
   float* pg;
   float* pon;
   float* scores;   // two-pass mode: [groups][Hkv][pages][16 columns][32 tokens] fp32
+  unsigned* merge_count;   // [B][Hkv] counters of the merge launch behind this one: cleared here
   int B, Hq, Hkv, D, G, nbpg, N, L_m, T;
   int n_split;   // splits the partial buffers have room for per head (the largest n[h])
   float sm_log2e;
@@ -293,6 +294,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const bool valid_r = lc < R;
   const int bb_r = lc / G, g_r = lc - bb_r * G;
   const int64_t qrow = valid_r ? ((int64_t)(b0 + bb_r) * p.Hq + h * G + g_r) : 0;
+  if (MODE != 1 && split == 0 && tid < nb && p.merge_count) p.merge_count[(b0 + tid) * p.Hkv + h] = 0u;
   const int fbase = sl * 16 * KS;
   const bool has_mn = sl < nb && sl < kFreqWaves;
   const int my_b = b0 + (has_mn ? sl : 0);
