@@ -59,11 +59,13 @@ __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ 
     const int lane = idx & 63, s = (idx >> 6) % KS, rb = ((idx >> 6) / KS) & 1, w = (idx >> 6) / (2 * KS);
     const int lg = lane >> 4, lc = lane & 15;
     const int i = rb * 16 + lc;
+    // kstep s = 2j + cs: the cosines (cs = 0) or the sines (cs = 1) of the eight frequencies of the row tiles
+    // 4j .. 4j + 3 that this lane group owns
+    const int j = s >> 1, cs = s & 1;
     half8 out;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int v = e >> 1, cs = e & 1;
-      const int f = w * 16 * KS + freq_of(2 * s + (v >> 1), lg, v & 1);
+      const int f = w * 16 * KS + freq_of(4 * j + (e >> 1), lg, e & 1);
       float sn, co;
       fa_sincos_phase(f, 2 * i + 1, 2 * T, &sn, &co);
       out[e] = (_Float16)(cs ? sn : co);
@@ -464,6 +466,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     };
 
+    // coefficient-domain part of the scores of a frame: C = sum over the cosine ksteps, S = over the sine ksteps.
+    // Computed on the first (mirrored) page of the frame, whose rows are C - S; the second page's are C + S.
+    float4v accC[2], accS[2];
     // one trip of the score pipeline: page `it` of the split (none on the trip after the last page)
     auto score_trip = [&](int it, auto mirrored_tag) {
       constexpr bool mirrored = decltype(mirrored_tag)::value;   // first page of its frame
@@ -495,23 +500,49 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           rot_issue<0>(rot_lane, rc[0]);
           if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
         }
-        float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
-        // The two pages of a frame convert the same W': without this the conversions of the second page are done
-        // together with those of the first and their results held across a whole page.
+        float4v cd[2];   // coefficient-domain part of this page's scores, scaled, with the constant term
+        if constexpr (MODE == 1) {
+          // the score pass has no registers for C and S next to its operands: every page runs the whole product.
+          // The two pages of a frame convert the same W': without the pin the conversions of the second page are
+          // done together with those of the first and their results held across a whole page.
 #pragma unroll
-        for (int rt = 0; rt < 2 * KS; ++rt)
-          asm volatile("" : "+v"(Wc[rt][0]), "+v"(Wc[rt][1]), "+v"(Ws[rt][0]), "+v"(Ws[rt][1]));
+          for (int rt = 0; rt < 2 * KS; ++rt)
+            asm volatile("" : "+v"(Wc[rt][0]), "+v"(Wc[rt][1]), "+v"(Ws[rt][0]), "+v"(Ws[rt][1]));
+          float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          half8 wb;
+          for (int s = 0; s < KS; ++s) {
+            half8 wb;
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const float ws = Ws[2 * s + (v >> 1)][v & 1];
-            wb[2 * v] = (_Float16)Wc[2 * s + (v >> 1)][v & 1];
-            wb[2 * v + 1] = (_Float16)(mirrored ? -ws : ws);   // offsets -(i + 1/2): the sines change sign
+            for (int e = 0; e < 8; ++e) {
+              const float wv = (s & 1) ? Ws[4 * (s >> 1) + (e >> 1)][e & 1] : Wc[4 * (s >> 1) + (e >> 1)][e & 1];
+              wb[e] = (_Float16)((mirrored && (s & 1)) ? -wv : wv);   // offsets -(i + 1/2): the sines change sign
+            }
+            accf[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][s], wb, accf[0], 0, 0, 0);
+            accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
           }
-          accf[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][s], wb, accf[0], 0, 0, 0);
-          accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
+          cd[0] = accf[0] * colscale + c0col;
+          cd[1] = accf[1] * colscale + c0col;
+        } else {
+          if constexpr (mirrored) {
+            accC[0] = accC[1] = accS[0] = accS[1] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < KS / 2; ++j) {
+              half8 wbc, wbs;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                wbc[e] = (_Float16)Wc[4 * j + (e >> 1)][e & 1];
+                wbs[e] = (_Float16)Ws[4 * j + (e >> 1)][e & 1];
+              }
+              accC[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j], wbc, accC[0], 0, 0, 0);
+              accC[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j], wbc, accC[1], 0, 0, 0);
+              accS[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j + 1], wbs, accS[0], 0, 0, 0);
+              accS[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j + 1], wbs, accS[1], 0, 0, 0);
+            }
+          }
+          // offsets -(i + 1/2) on the mirrored page: the sines change sign
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb)
+            cd[rb] = (mirrored ? accC[rb] - accS[rb] : accC[rb] + accS[rb]) * colscale + c0col;
         }
         // behind the second page of a frame: W' moves on to the centre of the next frame
         if constexpr (!mirrored) rot_apply_in_place_from<2 * KS, 0>(rot_lane, rc, Wc, Ws);
@@ -539,7 +570,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int rb = 0; rb < 2; ++rb) {
           float4v o;
 #pragma unroll
-          for (int v = 0; v < 4; ++v) o[v] = accf[rb][v] * colscale + accm[rb][v] * p.sm_log2e + c0col;
+          for (int v = 0; v < 4; ++v) o[v] = cd[rb][v] + accm[rb][v] * p.sm_log2e;
           *(float4v*)&s_part[it & 1][sl][lc * kPart + rb * 16 + 4 * lg] = o;
         }
       } else if (it > 0) {
