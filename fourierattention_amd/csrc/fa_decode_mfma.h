@@ -629,6 +629,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
 
+    // The probabilities of the first (mirrored) page of a frame wait here for the second page: the tokens at the
+    // offsets -(i + 1/2) and +(i + 1/2) meet the same cosine and, with opposite signs, the same sine, so g of the frame
+    // takes E_cos^T (P2 + P1) and E_sin^T (P2 - P1) in one product instead of one per page.
+    half8 p_first;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) p_first[e] = (_Float16)0.f;
     // one page of the value stage (page it - 1 of the split)
     // (whether this wave streams V is fixed for the whole loop: a parameter of the body, not a branch in it)
     auto value_page = [&](int it, auto first_tag, auto stream_tag) {
@@ -744,21 +750,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int rt = 0; rt < 2 * KS; ++rt) hacc[rt] *= alpha;
 #pragma unroll
           for (int f = 0; f < VMAX; ++f) oacc[f] *= alpha;
+          if constexpr (!first_of_frame) p_first *= (_Float16)alpha;   // taken against the reference of a page ago
         }
-#pragma unroll
-        for (int j = 0; j < KS; ++j)
-          hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], pf, hacc[2 * j], 0, 0, 0);
         if constexpr (first_of_frame) {
-          // offsets -(i + 1/2): the sine tiles take -P (the sign bits of the eight halves, flipped in place once
-          // the cosine tiles have been issued)
-          uint4v neg = __builtin_bit_cast(uint4v, pf);
-          asm volatile("" : "+v"(neg));
-          neg ^= uint4v{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
-          pf = __builtin_bit_cast(half8, neg);
-        }
+          p_first = pf;
+        } else {
+          const half8 p_sum = pf + p_first, p_dif = pf - p_first;
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
-          hacc[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j + 1], pf, hacc[2 * j + 1], 0, 0, 0);
+          for (int j = 0; j < KS; ++j)
+            hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], p_sum, hacc[2 * j], 0, 0, 0);
+#pragma unroll
+          for (int j = 0; j < KS; ++j)
+            hacc[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j + 1], p_dif, hacc[2 * j + 1], 0, 0, 0);
+        }
         if constexpr (has_v) {
 #pragma unroll
           for (int f0 = 0; f0 < VMAX; f0 += 4) {
@@ -797,6 +801,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     };
     if (streams_v) value_loop(std::true_type{});
     else value_loop(std::false_type{});
+    if (n_it & 1) {   // the last frame has a first page only: g takes E_cos^T P1 and -E_sin^T P1
+      const half8 p_neg = -p_first;
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+        hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], p_first, hacc[2 * j], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+        hacc[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j + 1], p_neg, hacc[2 * j + 1], 0, 0, 0);
+    }
 
     // ---- partials of this split ------------------------------------------------------
     const float dsum = fa_rows_sum(d_run);
