@@ -14,9 +14,13 @@
 //
 // Frames.  Two pages share one frame whose centre lies half a token before the first token of the second
 // page: its tokens sit at the offsets +(i + 1/2), those of the first page at -(i + 1/2), i = 0 .. 31.  Cosine is
-// even and sine is odd, so ONE constant operand E (offsets i + 1/2) serves both pages: on the first ("mirrored")
-// page the sine rows of W' enter negated and row i of the product is token 31 - i; for g the sine tiles take
-// -P.  W' and the g history are rotated once per frame (64 tokens), not once per page.  On a mirrored page every
+// even and sine is odd, so ONE constant operand E (offsets i + 1/2) serves both pages, and so does one product:
+// with C = E_cos . W'_cos and S = E_sin . W'_sin (cosine and sine ksteps in separate accumulators) the scores of
+// the second page are C + S and those of the first ("mirrored") page C - S, row i being token 31 - i there; g of
+// the frame takes E_cos^T (P2 + P1) and E_sin^T (P2 - P1), P1 / P2 being the probabilities of the first and of
+// the second page.  The coefficient-domain products are thus issued once per frame (the score pass of the two-pass
+// mode, which lacks the registers for C and S, still runs them per page with the sine rows of W' negated on the
+// mirrored page).  W' and the g history are rotated once per frame (64 tokens), not once per page.  On a mirrored page every
 // position-indexed quantity (score partials in LDS, probabilities) is held in the mirrored order; the K and V
 // pages come into LDS through per-lane addresses, so fetching a K fragment with its 16 rows reversed (and the two
 // 16-token blocks exchanged) or a V fragment with its four groups of 8 tokens exchanged costs nothing.
@@ -44,7 +48,8 @@ constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one 
 
 // ---------------------------------------------------------------------------
 // constant operand tables (depend on T and N only); KS = N / (16 * slices) ksteps per frequency slice
-//   tabE  [slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM, row i = offset i + 1/2
+//   tabE  [slices][2 row blocks][KS][64 lanes] x half8 : A operand of the score GEMM, row i = offset i + 1/2; kstep
+//         2j holds the cosines and kstep 2j + 1 the sines of the frequencies of the row tiles 4j .. 4j + 3
 //   tabET [slices][2*KS tiles][64 lanes] x half8 : A operand of the g GEMM; tile 2j holds the cosines and tile
 //         2j + 1 the sines of the 16 frequencies 16j .. 16j + 15 of the slice (row = frequency), columns = the
 //         offsets i + 1/2
@@ -246,11 +251,12 @@ struct MidParams {
 };
 
 // The workgroup is a two-stage pipeline over the pages of its split, one barrier per page:
-//   waves 0-3 ("score waves")  page t+1: S partial = E . W' (their frequency slice) + K_mn . Q_n (their batch
-//                              element) -> LDS; after the second page of a frame, W' moves on to the next frame
+//   waves 0-3 ("score waves")  page t+1: S partial = E . W' (their frequency slice; the product itself on the first
+//                              page of a frame, see above) + K_mn . Q_n (their batch element) -> LDS; after the second
+//                              page of a frame, W' moves on to the next frame
 //   waves 4-7 ("value waves")  page t  : sum the four partials, online softmax, before the first page of a frame
-//                              rotate the g history into it, rescale, g' += E^T . P (their frequency slice),
-//                              o_n += V_mn^T . P (their batch element)
+//                              rotate the g history into it, rescale, on the second page g' += E^T . (P2 +- P1)
+//                              (their frequency slice), on both o_n += V_mn^T . P (their batch element)
 // Pages at an even distance from the first page of the split are the mirrored pages of their frames.
 // Score wave i and value wave i own the same frequencies and stream the same batch element of the group.
 // KS: ksteps (32 coefficient rows) per slice = N / (16 * slices).  KMAX: ksteps of stored K dims a head may have
