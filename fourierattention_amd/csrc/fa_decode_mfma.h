@@ -761,7 +761,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (first_of_frame) {
           p_first = pf;
         } else {
-          const half8 p_sum = pf + p_first, p_dif = pf - p_first;
+          // (the difference as a sum with the sign bits flipped: packed adds, where a subtraction of two vectors of
+          // halves is taken apart into sixteen scalar ones)
+          const uint4v flipped = __builtin_bit_cast(uint4v, p_first) ^ uint4v{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+          const half8 p_sum = pf + p_first, p_dif = pf + __builtin_bit_cast(half8, flipped);
 #pragma unroll
           for (int j = 0; j < KS; ++j)
             hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], p_sum, hacc[2 * j], 0, 0, 0);
@@ -808,7 +811,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (streams_v) value_loop(std::true_type{});
     else value_loop(std::false_type{});
     if (n_it & 1) {   // the last frame has a first page only: g takes E_cos^T P1 and -E_sin^T P1
-      const half8 p_neg = -p_first;
+      const uint4v flipped = __builtin_bit_cast(uint4v, p_first) ^ uint4v{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+      const half8 p_neg = __builtin_bit_cast(half8, flipped);
 #pragma unroll
       for (int j = 0; j < KS; ++j)
         hacc[2 * j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ETa[2 * j], p_first, hacc[2 * j], 0, 0, 0);
