@@ -256,6 +256,26 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_linear_packed(p, 1536, p, p, 1, 1536, 16, 0, None) == -5         # K not a multiple of 1024
     assert lib.fa_linear_packed(p, 1000, p, p, 2, 1024, 16, 0, None) == -7         # rows of x closer than K
     assert lib.fa_linear_packed_ok(16, 4096, 6144) == 1 and lib.fa_linear_packed_ok(0, 4096, 6144) == 0
+    # the one-pass prefill: (src, dtype, bs, rs, row0, L, K_fft, store, st_bs, cap_pages, n_list, n_h, pad_h, c_list, c_h, Mc,
+    #                        coef, avg, dev, round_dtype, B, Hkv, D, N, T, is_v, workspace, bytes, stream)
+    pc = lambda *a: lib.fa_prefill_compress(*a)
+    ok_args = [p, 0, 1 << 20, 1024, 4, 1000, 1000, p, 1 << 20, 40, p, p, p, p, p, 512, p, p, p, 0, 1, 8, 128, 64, 4096, 0, p, 1 << 30, None]
+    names = {n: i for i, n in enumerate("src dtype bs rs row0 L K_fft store st_bs cap n_list n_h pad_h c_list c_h Mc coef avg dev rd B Hkv D N T is_v ws ws_bytes stream".split())}
+    arg = lambda **kw: [kw.get(n, ok_args[i]) for n, i in names.items()]
+    assert pc(*arg(src=None)) == -1
+    assert pc(*arg(L=0)) == -2
+    assert pc(*arg(cap=10)) == -2                                     # 1000 rows do not fit 10 pages
+    assert pc(*arg(dtype=2)) == -5                                    # float32 rows: the separate calls
+    assert pc(*arg(L=100, K_fft=100, cap=40)) == -5                   # too short for the matrix-core transform
+    assert pc(*arg(K_fft=1001)) == -5                                 # more rows into the transform than there are
+    assert pc(*arg(D=130)) == -5
+    assert pc(*arg(rs=1000)) == -7                                    # rows shorter than Hkv * D
+    assert pc(*arg(ws_bytes=1024)) == -4
+    assert b"workspace" in lib.fa_last_error_string()
+    assert lib.fa_prefill_compress_ok(0, 1000, 1000, 819, 64, 128) == 1 and lib.fa_prefill_compress_ok(2, 1000, 1000, 512, 64, 128) == 0
+    need = lib.fa_prefill_compress_workspace_bytes(1, 1000, 1000, 512, 64)
+    assert need > lib.fa_mat_fourier_workspace_bytes(0, 1, 1000, 512, 64) > 0       # + the partials of the column statistics
+    assert lib.fa_mat_fourier_workspace_bytes(0, 1, 1000, 819, 64) > 0               # an odd number of columns is fine
     assert lib.fa_stream_update(None, None) == -1
     sa = _lib.StreamArgs()
     assert lib.fa_stream_update(ctypes.byref(sa), None) == -2                  # empty shape
