@@ -138,20 +138,28 @@ __device__ __forceinline__ void fa_swap32(float x, float* lo, float* hi) {
   *lo = __builtin_bit_cast(float, r0);
   *hi = __builtin_bit_cast(float, r1);
 }
+// Maximum / minimum that hand a NaN on (v_maximum3_f32 / v_minimum3_f32 of gfx950, three operands per instruction).
+// fmaxf / fminf must drop a NaN, for which the compiler first passes every operand that comes out of a matrix
+// instruction or a lane exchange through an instruction of its own: three instructions per maximum instead of one.
+__device__ __forceinline__ float fa_fmax(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float fa_fmin(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+__device__ __forceinline__ float fa_fmax8(const float (&v)[8]) {
+  return fa_fmax(fa_fmax(fa_fmax(fa_fmax(fa_fmax(fa_fmax(fa_fmax(v[0], v[1]), v[2]), v[3]), v[4]), v[5]), v[6]), v[7]);
+}
 // max / sum over the four lanes that share (lane % 16); every lane gets the result
 __device__ __forceinline__ float fa_rows_max(float x) {
   float a, b;
   fa_swap16(x, &a, &b);
-  x = fmaxf(a, b);
+  x = fa_fmax(a, b);
   fa_swap32(x, &a, &b);
-  return fmaxf(a, b);
+  return fa_fmax(a, b);
 }
 __device__ __forceinline__ float fa_rows_min(float x) {
   float a, b;
   fa_swap16(x, &a, &b);
-  x = fminf(a, b);
+  x = fa_fmin(a, b);
   fa_swap32(x, &a, &b);
-  return fminf(a, b);
+  return fa_fmin(a, b);
 }
 __device__ __forceinline__ float fa_rows_sum(float x) {
   float a, b;

@@ -409,7 +409,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (!valid_r) c2 = s2 = float2v{0.f, 0.f};   // lanes of columns past the group hold nothing
         Wc[rt][0] = c2[0]; Wc[rt][1] = c2[1];
         Ws[rt][0] = s2[0]; Ws[rt][1] = s2[1];
-        wmax = fmaxf(wmax, fmaxf(fmaxf(fabsf(c2[0]), fabsf(c2[1])), fmaxf(fabsf(s2[0]), fabsf(s2[1]))));
+        wmax = fa_fmax(fa_fmax(fa_fmax(fa_fmax(wmax, fabsf(c2[0])), fabsf(c2[1])), fabsf(s2[0])), fabsf(s2[1]));
       }
     }
     wmax = fa_rows_max(wmax);
@@ -729,7 +729,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (tok >= p.L_m) sc[e] = -INFINITY;
           }
         }
-        float tmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        float tmax = fa_fmax8(sc);
         tmax = fa_rows_max(tmax);
         // The softmax reference of a column moves only when the page maximum exceeds it by more than kLazyLog2:
         // until then the probabilities are taken against the old reference (at most 2^kLazyLog2, exact in the

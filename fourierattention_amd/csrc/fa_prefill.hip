@@ -216,9 +216,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
           if (key > row_lim || key >= p.S) s[e] = -INFINITY;
         }
       }
-      float tmax = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+      float tmax = fa_fmax8(s);
       tmax = fa_rows_max(tmax) * p.sm_log2e;   // (the scale is positive)
-      const float m_new = fmaxf(m_run[rb], tmax);
+      const float m_new = fa_fmax(m_run[rb], tmax);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a row that has seen no key yet
       alpha[rb] = __builtin_amdgcn_exp2f(m_run[rb] - m_use);   // 0 on the row's first tile
       float psum = 0.f;
