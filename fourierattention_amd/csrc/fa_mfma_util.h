@@ -72,6 +72,11 @@ template <int AFTER>
 __device__ __forceinline__ void lds_wait_for4(uint4v (&r)[4]) {
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(AFTER) : "memory");
 }
+// the same for two reads
+template <int AFTER>
+__device__ __forceinline__ void lds_wait_for2(uint4v& a, uint4v& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(AFTER) : "memory");
+}
 // sum of eight floats STEP bytes apart, read like the accesses above and complete on return
 template <int STEP>
 __device__ __forceinline__ float lds_sum8_b32(unsigned lds_addr) {

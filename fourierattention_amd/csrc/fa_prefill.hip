@@ -152,44 +152,40 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
     // ---- S^T = K . Q^T
     float4v sacc[2][2] = {{float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}},
                           {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}}};
+    // K fragments f = block * KS + kstep, two at a time into alternating halves of kf: the reads of a pair are on
+    // their way while the matrix unit works on the pair before
     uint4v kf[4];
+    constexpr int NFK = 2 * KS;
+    auto s_pair = [&](uint4v& f0, uint4v& f1, int f) {   // fragments f, f + 1 (f is a constant after unrolling)
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int k0 = 0; k0 < KS; k0 += 4) {
-        if constexpr (KS >= 4) {
-          if (kb == 0) {
-            kf[0] = lds_read_b128_async_at<(0 * KS + 0) * 1024>(base + k0 * 1024);
-            kf[1] = lds_read_b128_async_at<(0 * KS + 1) * 1024>(base + k0 * 1024);
-            kf[2] = lds_read_b128_async_at<(0 * KS + 2) * 1024>(base + k0 * 1024);
-            kf[3] = lds_read_b128_async_at<(0 * KS + 3) * 1024>(base + k0 * 1024);
-          } else {
-            kf[0] = lds_read_b128_async_at<(1 * KS + 0) * 1024>(base + k0 * 1024);
-            kf[1] = lds_read_b128_async_at<(1 * KS + 1) * 1024>(base + k0 * 1024);
-            kf[2] = lds_read_b128_async_at<(1 * KS + 2) * 1024>(base + k0 * 1024);
-            kf[3] = lds_read_b128_async_at<(1 * KS + 3) * 1024>(base + k0 * 1024);
-          }
-          lds_wait_for4<0>(kf);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            sacc[kb][0] = M::mma(__builtin_bit_cast(vec8, kf[j]), Qf[0][k0 + j], sacc[kb][0]);
-            sacc[kb][1] = M::mma(__builtin_bit_cast(vec8, kf[j]), Qf[1][k0 + j], sacc[kb][1]);
-          }
-        } else {   // heads of 64 dims: both key blocks in one batch of four fragments
-          if (kb == 0) {
-            kf[0] = lds_read_b128_async_at<0 * 1024>(base);
-            kf[1] = lds_read_b128_async_at<1 * 1024>(base);
-            kf[2] = lds_read_b128_async_at<2 * 1024>(base);
-            kf[3] = lds_read_b128_async_at<3 * 1024>(base);
-            lds_wait_for4<0>(kf);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              sacc[j / 2][0] = M::mma(__builtin_bit_cast(vec8, kf[j]), Qf[0][j % 2], sacc[j / 2][0]);
-              sacc[j / 2][1] = M::mma(__builtin_bit_cast(vec8, kf[j]), Qf[1][j % 2], sacc[j / 2][1]);
-            }
-          }
-        }
+      for (int rb = 0; rb < 2; ++rb) {
+        sacc[f / KS][rb] = M::mma(__builtin_bit_cast(vec8, f0), Qf[rb][f % KS], sacc[f / KS][rb]);
+        sacc[(f + 1) / KS][rb] = M::mma(__builtin_bit_cast(vec8, f1), Qf[rb][(f + 1) % KS], sacc[(f + 1) / KS][rb]);
       }
+    };
+    kf[0] = lds_read_b128_async_at<0 * 1024>(base);
+    kf[1] = lds_read_b128_async_at<1 * 1024>(base);
+    kf[2] = lds_read_b128_async_at<2 * 1024>(base);
+    kf[3] = lds_read_b128_async_at<3 * 1024>(base);
+    if constexpr (NFK == 8) {
+      lds_wait_for2<2>(kf[0], kf[1]);
+      s_pair(kf[0], kf[1], 0);
+      kf[0] = lds_read_b128_async_at<4 * 1024>(base);
+      kf[1] = lds_read_b128_async_at<5 * 1024>(base);
+      lds_wait_for2<2>(kf[2], kf[3]);
+      s_pair(kf[2], kf[3], 2);
+      kf[2] = lds_read_b128_async_at<6 * 1024>(base);
+      kf[3] = lds_read_b128_async_at<7 * 1024>(base);
+      lds_wait_for2<2>(kf[0], kf[1]);
+      s_pair(kf[0], kf[1], 4);
+      lds_wait_for2<0>(kf[2], kf[3]);
+      s_pair(kf[2], kf[3], 6);
+    } else {   // heads of 64 dims: four fragments
+      static_assert(NFK == 4, "head dims of 64 or 128");
+      lds_wait_for2<2>(kf[0], kf[1]);
+      s_pair(kf[0], kf[1], 0);
+      lds_wait_for2<0>(kf[2], kf[3]);
+      s_pair(kf[2], kf[3], 2);
     }
     // V^T fragments of the first half of the dims are requested now and used after the softmax
     uint4v vf[4];
@@ -238,21 +234,33 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
         oacc[dg][1] *= alpha[1];
       }
     }
-    // ---- O^T += V^T . P^T
+    // ---- O^T += V^T . P^T (the fragments in pairs, like the K fragments above)
+    auto o_pair = [&](uint4v& f0, uint4v& f1, int dg) {
 #pragma unroll
-    for (int d0 = 0; d0 < DG; d0 += 4) {
-      if (d0 > 0) {
-        vf[0] = lds_read_b128_async_at<0>(vbase + d0 * 1024);
-        vf[1] = lds_read_b128_async_at<1024>(vbase + d0 * 1024);
-        vf[2] = lds_read_b128_async_at<2048>(vbase + d0 * 1024);
-        vf[3] = lds_read_b128_async_at<3072>(vbase + d0 * 1024);
+      for (int rb = 0; rb < 2; ++rb) {
+        oacc[dg][rb] = M::mma(__builtin_bit_cast(vec8, f0), pb[rb], oacc[dg][rb]);
+        oacc[dg + 1][rb] = M::mma(__builtin_bit_cast(vec8, f1), pb[rb], oacc[dg + 1][rb]);
       }
-      lds_wait_for4<0>(vf);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        oacc[d0 + j][0] = M::mma(__builtin_bit_cast(vec8, vf[j]), pb[0], oacc[d0 + j][0]);
-        oacc[d0 + j][1] = M::mma(__builtin_bit_cast(vec8, vf[j]), pb[1], oacc[d0 + j][1]);
-      }
+    };
+    if constexpr (DG == 8) {
+      lds_wait_for2<2>(vf[0], vf[1]);
+      o_pair(vf[0], vf[1], 0);
+      vf[0] = lds_read_b128_async_at<4 * 1024>(vbase);
+      vf[1] = lds_read_b128_async_at<5 * 1024>(vbase);
+      lds_wait_for2<2>(vf[2], vf[3]);
+      o_pair(vf[2], vf[3], 2);
+      vf[2] = lds_read_b128_async_at<6 * 1024>(vbase);
+      vf[3] = lds_read_b128_async_at<7 * 1024>(vbase);
+      lds_wait_for2<2>(vf[0], vf[1]);
+      o_pair(vf[0], vf[1], 4);
+      lds_wait_for2<0>(vf[2], vf[3]);
+      o_pair(vf[2], vf[3], 6);
+    } else {
+      static_assert(DG == 4, "head dims of 64 or 128");
+      lds_wait_for2<2>(vf[0], vf[1]);
+      o_pair(vf[0], vf[1], 0);
+      lds_wait_for2<0>(vf[2], vf[3]);
+      o_pair(vf[2], vf[3], 2);
     }
   }
 
