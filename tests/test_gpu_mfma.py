@@ -78,6 +78,11 @@ MFMA_CASES = [
     # 1024 frequencies: the mid rows run as a score pass and a value pass
     (torch.bfloat16, 5, 16, 4, 128, 4, 32, 2048, 4500, 2, [64] * 4, [64] * 4),
     (torch.float16, 2, 8, 2, 128, 4, 32, 2048, 4200, 2, [0, 128], [120, 7]),
+    # ... whose partials meet in the merge cut along the coefficient rows: one, two and eight query heads per KV
+    # head (one to eight classes of splits per block), head dims of 64, a head with nothing compressed
+    (torch.bfloat16, 3, 2, 2, 128, 4, 32, 2048, 4300, 2, [64, 128], [50, 0]),
+    (torch.bfloat16, 2, 4, 2, 64, 4, 32, 2048, 4300, 2, [32, 20], [64, 33]),
+    (torch.bfloat16, 1, 16, 2, 128, 4, 32, 2048, 4400, 2, [64, 100], [64, 127]),
 ]
 
 
