@@ -90,3 +90,20 @@ def test_two_calls_in_a_row_match_the_entry_point_with_a_workspace(dtype, tol):
     gpu, q, want = big
     out = torch.full((5, Hq, 1, D), float("nan"), device="cuda")
     assert torch.equal(gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True), gpu.decode_attention(q, 0, Hq, Hkv))
+
+
+@pytest.mark.gpu
+def test_two_calls_with_1024_frequencies():
+    """1024 frequencies take the two-pass mid rows and the merge whose blocks hand over through counters in the
+    buffer (cleared by the launch in front): two calls in a row, the second smaller, bit for bit as with a workspace."""
+    Hq, Hkv, D = 6, 2, 128
+    big = _cache_case(torch.bfloat16, 3, Hq, Hkv, D, 32, 2048, 4500, [64, 100], [64, 20], seed=3)
+    small = _cache_case(torch.bfloat16, 2, Hq, Hkv, D, 32, 2048, 4200, [64, 64], [64, 64], seed=4)
+    for gpu, q, want in (big, small, big):
+        gpu.balance_heads = False
+        ref = gpu.decode_attention(q, 0, Hq, Hkv)
+        out = torch.full_like(ref, float("nan"))
+        got = gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True)
+        assert got is out and torch.equal(got, ref)
+        err = np.abs(got.cpu().numpy() - want).max()
+        assert err <= 2e-3, err
