@@ -57,9 +57,12 @@ struct PrepArgs {
   int nbpg, n_slices, ks;
 };
 
-// bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx
+// LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head
+constexpr int kPrepLdsBytes = 2 * kGMax * 128 * (int)sizeof(float);
+
+// bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx; lds: kPrepLdsBytes
 template <typename E>
-__device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx) {
+__device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, void* lds) {
   const E* __restrict__ q = pa.q;
   const float* __restrict__ k_mc = pa.k_mc;
   const float* __restrict__ avg_u = pa.avg_u;
@@ -71,8 +74,8 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx) 
   float* __restrict__ c0 = pa.c0;
   const int Hq = pa.Hq, Hkv = pa.Hkv, D = pa.D, N = pa.N, Ck = pa.Ck;
   const float sm_log2e = pa.sm_log2e;
-  __shared__ float s_qs[kGMax][128];
-  __shared__ float s_qa[kGMax][128];
+  float (&s_qs)[kGMax][128] = *reinterpret_cast<float (*)[kGMax][128]>(lds);
+  float (&s_qa)[kGMax][128] = *reinterpret_cast<float (*)[kGMax][128]>((float*)lds + kGMax * 128);
   const int tid = threadIdx.x;
   const int h = blockIdx.y, b = blockIdx.z;
   const int G = Hq / Hkv;
@@ -132,7 +135,8 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx) 
 
 template <typename E>
 __global__ __launch_bounds__(256) void decode_prep_kernel(const PrepArgs<E> pa) {
-  decode_prep_body<E>(pa, blockIdx.x);
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kPrepLdsBytes];
+  decode_prep_body<E>(pa, blockIdx.x, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -1095,9 +1099,33 @@ struct IlArgs {
   float sm_log2e;
 };
 
-// bx: block index along x (tile of kIlFastTile rows); y, z come from blockIdx
+// a . b of two pairs of 16-bit values plus c, in one instruction
+typedef __bf16 fa_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 fa_f16x2 __attribute__((ext_vector_type(2)));
+template <typename E>
+__device__ __forceinline__ float fa_dot2(unsigned a, unsigned b, float c);
+template <>
+__device__ __forceinline__ float fa_dot2<bf16_t>(unsigned a, unsigned b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(fa_bf16x2, a), __builtin_bit_cast(fa_bf16x2, b), c, false);
+}
+template <>
+__device__ __forceinline__ float fa_dot2<f16_t>(unsigned a, unsigned b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(fa_f16x2, a), __builtin_bit_cast(fa_f16x2, b), c, false);
+}
+template <>
+__device__ __forceinline__ float fa_dot2<float>(unsigned, unsigned, float c) { return c; }   // never run: 16-bit rows only
+
+// LDS of a sink/window block: the four waves' maxima, denominators and outputs meet here
+template <int D, int GM>
+struct IlFastLds {
+  float m[4][GM];
+  float d[4][(64 / (D / 8)) / 2][GM];
+  __attribute__((aligned(16))) float o[4][(64 / (D / 8)) / 2][GM][D];
+};
+
+// bx: block index along x (tile of kIlFastTile rows); y, z come from blockIdx; lds: an IlFastLds<D, GM>
 template <typename E, int D, int GM>
-__device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx) {
+__device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx, void* lds) {
   const E* __restrict__ q = ia.q;
   const Seg s0 = ia.s0, s1 = ia.s1;
   float* __restrict__ pm = ia.pm;
@@ -1106,8 +1134,10 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
   const int Hq = ia.Hq, Hkv = ia.Hkv, n_split = ia.n_split;
   const float sm_log2e = ia.sm_log2e;
   constexpr int LPT = D / 8, TPW = 64 / LPT, ITERS = kIlFastTile / 4 / TPW;
-  __shared__ float s_m[4][GM], s_d[4][TPW / 2][GM];
-  __shared__ __attribute__((aligned(16))) float s_o[4][TPW / 2][GM][D];
+  IlFastLds<D, GM>& sh = *reinterpret_cast<IlFastLds<D, GM>*>(lds);
+  auto& s_m = sh.m;
+  auto& s_d = sh.d;
+  auto& s_o = sh.o;
   const int G = Hq / Hkv;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int sub = lane % LPT, tl = lane / LPT;
@@ -1129,13 +1159,7 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
 #pragma unroll
   for (int g = 0; g < GM; ++g)
     qraw[g] = *(const uint4*)(q + ((int64_t)b * Hq + h * G + min(g, G - 1)) * D + sub * 8);
-  float qv[GM][8];
-#pragma unroll
-  for (int g = 0; g < GM; ++g) {
-    const E* qe = (const E*)&qraw[g];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) qv[g][e] = g < G ? fa_to_float(qe[e]) * sm_log2e : 0.f;
-  }
+  // (the query stays packed: the scores are sums of pair products, v_dot2c, scaled once per score)
   // The wave holds only ITERS * TPW rows, so it takes one softmax block: all scores first, one maximum,
   // then the weighted sum (no running maximum, no rescaling).
   float sc[ITERS][GM], m[GM];
@@ -1144,16 +1168,14 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const bool ok = base + it * TPW + tl < n_il;
-    const E* ke = (const E*)&kraw[it];
-    float kf[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) kf[e] = fa_to_float(ke[e]);
+    const uint4 kr = kraw[it];
 #pragma unroll
     for (int g = 0; g < GM; ++g) {
-      float a = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) a = fmaf(kf[e], qv[g][e], a);
-      a = fa_group_sum<LPT>(a);
+      float a = fa_dot2<E>(kr.x, qraw[g].x, 0.f);
+      a = fa_dot2<E>(kr.y, qraw[g].y, a);
+      a = fa_dot2<E>(kr.z, qraw[g].z, a);
+      a = fa_dot2<E>(kr.w, qraw[g].w, a);
+      a = fa_group_sum<LPT>(a) * sm_log2e;
       sc[it][g] = (ok && g < G) ? a : -INFINITY;
       m[g] = fmaxf(m[g], sc[it][g]);
     }
@@ -1163,51 +1185,53 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
     if (LPT == 8) m[g] = fmaxf(m[g], fa_dpp<FA_DPP_ROR8>(m[g]));
     m[g] = fa_rows_max(m[g]);
   }
-  float d[GM], o[GM][8];
+  // The weighted sums take the query heads two at a time (the rows' V values are converted once per pair): sixteen
+  // accumulators live instead of eight per head, which is what lets six waves share a SIMD.
+  // Rows held side by side in the wave: lanes i and i + 32 meet in registers, the rest in LDS together with the
+  // four waves.
 #pragma unroll
-  for (int g = 0; g < GM; ++g) {
-    d[g] = 0.f;
+  for (int g0 = 0; g0 < GM; g0 += 2) {
+    float d[2] = {0.f, 0.f}, o[2][8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
-  }
+    for (int gg = 0; gg < 2; ++gg)
 #pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const E* ve = (const E*)&vraw[it];
-    float vf[8];
+      for (int e = 0; e < 8; ++e) o[gg][e] = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) vf[e] = fa_to_float(ve[e]);
+    for (int it = 0; it < ITERS; ++it) {
+      const E* ve = (const E*)&vraw[it];
+      float vf[8];
 #pragma unroll
-    for (int g = 0; g < GM; ++g) {
-      const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[it][g] - m[g]);
-      d[g] += pv;
+      for (int e = 0; e < 8; ++e) vf[e] = fa_to_float(ve[e]);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[g][e] = fmaf(pv, vf[e], o[g][e]);
+      for (int gg = 0; gg < 2; ++gg) {
+        const int g = g0 + gg;
+        const float pv = m[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[it][g] - m[g]);
+        d[gg] += pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[gg][e] = fmaf(pv, vf[e], o[gg][e]);
+      }
+    }
+#pragma unroll
+    for (int gg = 0; gg < 2; ++gg) {
+      const int g = g0 + gg;
+      float lo, hi;
+      fa_swap32(d[gg], &lo, &hi);
+      d[gg] = lo + hi;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        fa_swap32(o[gg][e], &lo, &hi);
+        o[gg][e] = lo + hi;
+      }
+      if (lane < 32) {
+        *(float4*)&s_o[w][tl][g][sub * 8] = make_float4(o[gg][0], o[gg][1], o[gg][2], o[gg][3]);
+        *(float4*)&s_o[w][tl][g][sub * 8 + 4] = make_float4(o[gg][4], o[gg][5], o[gg][6], o[gg][7]);
+        if (sub == 0) s_d[w][tl][g] = d[gg];
+      }
     }
   }
-  // rows held side by side in the wave: lanes i and i + 32 meet in registers, the rest in LDS together
-  // with the four waves
+  if (lane == 0) {
 #pragma unroll
-  for (int g = 0; g < GM; ++g) {
-    float lo, hi;
-    fa_swap32(d[g], &lo, &hi);
-    d[g] = lo + hi;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      fa_swap32(o[g][e], &lo, &hi);
-      o[g][e] = lo + hi;
-    }
-  }
-  if (lane < 32) {
-#pragma unroll
-    for (int g = 0; g < GM; ++g) {
-      *(float4*)&s_o[w][tl][g][sub * 8] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-      *(float4*)&s_o[w][tl][g][sub * 8 + 4] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
-      if (sub == 0) s_d[w][tl][g] = d[g];
-    }
-    if (lane == 0) {
-#pragma unroll
-      for (int g = 0; g < GM; ++g) s_m[w][g] = m[g];
-    }
+    for (int g = 0; g < GM; ++g) s_m[w][g] = m[g];
   }
   __syncthreads();
   for (int idx = tid; idx < G * D; idx += 256) {
@@ -1237,16 +1261,21 @@ __device__ __forceinline__ void decode_il_fast_body(const IlArgs<E>& ia, int bx)
 
 template <typename E, int D, int GM>
 __global__ __launch_bounds__(256) void decode_il_fast_kernel(const IlArgs<E> ia) {
-  decode_il_fast_body<E, D, GM>(ia, blockIdx.x);
+  __shared__ __attribute__((aligned(16))) unsigned char lds[sizeof(IlFastLds<D, GM>)];
+  decode_il_fast_body<E, D, GM>(ia, blockIdx.x, lds);
 }
 
 // The coefficient-domain query and the sink/window rows do not depend on each other and are both short,
 // latency-bound pieces of work: one launch runs them side by side (blocks [0, n_prep) prepare the query,
 // the rest attend over sink/window tiles).
 template <typename E, int D, int GM>
-__global__ __launch_bounds__(256) void decode_prep_il_kernel(const PrepArgs<E> pa, const IlArgs<E> ia, int n_prep) {
-  if ((int)blockIdx.x < n_prep) decode_prep_body<E>(pa, blockIdx.x);
-  else decode_il_fast_body<E, D, GM>(ia, blockIdx.x - n_prep);
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GM <= 4 ? 6 : 4, GM <= 4 ? 6 : 4)))
+void decode_prep_il_kernel(const PrepArgs<E> pa, const IlArgs<E> ia, int n_prep) {
+  // one buffer for whichever piece the block runs: what a block holds in LDS decides how many run side by side
+  constexpr int kLds = (int)sizeof(IlFastLds<D, GM>) > kPrepLdsBytes ? (int)sizeof(IlFastLds<D, GM>) : kPrepLdsBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kLds];
+  if ((int)blockIdx.x < n_prep) decode_prep_body<E>(pa, blockIdx.x, lds);
+  else decode_il_fast_body<E, D, GM>(ia, blockIdx.x - n_prep, lds);
 }
 
 // ---------------------------------------------------------------------------
