@@ -55,6 +55,14 @@ struct PrepArgs {
   // that each of its loads is one contiguous 512-byte line
   float* W_lane;
   int nbpg, n_slices, ks;
+  // and the stored query dims of a column go out as that kernel's B operands (16-bit, zeros where a lane holds
+  // nothing): [batch group][KV head][batch element of the group, 4][kstep, 4][64 lanes] x 8 values, lane
+  // (lg, lc) of kstep s holding the dims kn_list[32 s + 8 lg + 0 .. 7] of column lc if the column belongs to
+  // that batch element.  The mid-row launch then starts with one load per kstep instead of an index load and a
+  // gather that depends on it.
+  E* q_stored;
+  const int32_t* kn_list;
+  const int32_t* kn_h;
 };
 
 // LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head
@@ -100,6 +108,23 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
       float v = fa_wave_sum(s_qa[g][tid] + s_qa[g][tid + 64]);
       if (tid == 0) c0[(int64_t)b * Hq + h * G + g] = v * sm_log2e;
     }
+  }
+  if constexpr (sizeof(E) == 2) if (bx == 1 && pa.q_stored) {
+    const int kn0 = pa.kn_h[h], kn_len = pa.kn_h[h + 1] - kn0;
+    const int s = tid >> 6, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
+    const int grp = b / pa.nbpg, sl = b - grp * pa.nbpg;
+    const int g = lc - sl * G;   // the column's query head if the column is this batch element's
+    const bool mine = g >= 0 && g < G;
+    const E* qr = q + ((int64_t)b * Hq + h * G + (mine ? g : 0)) * D - h * D;
+    union { E e[8]; uint4 raw; } o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = s * 32 + 8 * lg + e;
+      const E qv = qr[pa.kn_list[kn0 + min(j, max(kn_len - 1, 0))]];   // clamped: no load under a condition
+      o.e[e] = (mine && j < kn_len) ? qv : E();
+    }
+    if (kn_len > 0)
+      *(uint4*)(pa.q_stored + ((((int64_t)(grp * Hkv + h) * 4 + sl) * 4 + s) * 64 + lane) * 8) = o.raw;
   }
   const int n = bx * kPrepRows + (tid >> 2), jq = tid & 3;
   if (n >= 2 * N) return;
@@ -1309,6 +1334,7 @@ struct Plan {
   // merge after the matrix-core mid rows: contributions per block of coefficient rows, staged sums, counters
   int n_row_blocks;
   size_t off_pc, off_sil, off_son, off_cnt;
+  size_t off_qn;   // stored query dims as B operands of the mid-row kernel
 };
 
 bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
@@ -1424,6 +1450,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_sil = take(mfma ? rows * D * 4 : 0);
   p.off_son = take(mfma ? rows * D * 4 : 0);
   p.off_cnt = take(mfma ? (size_t)B * Hkv * 4 : 0);
+  p.off_qn = take(mfma ? (size_t)p.n_groups * Hkv * 4 * 4 * 64 * 16 : 0);
   p.total = o;
   return p;
 }
@@ -1496,7 +1523,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   if (p.n_mid_split > 0) {
     PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
                    a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e,
-                   p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks};
+                   p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks,
+                   p.path == Path::Mfma ? (E*)(ws + p.off_qn) : nullptr, a.kn_list, a.kn_h_list};
     const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
@@ -1528,6 +1556,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.scores = (float*)(ws + p.off_scores);
         mp.merge_count = (unsigned*)(ws + p.off_cnt);
+        mp.q_stored = (const E*)(ws + p.off_qn);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.st = p.st;
         mp.sm_log2e = sm_log2e;

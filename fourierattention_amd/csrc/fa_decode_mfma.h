@@ -223,6 +223,7 @@ struct SplitTable {
 template <typename E>
 struct MidParams {
   const E* q;
+  const E* q_stored;    // the stored query dims as B operands: [batch group][KV head][batch element, 4][kstep, 4][lane] x 8
   const float* W;       // fp32, already carrying sm_scale*log2e/N, in the lane layout of the score waves:
                         // [batch group][KV head][slice][row tile][cos | sin][column][pair of frequencies] x float2
   const float* c0;      // [B][Hq]
@@ -292,8 +293,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int sl = MODE == 0 ? (w & 3) : w;  // frequency slice; below 4 also the batch element of the group
   // workgroup -> (KV head, split of that head)
   const int grp = blockIdx.y;
+  // (the first sixteen entries are compared at once: they arrive with one load of the argument block, where a
+  // scan waits for one dependent load per head)
   int h = 0;
-  while (h + 1 < p.Hkv && (int)blockIdx.x >= p.st.first[h + 1]) ++h;
+#pragma unroll
+  for (int i = 1; i < 16; ++i) h += (int)blockIdx.x >= p.st.first[i] ? 1 : 0;
+  if (p.Hkv > 16)
+    while (h + 1 < p.Hkv && (int)blockIdx.x >= p.st.first[h + 1]) ++h;
   const int split = blockIdx.x - p.st.first[h];
   const int G = p.G, N = p.N;
   const int b0 = grp * p.nbpg;
@@ -340,9 +346,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   if (score_wave) {
     // =============================== score waves ===============================
-    // stored K dims of batch element sl: both 16-token blocks of the page.  The first pages are requested
-    // before anything else, so that HBM is busy while the tables and the query are being set up.
-    const int kn0 = p.kn_h[h], kn_len = p.kn_h[h + 1] - kn0;
+    // stored K dims of batch element sl: both 16-token blocks of the page
     const int kp0 = p.kpad_h[h], dpk = p.kpad_h[h + 1] - kp0;
     const int nks = dpk >> 5;
     const E* kbase = p.k_mid + (int64_t)my_b * p.k_bs + (int64_t)kp0 * 32 * p.cap_pages;  // wave-uniform
@@ -358,30 +362,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int ks = 0; ks < KMAX; ++ks)
           if (ks < nks) load_frag_to_lds<2>(kp + ((mir ? 1 - tb : tb) * nks + ks) * 512, st + (tb * KMAX + ks) * 1024);
     };
-    if (has_k) {
-#pragma unroll
-      for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_k(t_beg + i, (i & 1) == 0);
-    }
     rot_fetch();
-    // the index list of the gathered query dims is requested now: the query loads that depend on it then go out
-    // while the tables and the weights are still on their way, instead of starting a round trip of their own later
-    int dim[KMAX][8];
-    if (kn_len > 0) {
-      const int32_t* kl = p.kn_list + kn0;
-#pragma unroll
-      for (int s = 0; s < KMAX; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dim[s][e] = kl[min(s * 32 + 8 * lg + e, kn_len - 1)];
-    }
     half8 Ea[2][KS];
 
     // coefficient-domain query: Wc/Ws[rt][f2] = (cos-row, sin-row) weights of frequency
     // freq_of(rt, lg, f2) for column lc; normalised per column, rotated to the centre of the first frame
     float Wc[2 * KS][2], Ws[2 * KS][2];
     float wmax = 0.f;
-    // the gathered query values: requested behind the weights, needed only once those have been processed
-    E qv[KMAX][8];
+    // the stored query dims of this wave's batch element, laid out as B operands by the launch in front (zeros in
+    // the lanes of other batch elements and past the head's count): requested behind the weights
+    vec8 Qb[KMAX];
     {
       const float2v* wl = (const float2v*)p.W + ((int64_t)((grp * p.Hkv + h) * NSL + sl) * 2 * KS * 2) * 64 + (lc * 4 + lg);
       float2v wc2[2 * KS], ws2[2 * KS];
@@ -396,12 +386,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int s = 0; s < KS; ++s) Ea[rb][s] = p.tabE[((sl * 2 + rb) * KS + s) * 64 + lane];
-      if (kn_len > 0) {
-        const E* qr = p.q + qrow * p.D - h * p.D;
+      {
+        const vec8* qs = (const vec8*)p.q_stored + ((int64_t)((grp * p.Hkv + h) * 4 + stw) * 4) * 64 + lane;
 #pragma unroll
-        for (int s = 0; s < KMAX; ++s)
+        for (int s = 0; s < KMAX; ++s) Qb[s] = qs[s * 64];   // used by waves that stream K pages only
+      }
+      // The first pages go out behind the operand loads: loads return in order, and a first access to a page of
+      // the store takes about twice as long as the operands, which the weights below would otherwise wait for.
+      if (has_k) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) qv[s][e] = qr[dim[s][e]];
+        for (int i = 0; i < NST - 1; ++i)
+          if (i < n_it) issue_k(t_beg + i, (i & 1) == 0);
       }
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) {
@@ -439,21 +434,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
-    // the gathered query dims: all index loads first, then all query loads (clamped so that none is
-    // conditional: conditional loads would be issued one round trip after the other)
-    vec8 Qb[KMAX];
-#pragma unroll
-    for (int s = 0; s < KMAX; ++s)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Qb[s][e] = (typename M::elem)0.f;
-    if (kn_len > 0) {   // nothing inside these branches is conditional
-      const bool mine = has_mn && valid_r && bb_r == sl;
-#pragma unroll
-      for (int s = 0; s < KMAX; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (mine && s * 32 + 8 * lg + e < kn_len) Qb[s][e] = M::from_bits(qv[s][e]);
-    }
     // every table and weight load above must have landed before the loop starts: inside it the only
     // waits on vector memory in this wave are the explicit page waits
 #pragma unroll
@@ -602,15 +582,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int f = 0; f < VMAX; ++f)
         if (f < ndg) load_frag_to_lds<2>(vp + f * 512, st + f * 1024);
     };
-    if (streams_v) {   // first pages requested before the tables (see the score waves)
-#pragma unroll
-      for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_v(t_beg + i, (i & 1) == 0);
-    }
     rot_fetch();
     half8 ETa[2 * KS];   // tile 2j: cosines, tile 2j + 1: sines of the frequencies 16j .. 16j + 15 of the slice
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
+    if (streams_v) {   // first pages requested behind the table (see the score waves)
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i)
+        if (i < n_it) issue_v(t_beg + i, (i & 1) == 0);
+    }
     rot_store();
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
