@@ -808,7 +808,7 @@ __global__ __launch_bounds__(1024) void decode_merge_kernel(
 constexpr int kMrTiles = 8;               // g tiles of 8 frequencies per block
 constexpr int kMrRows = kMrTiles * 16;    // coefficient rows per block (cos and sin of 64 frequencies)
 constexpr int kMrGPre = 8;                // g partials (16 bytes each) a thread requests ahead
-constexpr int kMrVPre = 32;               // V-coefficient values a thread requests ahead
+constexpr int kMrVPre = 8;                // V-coefficient groups of four dims a thread requests ahead
 constexpr int kMrSub = 4;                 // lanes that share one (query head, dim) of the staged sums
 constexpr int kMrIlPre = 6, kMrOnPre = 4; // sink/window and mid partial outputs requested ahead per lane
 
@@ -818,6 +818,28 @@ constexpr int kMrIlPre = 6, kMrOnPre = 4; // sink/window and mid partial outputs
 // loads after it has seen the count, so no cache write-back or invalidate is needed around the counter.
 __device__ __forceinline__ void st_device(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float ld_device(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+template <int CTRL>
+__device__ __forceinline__ float4 fa_dpp4_add(float4 v) {
+  v.x += fa_dpp<CTRL>(v.x); v.y += fa_dpp<CTRL>(v.y); v.z += fa_dpp<CTRL>(v.z); v.w += fa_dpp<CTRL>(v.w);
+  return v;
+}
+// sum over the lanes q, q + nqp, q + 2 nqp, ... of a wave (nqp a power of two up to 32, uniform over the wave); every
+// lane gets the sum of its class
+__device__ __forceinline__ float4 fa_sum_lane_classes(float4 v, int nqp) {
+  if (nqp <= 1) v = fa_dpp4_add<0x121>(v);   // row_ror:1
+  if (nqp <= 2) v = fa_dpp4_add<0x122>(v);   // row_ror:2
+  if (nqp <= 4) v = fa_dpp4_add<0x124>(v);   // row_ror:4
+  if (nqp <= 8) v = fa_dpp4_add<0x128>(v);   // row_ror:8
+  float lo, hi;
+  if (nqp <= 16) {
+    fa_swap16(v.x, &lo, &hi); v.x = lo + hi; fa_swap16(v.y, &lo, &hi); v.y = lo + hi;
+    fa_swap16(v.z, &lo, &hi); v.z = lo + hi; fa_swap16(v.w, &lo, &hi); v.w = lo + hi;
+  }
+  fa_swap32(v.x, &lo, &hi); v.x = lo + hi; fa_swap32(v.y, &lo, &hi); v.y = lo + hi;
+  fa_swap32(v.z, &lo, &hi); v.z = lo + hi; fa_swap32(v.w, &lo, &hi); v.w = lo + hi;
+  return v;
+}
 
 struct MergeRowsArgs {
   const float* il_m; const float* il_d; const float* il_o; int n_il_split;
@@ -844,8 +866,8 @@ __global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsA
   float* s_d = s_w + G * n_all;             // [G][n_all]
   float* s_sc = s_d + G * n_all;            // [2][kGMax]
   float* s_g = s_sc + 2 * kGMax;            // [G][128]: cos rows of the block's 64 frequencies, then sin rows
-  float* s_x = s_g + G * kMrRows;           // max(1024, 256 * G): g per split class, then the row classes of the product
-  float* s_o = s_x + (256 * G > 1024 ? 256 * G : 1024);   // [G][D], last block
+  float* s_x = s_g + G * kMrRows;           // max(1024, 512 * G): g per split class, then the four waves' sums of the product
+  float* s_o = s_x + (512 * G > 1024 ? 512 * G : 1024);   // [G][D], last block
   __shared__ int s_last;
 
   // ---- requests: first those whose addresses do not wait for the head's entries of the index lists ------------
@@ -886,20 +908,31 @@ __global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsA
   }
   const int vc0 = a.vc_h[h], vc_len = a.vc_h[h + 1] - vc0;
   const int vn0 = a.vn_h[h], vn_len = a.vn_h[h + 1] - vn0;
-  int cwp = 2;                              // power of two >= vc_len: threads = (dim, row class)
-  while (cwp < vc_len) cwp <<= 1;
-  const int parts = 256 / cwp;              // vc_len <= D <= 128: at least two row classes
+  int nqp = 2;                              // groups of four dims, a power of two (at least two: no more row classes
+                                            // than rows): threads = (group, row class)
+  while (4 * nqp < vc_len) nqp <<= 1;
+  const int cwp = 4 * nqp;
+  const int parts = 256 / nqp;              // vc_len <= D <= 128: at least eight row classes
   const bool has_coef = vc_len > 0;
-  // V coefficients: local row rr < 64 is the cos row of frequency 64 z + rr, rr >= 64 the sin row of 64 z + rr - 64
-  const int j = tid & (cwp - 1), part = tid / cwp;
+  // V coefficients: local row rr < 64 is the cos row of frequency 64 z + rr, rr >= 64 the sin row of 64 z + rr - 64;
+  // 16 bytes per load where the head's columns allow it (the address path takes one load instruction of a wave per
+  // 16 clocks whatever its width)
+  const int vq = tid & (nqp - 1), part = tid / nqp;
   const int rows_per_thread = kMrRows / parts;           // parts divides 128
   auto v_row = [&](int rr) { return rr < 64 ? 64 * z + rr : N + 64 * z + (rr - 64); };
-  const float* vp = a.v_mc + (int64_t)b * 2 * N * a.Cv + vc0 + j;
-  const bool v_on = has_coef && j < vc_len;
-  float v_pre[kMrVPre];
+  const float* vp = a.v_mc + (int64_t)b * 2 * N * a.Cv + vc0 + 4 * vq;
+  const bool v_on = has_coef && 4 * vq < vc_len;
+  const int v_lim = vc_len - 4 * vq - 1;    // last valid offset within the group of four
+  const bool v_wide = v_lim >= 3 && ((vc0 | a.Cv) & 3) == 0 && ((uintptr_t)a.v_mc & 15) == 0;
+  auto v_load = [&](int rr) {
+    const float* p4 = vp + (int64_t)v_row(min(rr, kMrRows - 1)) * a.Cv;
+    if (v_wide) return *(const float4*)p4;
+    return make_float4(p4[0], p4[min(1, v_lim)], p4[min(2, v_lim)], p4[min(3, v_lim)]);   // dims past the head's: unused
+  };
+  float4 v_pre[kMrVPre];
   if (v_on) {
 #pragma unroll
-    for (int u = 0; u < kMrVPre; ++u) v_pre[u] = vp[(int64_t)v_row(min(part + u * parts, kMrRows - 1)) * a.Cv];
+    for (int u = 0; u < kMrVPre; ++u) v_pre[u] = v_load(part + u * parts);
   }
   // this block's share of the stored positions of the mid rows
   const int nsh = (vn_len + R - 1) / R, n_lo = min(vn_len, z * nsh), n_n = min(vn_len, n_lo + nsh) - n_lo;
@@ -976,42 +1009,42 @@ __global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsA
     }
     __syncthreads();
     // ---- times the block's rows of the V coefficients
-    float acc[kGMax];
+    float4 acc[kGMax];
 #pragma unroll
-    for (int g = 0; g < kGMax; ++g) acc[g] = 0.f;
+    for (int g = 0; g < kGMax; ++g) acc[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fma_row = [&](int rr, const float4& v) {
+#pragma unroll
+      for (int g = 0; g < kGMax; ++g)
+        if (g < G) {
+          const float gg = s_g[g * kMrRows + rr];
+          acc[g].x = fmaf(gg, v.x, acc[g].x); acc[g].y = fmaf(gg, v.y, acc[g].y);
+          acc[g].z = fmaf(gg, v.z, acc[g].z); acc[g].w = fmaf(gg, v.w, acc[g].w);
+        }
+    };
     if (v_on) {
 #pragma unroll
-      for (int u = 0; u < kMrVPre; ++u) {
-        const int rr = part + u * parts;
-        if (u < rows_per_thread) {
-#pragma unroll
-          for (int g = 0; g < kGMax; ++g)
-            if (g < G) acc[g] = fmaf(s_g[g * kMrRows + rr], v_pre[u], acc[g]);
-        }
-      }
-      for (int u0 = kMrVPre; u0 < rows_per_thread; u0 += 16) {
-        float v[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) v[u] = vp[(int64_t)v_row(min(part + (u0 + u) * parts, kMrRows - 1)) * a.Cv];
-#pragma unroll
-        for (int u = 0; u < 16; ++u)
-          if (u0 + u < rows_per_thread) {
-#pragma unroll
-            for (int g = 0; g < kGMax; ++g)
-              if (g < G) acc[g] = fmaf(s_g[g * kMrRows + part + (u0 + u) * parts], v[u], acc[g]);
-          }
-      }
+      for (int u = 0; u < kMrVPre; ++u)
+        if (u < rows_per_thread) fma_row(part + u * parts, v_pre[u]);
+      for (int u = kMrVPre; u < rows_per_thread; ++u) fma_row(part + u * parts, v_load(part + u * parts));
     }
+    // the row classes of a wave meet through lane exchanges, the four waves in LDS
 #pragma unroll
     for (int g = 0; g < kGMax; ++g)
-      if (g < G) s_x[(part * G + g) * cwp + j] = acc[g];
+      if (g < G) {
+        const float4 v = fa_sum_lane_classes(acc[g], nqp);
+        if (lane < nqp) {
+          float* dst = s_x + (wv * G + g) * cwp + 4 * lane;
+          dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+        }
+      }
     __syncthreads();
     float* pc = a.part_c + (((int64_t)b * Hkv + h) * R + z) * G * 128;
     for (int idx = tid; idx < G * cwp; idx += 256) {
       const int g = idx / cwp, jj = idx - g * cwp;
       if (jj < vc_len) {
         float v = 0.f;
-        for (int pp = 0; pp < parts; ++pp) v += s_x[(pp * G + g) * cwp + jj];
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) v += s_x[(ww * G + g) * cwp + jj];
         st_device(pc + g * 128 + jj, v);
       }
     }
@@ -1104,6 +1137,294 @@ __global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsA
     }
   }
 }
+
+// ---------------------------------------------------------------------------
+// merge after the matrix-core mid rows, up to four query heads per KV head: the result of decode_merge_kernel with
+// the loads laid out for the address path.  A compute unit takes one load instruction of a wave every 16 clocks
+// whatever its width, and this kernel's time is the number of such instructions: every thread therefore reads 16
+// bytes per load wherever the data allow it, and nothing is loaded after the first barrier on the common shapes.
+//   g partials     one thread per group of four values {cos f, sin f, cos f+1, sin f+1} of one query head, GPRE
+//                  splits requested ahead (all of them for an even share of the mid rows)
+//   V coefficients thread = (four neighbouring dims of the block's share, row class): 16-byte loads where the head's
+//                  columns allow it; the row classes of a wave are folded with lane exchanges, the waves in LDS
+//   sink/window    thread = (query head, four neighbouring dims, one of eight split groups)
+//   stored dims    thread = (query head, position in the head's list, split group)
+// Block (KV head, b, z) applies the V coefficients of share z of the head's dims, like decode_merge_kernel.
+// ---------------------------------------------------------------------------
+constexpr int kMfG = 4;        // query heads per KV head (one 16-byte row of the folded g per coefficient row)
+constexpr int kMfIlPre = 3;    // sink/window partial outputs (16 bytes each) a thread requests ahead
+constexpr int kMfOnPre = 2;    // stored-dim partial outputs a thread requests ahead
+
+template <int GPRE, int VPRE>
+__global__ __launch_bounds__(1024) void decode_merge_fast_kernel(const MergeRowsArgs a) {
+  auto put = [&](int64_t at, float v) {
+    if (a.out) a.out[at] = v;
+    if (a.out_cast) {
+      if (a.cast_dtype == FA_BF16) ((bf16_t*)a.out_cast)[at] = bf16_t{fa_f32_to_bf16_bits(v)};
+      else if (a.cast_dtype == FA_FP16) ((f16_t*)a.out_cast)[at] = f16_t{(_Float16)v};
+      else ((float*)a.out_cast)[at] = v;
+    }
+  };
+  extern __shared__ float smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h = blockIdx.x, b = blockIdx.y, z = blockIdx.z, n_chunks = gridDim.z;
+  const int Hq = a.Hq, Hkv = a.Hkv, D = a.D, N = a.N, Cv = a.Cv, G = Hq / Hkv;
+  const int n_il = a.n_il_split, n_mid = min(a.st.n[h], a.n_mid_stride), n_all = n_il + n_mid;
+  const int WM = (a.n_mid_stride + 3) & ~3;   // row of the mid-split weights, 16-byte aligned
+  const int64_t r0 = (int64_t)b * Hq + h * G;
+  const int vc0 = a.vc_h[h], vc_len = a.vc_h[h + 1] - vc0;
+  const int vn0 = a.vn_h[h], vn_len = a.vn_h[h + 1] - vn0;
+  // this block's share of the compressed and of the stored dims (by position in the head's lists)
+  const int cw = (vc_len + n_chunks - 1) / n_chunks;
+  const int c_lo = min(vc_len, z * cw), cn = min(vc_len, c_lo + cw) - c_lo;
+  const int nw = (vn_len + n_chunks - 1) / n_chunks;
+  const int n_lo = min(vn_len, z * nw), nn = min(vn_len, n_lo + nw) - n_lo;
+  const bool has_coef = n_mid > 0 && cn > 0;
+  int nqp = 1;   // groups of four dims in the share, rounded up to a power of two (at most 32: 128 dims)
+  while (4 * nqp < cw) nqp <<= 1;
+  const int CWP = 4 * nqp;
+
+  // (what is read 16 bytes at a time comes first)
+  float* s_g = smem;                           // [2N][4]: folded g, one 16-byte row per coefficient row
+  float* s_wm = s_g + 2 * N * kMfG;            // [4][WM]: weights of the mid splits (zero past the head's count)
+  float* s_part = s_wm + kMfG * WM;            // [16 waves][4][CWP]
+  float* s_w = s_part + 16 * kMfG * CWP;       // [G][n_all]
+  float* s_d = s_w + G * n_all;                // [G][n_all]
+  float* s_sc = s_d + G * n_all;               // [2][kGMax]: sum of d, sum of d over the mid rows
+  float* s_o = s_sc + 2 * kGMax;               // [G][D]
+  int* s_own = (int*)(s_o + G * D);            // [D]: bit 0 = some list holds the dim, bit 1 = this block writes it
+
+  // ---- every load of the common shapes, issued before anything is waited for ---------------------------------
+  // (first the dim that position tid of the head's lists names: G * D <= 512 threads cover both lists)
+  int own_dim = -1;
+  if (tid < vc_len + vn_len) own_dim = (tid < vc_len ? a.vc_list[vc0 + tid] : a.vn_list[vn0 + tid - vc_len]) - h * D;
+  float m_raw = -INFINITY, d_raw = 0.f;
+  if (tid < G * n_all) {
+    const int g = tid / n_all, s_ = tid - g * n_all;
+    const int64_t r = r0 + g;
+    const bool il = s_ < n_il;
+    m_raw = il ? a.il_m[r * n_il + s_] : a.md_m[r * a.n_mid_stride + (s_ - n_il)];
+    d_raw = il ? a.il_d[r * n_il + s_] : a.md_d[r * a.n_mid_stride + (s_ - n_il)];
+  }
+  // g partials: item = (tile of 8 frequencies, query head, pair of frequencies within the tile); consecutive items
+  // walk through the 64 * G contiguous bytes this block owns in a tile of a split
+  const int n_items = G * (N / 2);
+  const int64_t g_stride = (int64_t)16 * 2 * N;   // floats between two splits
+  const int g_of = (tid >> 2) % G, n4 = (tid / (4 * G)) * 4 + (tid & 3);
+  const float* gp = nullptr;
+  float4 gv[GPRE];
+  const bool g_on = has_coef && tid < n_items;
+  if (g_on) {
+    const int grp = b / a.nbpg, lc = (b - grp * a.nbpg) * G + g_of;
+    gp = a.md_g + (int64_t)(grp * Hkv + h) * a.n_mid_stride * g_stride + (int64_t)(n4 >> 2) * 256 + (lc * 4 + (n4 & 3)) * 4;
+#pragma unroll
+    for (int u = 0; u < GPRE; ++u) gv[u] = *(const float4*)(gp + (int64_t)min(u, n_mid - 1) * g_stride);
+  }
+  // V coefficients: dims c_lo + 4 q .. + 3 of the head's list, rows cls, cls + classes, ...
+  const int q = tid & (nqp - 1), cls = tid / nqp, classes = 1024 / nqp;
+  const bool v_on = has_coef && 4 * q < cn;
+  const int v_lim = cn - 4 * q - 1;   // last valid offset within the group of four
+  const float* vp = a.v_mc + (int64_t)b * 2 * N * Cv + vc0 + c_lo + 4 * q;
+  const bool v_wide = v_lim >= 3 && ((vc0 + c_lo) & 3) == 0 && (Cv & 3) == 0 && ((uintptr_t)a.v_mc & 15) == 0;
+  auto v_load = [&](int n) {
+    const float* p4 = vp + (int64_t)min(n, 2 * N - 1) * Cv;
+    if (v_wide) return *(const float4*)p4;
+    return make_float4(p4[0], p4[min(1, v_lim)], p4[min(2, v_lim)], p4[min(3, v_lim)]);   // dims past the share: unused
+  };
+  float4 vv[VPRE];
+  if (v_on) {
+#pragma unroll
+    for (int u = 0; u < VPRE; ++u) vv[u] = v_load(cls + u * classes);
+  }
+  // what the last step of the compressed dims needs: thread = (query head, dim of the share)
+  const int fin_g = tid / CWP, fin_j = tid - fin_g * CWP;
+  const bool fin_on = has_coef && fin_g < G && fin_j < cn;
+  float fin_scale = 0.f, fin_au = 0.f, fin_ad = 0.f;
+  int fin_dim = 0;
+  if (fin_on) {
+    const int64_t o = (int64_t)b * Cv + vc0 + c_lo + fin_j;
+    fin_scale = a.scale[o]; fin_au = a.avg_u[o]; fin_ad = a.avg_d[o];
+    fin_dim = a.vc_list[vc0 + c_lo + fin_j] - h * D;
+  }
+
+  // ---- split weights: one wave per query head ------------------------------------------------------------------
+  if (tid < G * n_all) {
+    s_w[tid] = m_raw;
+    s_d[tid] = d_raw;
+  }
+  for (int idx = tid; idx < kMfG * WM; idx += 1024) s_wm[idx] = 0.f;
+  for (int idx = tid; idx < G * D; idx += 1024) s_o[idx] = 0.f;
+  for (int idx = tid; idx < D; idx += 1024) s_own[idx] = 0;
+  __syncthreads();
+  // which dims this block writes: its list shares; block 0 also takes dims that no list names
+  if (own_dim >= 0) {
+    const bool c = tid < vc_len;
+    const int pos = c ? tid : tid - vc_len;
+    const bool mine = c ? (pos >= c_lo && pos < c_lo + cn) : (pos >= n_lo && pos < n_lo + nn);
+    s_own[own_dim] = mine ? 3 : 1;
+  }
+  if (wave < G) {
+    const int g = wave;
+    float mstar = -INFINITY;
+    for (int s_ = lane; s_ < n_all; s_ += 64) mstar = fmaxf(mstar, s_w[g * n_all + s_]);
+    mstar = fa_wave_max(mstar);
+    float dsum = 0.f, pmid = 0.f;
+    for (int s_ = lane; s_ < n_all; s_ += 64) {
+      const float m = s_w[g * n_all + s_];
+      const float wgt = m == -INFINITY ? 0.f : exp2f(m - mstar);
+      s_w[g * n_all + s_] = wgt;
+      if (s_ < n_il) {
+        dsum += wgt * s_d[g * n_all + s_];
+      } else {
+        pmid += wgt * s_d[g * n_all + s_];
+        s_wm[g * WM + (s_ - n_il)] = wgt;
+      }
+    }
+    dsum = fa_wave_sum(dsum);
+    pmid = fa_wave_sum(pmid);
+    if (lane == 0) {
+      s_sc[g] = dsum + pmid;
+      s_sc[kGMax + g] = pmid;
+    }
+  }
+  __syncthreads();
+
+  // ---- g summed over the splits, left as one row of the query heads' values per coefficient row ---------------
+  if (g_on) {
+    const float* wg = s_wm + g_of * WM;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fold = [&](const float4& v, float wt) {
+      acc.x = fmaf(wt, v.x, acc.x); acc.y = fmaf(wt, v.y, acc.y);
+      acc.z = fmaf(wt, v.z, acc.z); acc.w = fmaf(wt, v.w, acc.w);
+    };
+#pragma unroll
+    for (int u = 0; u < GPRE; u += 4) {
+      if (u < WM) {   // (splits past the head's count: the clamped loads meet a weight of zero)
+        const float4 w4 = *(const float4*)(wg + u);
+        fold(gv[u], w4.x); fold(gv[u + 1], w4.y); fold(gv[u + 2], w4.z); fold(gv[u + 3], w4.w);
+      }
+    }
+    for (int u = GPRE; u < n_mid; ++u) fold(*(const float4*)(gp + (int64_t)u * g_stride), wg[u]);
+    // {cos f, sin f, cos f+1, sin f+1} with f = 2 * n4
+    s_g[(2 * n4) * kMfG + g_of] = acc.x;
+    s_g[(N + 2 * n4) * kMfG + g_of] = acc.y;
+    s_g[(2 * n4 + 1) * kMfG + g_of] = acc.z;
+    s_g[(N + 2 * n4 + 1) * kMfG + g_of] = acc.w;
+  }
+  // The loads of the last two steps go out here: their results are not needed before the products below are done,
+  // and the registers of the g partials are free now.
+  // sink/window partial outputs: thread = (query head, four dims, split group); needs 2 G D <= 1024
+  const int QD = D >> 2;
+  const int il_sg = tid & 7, il_d4 = (tid >> 3) % QD, il_g = tid / (8 * QD);
+  const bool il_on = n_il > 0 && il_g < G;
+  const float* ip = nullptr;
+  float4 iv[kMfIlPre];
+  if (il_on) {
+    ip = a.il_o + (r0 + il_g) * n_il * D + 4 * il_d4;
+#pragma unroll
+    for (int u = 0; u < kMfIlPre; ++u) iv[u] = *(const float4*)(ip + (int64_t)min(il_sg + 8 * u, n_il - 1) * D);
+  }
+  // stored-dim partial outputs of the mid rows: thread = (query head, position in the share, split group), taken
+  // from the far end of the block so that they do not add to the loads of the sink/window threads
+  int SP = 16;
+  while (SP > 1 && G * nn * SP > 1024) SP >>= 1;
+  const int on_t = 1023 - tid;
+  const int on_sp = on_t & (SP - 1), on_j = (on_t / SP) % max(nn, 1), on_g = on_t / (SP * max(nn, 1));
+  const bool on_on = n_mid > 0 && nn > 0 && on_g < G;
+  const float* op = nullptr;
+  float ov[kMfOnPre];
+  int on_dim = 0;
+  if (on_on) {
+    op = a.md_on + (r0 + on_g) * a.n_mid_stride * D + n_lo + on_j;
+#pragma unroll
+    for (int u = 0; u < kMfOnPre; ++u) ov[u] = op[(int64_t)min(on_sp + SP * u, n_mid - 1) * D];
+    on_dim = a.vn_list[vn0 + n_lo + on_j] - h * D;
+  }
+  __syncthreads();
+
+  // ---- g . V_coef: rows of this thread's class, then the classes of the wave, then the waves ------------------
+  if (has_coef) {
+    float4 acc[kMfG];
+#pragma unroll
+    for (int g = 0; g < kMfG; ++g) acc[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto fma_row = [&](int n, const float4& v) {
+      const float4 gq = *(const float4*)(s_g + n * kMfG);
+      const float gg[kMfG] = {gq.x, gq.y, gq.z, gq.w};
+#pragma unroll
+      for (int g = 0; g < kMfG; ++g) {
+        acc[g].x = fmaf(gg[g], v.x, acc[g].x); acc[g].y = fmaf(gg[g], v.y, acc[g].y);
+        acc[g].z = fmaf(gg[g], v.z, acc[g].z); acc[g].w = fmaf(gg[g], v.w, acc[g].w);
+      }
+    };
+    if (v_on) {
+#pragma unroll
+      for (int u = 0; u < VPRE; ++u)
+        if (cls + u * classes < 2 * N) fma_row(cls + u * classes, vv[u]);
+      for (int n = cls + VPRE * classes; n < 2 * N; n += classes) fma_row(n, v_load(n));
+    }
+    // lanes q, q + nqp, q + 2 nqp, ... of the wave hold the same dims
+#pragma unroll
+    for (int g = 0; g < kMfG; ++g) {
+      if (g < G) {
+        const float4 v = fa_sum_lane_classes(acc[g], nqp);
+        if (lane < nqp) *(float4*)(s_part + (wave * kMfG + g) * CWP + 4 * lane) = v;
+      }
+    }
+    __syncthreads();
+    if (fin_on) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) s += s_part[(w * kMfG + fin_g) * CWP + fin_j];
+      s /= (float)N;
+      const float pmid = s_sc[kGMax + fin_g];
+      s_o[fin_g * D + fin_dim] = fin_scale * (s - fin_ad * pmid) + fin_au * pmid;
+    }
+  }
+  // stored dims of the mid rows
+  {
+    float s = 0.f;
+    if (on_on) {
+      const float* wg = s_w + on_g * n_all + n_il;
+#pragma unroll
+      for (int u = 0; u < kMfOnPre; ++u)
+        if (on_sp + SP * u < n_mid) s = fmaf(wg[on_sp + SP * u], ov[u], s);
+      for (int sp = on_sp + SP * kMfOnPre; sp < n_mid; sp += SP) s = fmaf(wg[sp], op[(int64_t)sp * D], s);
+    }
+    // (the split groups of an element are neighbouring lanes)
+    if (SP >= 2) s += fa_dpp<FA_DPP_XOR1>(s);
+    if (SP >= 4) s += fa_dpp<FA_DPP_XOR2>(s);
+    if (SP >= 8) s += fa_dpp<FA_DPP_HALF_MIRROR>(s);
+    if (SP >= 16) s += fa_dpp<FA_DPP_MIRROR>(s);
+    if (on_on && on_sp == 0) s_o[on_g * D + on_dim] = s;
+  }
+  __syncthreads();
+  // ---- sink/window rows, sum, normalisation ---------------------------------------------------------------------
+  {
+    float4 s4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (il_on) {
+      const float* wg = s_w + il_g * n_all;
+      auto fold = [&](const float4& v, float wt) {
+        s4.x = fmaf(wt, v.x, s4.x); s4.y = fmaf(wt, v.y, s4.y); s4.z = fmaf(wt, v.z, s4.z); s4.w = fmaf(wt, v.w, s4.w);
+      };
+#pragma unroll
+      for (int u = 0; u < kMfIlPre; ++u)
+        if (il_sg + 8 * u < n_il) fold(iv[u], wg[il_sg + 8 * u]);
+      for (int sp = il_sg + 8 * kMfIlPre; sp < n_il; sp += 8) fold(*(const float4*)(ip + (int64_t)sp * D), wg[sp]);
+    }
+    s4 = fa_dpp4_add<FA_DPP_XOR1>(s4);
+    s4 = fa_dpp4_add<FA_DPP_XOR2>(s4);
+    s4 = fa_dpp4_add<FA_DPP_HALF_MIRROR>(s4);
+    if (il_g < G && il_sg < 4) {   // lane il_sg writes dim 4 * il_d4 + il_sg
+      const int d = 4 * il_d4 + il_sg;
+      const int own = s_own[d];
+      if ((own & 2) || (z == 0 && own == 0)) {
+        const float mine = il_sg == 0 ? s4.x : il_sg == 1 ? s4.y : il_sg == 2 ? s4.z : s4.w;
+        put((r0 + il_g) * D + d, (s_o[il_g * D + d] + mine) / s_sc[il_g]);
+      }
+    }
+  }
+}
+
 
 // ---------------------------------------------------------------------------
 // sink + local window, vectorised (16-bit storage, head_dim 64 or 128, 16-byte aligned rows):
@@ -1615,7 +1936,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   // rows, 32 splits); up to 512 frequencies the blocks per share of dims below are as fast or 1 us faster
   if (p.path == Path::Mfma && p.n_mid_split > 0 && a.N >= 1024) {
     const int n_all = p.n_il_split + p.n_mid_split;
-    const size_t lds = (2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * kMrRows + (256 * (size_t)G > 1024 ? 256 * (size_t)G : 1024) +
+    const size_t lds = (2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * kMrRows + (512 * (size_t)G > 1024 ? 512 * (size_t)G : 1024) +
                         (size_t)G * a.D) * sizeof(float);
     MergeRowsArgs ma{};
     ma.il_m = ilm; ma.il_d = ild; ma.il_o = ilo; ma.n_il_split = p.n_il_split;
@@ -1628,6 +1949,26 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     ma.Hq = a.Hq; ma.Hkv = a.Hkv; ma.D = a.D; ma.N = a.N; ma.Cv = a.Cv; ma.nbpg = p.nbpg;
     ma.st = p.st;
     decode_merge_rows_kernel<<<dim3(p.n_row_blocks, a.Hkv, a.B), 256, lds, st>>>(ma);
+  } else if (p.path == Path::Mfma && p.n_mid_split > 0 && G <= kMfG && G * (a.N / 2) <= 1024 && a.N % 8 == 0 &&
+             a.D % 4 == 0 && 2 * G * a.D <= 1024 && a.D <= 128 * p.n_merge_chunks) {
+    const int n_all = p.n_il_split + p.n_mid_split;
+    int nqp = 1;
+    while (4 * nqp * p.n_merge_chunks < a.D) nqp <<= 1;   // the largest share of dims a head can have
+    const size_t lds = ((size_t)2 * a.N * kMfG + (size_t)kMfG * ((p.n_mid_split + 3) & ~3) + (size_t)16 * kMfG * 4 * nqp +
+                        2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * a.D + a.D) * sizeof(float);
+    FA_REQUIRE(lds <= 64 * 1024, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS for the merge", lds);
+    MergeRowsArgs ma{};
+    ma.il_m = ilm; ma.il_d = ild; ma.il_o = ilo; ma.n_il_split = p.n_il_split;
+    ma.md_m = mm; ma.md_d = md; ma.md_g = mg; ma.md_on = mon; ma.n_mid_stride = p.n_mid_split;
+    ma.v_mc = a.v_mc; ma.avg_u = a.avg_v_u; ma.avg_d = a.avg_v_d; ma.scale = a.scale_v;
+    ma.vc_list = a.vc_list; ma.vc_h = a.vc_h_list; ma.vn_list = a.vn_list; ma.vn_h = a.vn_h_list;
+    ma.out = a.out; ma.out_cast = a.out_cast; ma.cast_dtype = a.dtype;
+    ma.Hq = a.Hq; ma.Hkv = a.Hkv; ma.D = a.D; ma.N = a.N; ma.Cv = a.Cv; ma.nbpg = p.nbpg;
+    ma.st = p.st;
+    const dim3 grid(a.Hkv, a.B, p.n_merge_chunks);
+    // (with few splits the registers go to more rows of the V coefficients per thread instead)
+    if (p.n_mid_split <= 8) decode_merge_fast_kernel<8, 8><<<grid, 1024, lds, st>>>(ma);
+    else decode_merge_fast_kernel<16, 4><<<grid, 1024, lds, st>>>(ma);
   } else {
     const int n_all = p.n_il_split + p.n_mid_split;
     size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * n_all + 2 * kGMax + 1024 * (size_t)G + (size_t)G * a.D + a.D) * sizeof(float);
