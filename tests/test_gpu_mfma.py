@@ -197,6 +197,55 @@ def test_mfma_random_shapes_agree_with_the_generic_kernels():
             assert err <= 5e-3, (tag, err)
 
 
+
+def test_merge_for_few_query_heads_agrees_with_the_generic_kernels():
+    """The merge launch behind the matrix-core mid rows for up to four query heads per KV head and up to 512
+    frequencies (16-byte loads where a head's columns are aligned, single values otherwise; shares of the dims per
+    block): heads whose V dims are all compressed, all stored or none at all, odd totals of compressed dims (rows of
+    the coefficient tensor that are no multiple of 16 bytes), no sink rows, batches that do not fill a group, windows
+    long enough for more than one tile."""
+    from fourierattention_amd import DynamicCache
+    rng = np.random.default_rng(77)
+    fixed = [   # (D, Hkv, G, B, I, W, M, k dims compressed per head, v dims compressed per head)
+        (128, 2, 4, 5, 0, 3, 256, [64, 64], [128, 0]),
+        (128, 3, 3, 2, 4, 130, 512, [1, 127, 64], [1, 2, 3]),
+        (64, 4, 4, 9, 2, 64, 1024, [32, 32, 32, 32], [64, 64, 64, 64]),
+        (64, 1, 1, 1, 1, 1, 256, [64], [63]),
+        (128, 4, 2, 3, 4, 70, 1024, [60, 64, 68, 4], [4, 8, 12, 124]),
+    ]
+    cases = [(*f, torch.bfloat16) for f in fixed]
+    for _ in range(10):
+        D = [64, 128][rng.integers(2)]
+        Hkv = int(rng.integers(1, 5)); G = int(rng.integers(1, 5))
+        cases.append((D, Hkv, G, int(rng.integers(1, 10)), int(rng.integers(0, 6)), int(rng.integers(1, 200)),
+                      int([256, 512, 1024][rng.integers(3)]),
+                      [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)],
+                      [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)],
+                      [torch.bfloat16, torch.float16][rng.integers(2)]))
+    for case, (D, Hkv, G, B, I, W, M, kc, vc, dtype) in enumerate(cases):
+        Hq = Hkv * G
+        prompt = int(I + W + M + 40 + rng.integers(1, 1200))
+        tag = f"case {case}: {dtype} B={B} Hq={Hq} Hkv={Hkv} D={D} I={I} W={W} M={M} prompt={prompt} k={kc} v={vc}"
+        print(tag, flush=True)
+        masks = _masks(1, Hkv, D, kc, vc, seed=100 + case)
+        cfg = _cfg(masks, numinittokens=I, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=8,
+                   max_position_embeddings=1 << 20)
+        gpu = DynamicCache(cfg)
+        g = torch.Generator(device="cuda").manual_seed(1000 + case)
+        rn = lambda *sh: torch.randn(*sh, generator=g, device="cuda")
+        gpu.update(rn(B, Hkv, prompt, D).to(dtype), rn(B, Hkv, prompt, D).to(dtype), 0)
+        assert gpu._tables is not None, tag
+        gpu.update(rn(B, Hkv, 1, D).to(dtype), rn(B, Hkv, 1, D).to(dtype), 0)
+        q = (rn(B, Hq, 1, D) * 1.5).to(dtype)
+        got = gpu.decode_attention(q, 0, Hq, Hkv)
+        gpu.force_generic = True
+        ref = gpu.decode_attention(q, 0, Hq, Hkv)
+        gpu.force_generic = False
+        assert torch.isfinite(got).all(), tag
+        err = (got - ref).abs().max().item()
+        assert err <= 5e-3, (tag, err)
+
+
 def test_full_size_properties():
     """BASELINE config 3 at full size (B=8, 32k context): properties that need no CPU oracle.
     (1) the matrix-core path and the generic path (independent kernels, each checked against the oracle at
