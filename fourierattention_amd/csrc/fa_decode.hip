@@ -1819,6 +1819,19 @@ void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wid
     fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2><<<grid, 512, 0, st>>>(mp);
 }
 
+// bytes of LDS decode_merge_fast_kernel needs for this call, 0 where it does not apply (then decode_merge_kernel runs)
+static size_t merge_fast_lds(const fa_decode_args& a, const Plan& p, int G) {
+  const int n_all = p.n_il_split + p.n_mid_split;
+  if (p.path != Path::Mfma || p.n_mid_split <= 0 || G > kMfG || G * (a.N / 2) > 1024 || a.N % 8 != 0 || a.D % 4 != 0 ||
+      2 * G * a.D > 1024 || a.D > 128 * p.n_merge_chunks || G * n_all > 1024)
+    return 0;
+  int nqp = 1;
+  while (4 * nqp * p.n_merge_chunks < a.D) nqp <<= 1;   // the largest share of dims a head can have
+  const size_t lds = ((size_t)2 * a.N * kMfG + (size_t)kMfG * ((p.n_mid_split + 3) & ~3) + (size_t)16 * kMfG * 4 * nqp +
+                      2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * a.D + a.D) * sizeof(float);
+  return lds <= 64 * 1024 ? lds : 0;
+}
+
 // ev (optional): five events recorded before the first kernel and after each of prep (+ tables),
 // mid, sink/window and merge
 template <typename E>
@@ -1949,14 +1962,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     ma.Hq = a.Hq; ma.Hkv = a.Hkv; ma.D = a.D; ma.N = a.N; ma.Cv = a.Cv; ma.nbpg = p.nbpg;
     ma.st = p.st;
     decode_merge_rows_kernel<<<dim3(p.n_row_blocks, a.Hkv, a.B), 256, lds, st>>>(ma);
-  } else if (p.path == Path::Mfma && p.n_mid_split > 0 && G <= kMfG && G * (a.N / 2) <= 1024 && a.N % 8 == 0 &&
-             a.D % 4 == 0 && 2 * G * a.D <= 1024 && a.D <= 128 * p.n_merge_chunks) {
-    const int n_all = p.n_il_split + p.n_mid_split;
-    int nqp = 1;
-    while (4 * nqp * p.n_merge_chunks < a.D) nqp <<= 1;   // the largest share of dims a head can have
-    const size_t lds = ((size_t)2 * a.N * kMfG + (size_t)kMfG * ((p.n_mid_split + 3) & ~3) + (size_t)16 * kMfG * 4 * nqp +
-                        2 * (size_t)G * n_all + 2 * kGMax + (size_t)G * a.D + a.D) * sizeof(float);
-    FA_REQUIRE(lds <= 64 * 1024, FA_ERR_UNSUPPORTED, "fa_decode_attn: %zu bytes of LDS for the merge", lds);
+  } else if (merge_fast_lds(a, p, G) > 0) {
+    const size_t lds = merge_fast_lds(a, p, G);
     MergeRowsArgs ma{};
     ma.il_m = ilm; ma.il_d = ild; ma.il_o = ilo; ma.n_il_split = p.n_il_split;
     ma.md_m = mm; ma.md_d = md; ma.md_g = mg; ma.md_on = mon; ma.n_mid_stride = p.n_mid_split;

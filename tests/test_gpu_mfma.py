@@ -203,7 +203,7 @@ def test_merge_for_few_query_heads_agrees_with_the_generic_kernels():
     frequencies (16-byte loads where a head's columns are aligned, single values otherwise; shares of the dims per
     block): heads whose V dims are all compressed, all stored or none at all, odd totals of compressed dims (rows of
     the coefficient tensor that are no multiple of 16 bytes), no sink rows, batches that do not fill a group, windows
-    long enough for more than one tile."""
+    of one tile, of many tiles, and of more tiles than that kernel takes (the general merge kernel runs then)."""
     from fourierattention_amd import DynamicCache
     rng = np.random.default_rng(77)
     fixed = [   # (D, Hkv, G, B, I, W, M, k dims compressed per head, v dims compressed per head)
@@ -212,6 +212,8 @@ def test_merge_for_few_query_heads_agrees_with_the_generic_kernels():
         (64, 4, 4, 9, 2, 64, 1024, [32, 32, 32, 32], [64, 64, 64, 64]),
         (64, 1, 1, 1, 1, 1, 256, [64], [63]),
         (128, 4, 2, 3, 4, 70, 1024, [60, 64, 68, 4], [4, 8, 12, 124]),
+        (128, 2, 4, 2, 4, 8200, 512, [64, 64], [64, 60]),      # 129 sink/window tiles: more than are requested ahead
+        (128, 1, 4, 1, 4, 20000, 512, [64], [64]),             # more split weights than the kernel has threads for
     ]
     cases = [(*f, torch.bfloat16) for f in fixed]
     for _ in range(10):
