@@ -1803,10 +1803,10 @@ void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bo
   dim3 grid(p.n_wg, p.n_groups);
   if (wide) {
     fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 2><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2><<<grid, 512, 0, st>>>(mp);
   } else {
     fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 1><<<grid, 512, 0, st>>>(mp);
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 2><<<grid, 512, 0, st>>>(mp);
+    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2><<<grid, 512, 0, st>>>(mp);
   }
 }
 

@@ -277,10 +277,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   using M = Mma<E>;
   using vec8 = typename M::vec8;
   constexpr int kFragsMax = (2 * KMAX > VMAX ? 2 * KMAX : VMAX);   // fragments (1 KiB) of one page of one wave
-  static_assert(MODE == 0 || NST == 2, "the passes wait for every outstanding load at the top of a page");
   // in the two-pass modes only waves 0-3 stream pages
+  static_assert(MODE != 1 || NST == 2, "the score pass waits for every outstanding access at the top of a page");
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[MODE == 0 ? 8 : 4][NST][kFragsMax * 1024];
   __shared__ float s_part[MODE == 2 ? 1 : 2][MODE == 2 ? 1 : NSL][16 * kPart];
+  // value pass: the scores of a page travel like its V fragments, memory -> LDS without registers, every wave its own
+  // copy (two fragments: positions 8 lg .. 8 lg + 3 and 8 lg + 4 .. 8 lg + 7 of column lc at lane * 16), so that
+  // the only accesses to vector memory inside the loop are page requests, whose arrival can be counted
+  __shared__ __attribute__((aligned(16))) unsigned char s_sc[MODE == 2 ? 8 : 1][MODE == 2 ? NST : 1][MODE == 2 ? 2048 : 16];
   // frame-to-frame rotation constants, float4 = (c, s) of two neighbouring frequencies, [slice][unit][lane group]:
   // for the score waves unit = row tile rt, frequencies freq_of(rt, lg, 0 / 1); for the value waves unit u covers
   // the frequencies 16 (u / 2) + 4 lg + 2 (u % 2) + 0 / 1, the rows 4 lg + 2 (u % 2) + 0 / 1 of tile pair u / 2
@@ -586,11 +590,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     half8 ETa[2 * KS];   // tile 2j: cosines, tile 2j + 1: sines of the frequencies 16j .. 16j + 15 of the slice
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
-    if (streams_v) {   // first pages requested behind the table (see the score waves)
+    // value pass: the scores of page pgi of the split, into this wave's stage of that page
+    auto issue_sc = [&](int pgi) {
+      if constexpr (MODE == 2) {
+        const float* src = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pgi) * 512 + lc * 32 + 8 * lg;
+        unsigned char* st = &s_sc[w][pgi % NST][0];
+        load_frag_to_lds<0>(src, st);
+        load_frag_to_lds<0>(src + 4, st + 1024);
+      }
+    };
+    // first pages requested behind the table (see the score waves); page by page, so that the requests of a page
+    // sit together in the order of arrival
 #pragma unroll
-      for (int i = 0; i < NST - 1; ++i)
-        if (i < n_it) issue_v(t_beg + i, (i & 1) == 0);
-    }
+    for (int i = 0; i < NST - 1; ++i)
+      if (i < n_it) {
+        if (streams_v) issue_v(t_beg + i, (i & 1) == 0);
+        issue_sc(i);
+      }
     rot_store();
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
@@ -604,16 +620,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) asm volatile("" ::"v"(ETa[rt]));
     const unsigned rot_lane = lds_addr_of(&s_rotv[(MODE == 1 ? 0 : sl * 2 * KS) * 4 + lg]);
-    // value pass: the scores of a page (column lc, positions 8*lg .. 8*lg+7) are fetched one page ahead
-    float4v sc_next[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
-    const float* sc_src = nullptr;
-    if constexpr (MODE == 2) {
-      sc_src = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg) * 512 + lc * 32 + 8 * lg;
-      if (n_it > 0) {
-        sc_next[0] = *(const float4v*)sc_src;
-        sc_next[1] = *(const float4v*)(sc_src + 4);
-      }
-    }
 
     // The probabilities of the first (mirrored) page of a frame wait here for the second page: the tokens at the
     // offsets -(i + 1/2) and +(i + 1/2) meet the same cosine and, with opposite signs, the same sine, so g of the frame
@@ -636,24 +642,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         float sc[8];
         if constexpr (MODE == 2) {
-          // taken before the next page is requested: a wait placed here by the compiler then covers loads that
-          // have had a whole page to land, and nothing that was issued a moment ago
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            sc[e] = sc_next[e >> 2][e & 3];
-            asm volatile("" : "+v"(sc[e]));
+          // a page of this wave is its V fragments (if it streams V) and its two fragments of scores
+          if (pg + NST - 2 < n_it) wait_pages_in_flight<NST - 2, VMAX + 2, 1>((has_v ? ndg : 0) + 2);
+          else wait_vmcnt<0>();
+          // refills the stages read one page ago
+          if (pg + NST - 1 < n_it) {
+            if constexpr (has_v) issue_v(t + NST - 1, first_of_frame == (((NST - 1) & 1) == 0));
+            issue_sc(pg + NST - 1);
           }
-        }
-        if constexpr (has_v) {
+        } else if constexpr (has_v) {
           if (pg + NST - 2 < n_it) wait_pages_in_flight<NST - 2, VMAX, 1>(ndg);
           else wait_vmcnt<0>();
           // refills the stage read one page ago
           if (pg + NST - 1 < n_it) issue_v(t + NST - 1, first_of_frame == (((NST - 1) & 1) == 0));
-        }
-        if constexpr (MODE == 2) {
-          const float* nx = sc_src + (int64_t)min(pg + 1, n_it - 1) * 512;   // clamped: the load is unconditional
-          sc_next[0] = *(const float4v*)nx;
-          sc_next[1] = *(const float4v*)(nx + 4);
         }
         // the g history moves into the frame of this pair of pages: unit u of the constants belongs to the rows
         // 2 (u % 2) + f2 of the cosine tile 2 (u / 2) and of the sine tile behind it
@@ -694,6 +695,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     (__builtin_bit_cast(float, u2) + __builtin_bit_cast(float, u3));
           }
         }
+        uint4v sraw[2];   // value pass: the scores of the page, column lc, positions 8*lg .. 8*lg + 7
+        if constexpr (MODE == 2) {
+          const unsigned sst = lds_addr_of(&s_sc[w][pg % NST][0]) + lane * 16;
+          sraw[0] = lds_read_b128_async_at<0>(sst);
+          sraw[1] = lds_read_b128_async_at<1024>(sst);
+        }
         uint4v vraw[4];   // four dim groups at a time
         const unsigned vst = lds_addr_of(&s_stage[MODE == 0 ? w : stw][pg % NST][0]) + lane * 16;
         if constexpr (has_v) {
@@ -701,6 +708,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           vraw[1] = lds_read_b128_async_at<1024>(vst);
           vraw[2] = lds_read_b128_async_at<2048>(vst);
           vraw[3] = lds_read_b128_async_at<3072>(vst);
+        }
+        if constexpr (MODE == 2) {
+          if constexpr (has_v) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(sraw[0]), "+v"(sraw[1])::"memory");
+          else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sraw[0]), "+v"(sraw[1])::"memory");
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const uint4v r = sraw[e >> 2];
+            const unsigned u = r[e & 3];
+            sc[e] = __builtin_bit_cast(float, u);
+          }
         }
         if (ragged_tail && t == n_tiles - 1) {
 #pragma unroll
