@@ -115,16 +115,17 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
     const int grp = b / pa.nbpg, sl = b - grp * pa.nbpg;
     const int g = lc - sl * G;   // the column's query head if the column is this batch element's
     const bool mine = g >= 0 && g < G;
-    const E* qr = q + ((int64_t)b * Hq + h * G + (mine ? g : 0)) * D - h * D;
-    union { E e[8]; uint4 raw; } o;
+    if (kn_len > 0) {   // (a head that stores no K dims has no entries in the list and nobody reads its operands)
+      const E* qr = q + ((int64_t)b * Hq + h * G + (mine ? g : 0)) * D - h * D;
+      union { E e[8]; uint4 raw; } o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = s * 32 + 8 * lg + e;
-      const E qv = qr[pa.kn_list[kn0 + min(j, max(kn_len - 1, 0))]];   // clamped: no load under a condition
-      o.e[e] = (mine && j < kn_len) ? qv : E();
-    }
-    if (kn_len > 0)
+      for (int e = 0; e < 8; ++e) {
+        const int j = s * 32 + 8 * lg + e;
+        const E qv = qr[pa.kn_list[kn0 + min(j, kn_len - 1)]];   // clamped: no load under a per-lane condition
+        o.e[e] = (mine && j < kn_len) ? qv : E();
+      }
       *(uint4*)(pa.q_stored + ((((int64_t)(grp * Hkv + h) * 4 + sl) * 4 + s) * 64 + lane) * 8) = o.raw;
+    }
   }
   const int n = bx * kPrepRows + (tid >> 2), jq = tid & 3;
   if (n >= 2 * N) return;
