@@ -107,3 +107,33 @@ def test_two_calls_with_1024_frequencies():
         assert got is out and torch.equal(got, ref)
         err = np.abs(got.cpu().numpy() - want).max()
         assert err <= 2e-3, err
+
+
+@pytest.mark.gpu
+def test_captured_in_a_graph_and_replayed():
+    """``fa_decode_attn_noalloc`` recorded into a graph (no allocation, no clearing of memory by the runtime: the
+    counters of the merge are cleared by the launch in front of it) and replayed on new queries in the same buffers:
+    every replay bit for bit what the eager call returns."""
+    Hq, Hkv, D = 8, 2, 128
+    for M, prompt in ((512, 2000), (2048, 4300)):     # the fused mid rows / the two passes of 1024 frequencies
+        gpu, q, want = _cache_case(torch.bfloat16, 3, Hq, Hkv, D, 64, M, prompt, [64, 40], [64, 96], seed=5)
+        gpu.balance_heads = False
+        ref = gpu.decode_attention(q, 0, Hq, Hkv)
+        out = torch.full_like(ref, float("nan"))
+        qbuf = q.clone()
+        # first call outside the capture: the address of the built-in buffer is looked up once per device
+        assert torch.equal(gpu.decode_attention(qbuf, 0, Hq, Hkv, out=out, no_alloc=True), ref)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            gpu.decode_attention(qbuf, 0, Hq, Hkv, out=out, no_alloc=True)
+        gen = torch.Generator(device="cuda").manual_seed(7)
+        for _ in range(3):
+            qk = (torch.randn(q.shape, generator=gen, device="cuda") * 1.5).to(q.dtype)
+            eager = gpu.decode_attention(qk, 0, Hq, Hkv)
+            qbuf.copy_(qk)
+            out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
