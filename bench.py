@@ -385,6 +385,9 @@ def main():
     ap.add_argument("--even-splits", action="store_true",
                     help="give every KV head the same number of splits of the mid rows (default: heads that store more dims "
                          "get more; no difference with a uniform mask)")
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="run sink/window tiles, mid rows and merge as launches of their own where the library would run the "
+                         "merge inside the mid-row launch (for comparison)")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
                     help="run the end-to-end decode of a random-init model instead (its own JSON line); --steps caps the "
                          "number of timed tokens per sequence")
@@ -432,6 +435,7 @@ def main():
             sys.exit(1)
     cache, q, kn, vn = build_cache(w, dtype, device)
     cache.balance_heads = not args.even_splits
+    cache.fuse_decode = not args.no_fuse
     Hq, Hkv = w["Hq"], w["Hkv"]
     for _ in range(args.warmup):
         out = cache.decode_attention(q, 0, Hq, Hkv)
@@ -460,18 +464,22 @@ def main():
         cache.decode_attention(q, 0, Hq, Hkv, timings=tm)
         per += np.array(tm)
     per /= reps
+    merge_in_mid_rows = bool(_lib.load().fa_decode_attn_last_fused())
     # three launches: the coefficient-domain query shares one with the sink/window tiles (the third slot is the
     # gap left between the event pairs, a few microseconds of event overhead)
-    kernel_ms = {"query_and_sink_window": per[0] + per[2], "mid_rows": per[1], "merge": per[3]}
+    # (with the merge inside the mid-row launch the step has two launches and the last slot is event overhead only)
+    kernel_ms = {"query_and_sink_window": per[0] + per[2], "mid_rows_and_merge" if merge_in_mid_rows else "mid_rows": per[1],
+                 "merge": per[3]}
     # algorithmic bytes of each kernel's own launch
     kbytes = {
         "query_and_sink_window": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4 + w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,
         "mid_rows": w["B"] * L * (2 * hd - ck - cv) * 2,
+        "mid_rows_and_merge": w["B"] * L * (2 * hd - ck - cv) * 2 + w["B"] * w["M"] * cv * 4,
         "merge": w["B"] * w["M"] * cv * 4,
     }
     dom = max(kernel_ms, key=kernel_ms.get)
     dom_gbs = kbytes[dom] / (kernel_ms[dom] * 1e-3) / 1e9
-    traffic, traffic_source = recorded_traffic(dom, args.workload)
+    traffic, traffic_source = recorded_traffic("mid_rows" if dom.startswith("mid_rows") else dom, args.workload)
     full = 2 * w["ctx"] * hd * 2
     fourier = 2 * (w["I"] + w["W"]) * hd * 2 + L * (2 * hd - ck - cv) * 2 + w["M"] * (ck + cv) * 4
     result = {
@@ -490,6 +498,7 @@ def main():
         "parity_max_abs_err": parity,
         "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
         "kernel_ms": {k: round(float(v), 5) for k, v in kernel_ms.items()},
+        "merge_inside_mid_row_launch": merge_in_mid_rows,
         # each launch of kernel_ms sits between its own pair of HIP events; the pairs cost a few microseconds each,
         # which is why the three figures add up to more than ms_per_step (timed without events inside)
         "event_overhead_ms": round(float(sum(kernel_ms.values())) - ms, 5),

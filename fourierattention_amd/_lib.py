@@ -56,6 +56,7 @@ class DecodeArgs(ctypes.Structure):
         ("q_len", c_int32), ("N", c_int32), ("L_m", c_int32), ("T", c_int32),
         ("sm_scale", c_float), ("dtype", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("no_fuse", c_int32),
     ]
 
 
@@ -98,6 +99,7 @@ _SIGNATURES = {
     "fa_decode_attn": (c_int, [POINTER(DecodeArgs), c_void_p]),
     "fa_decode_attn_noalloc": (c_int, [POINTER(DecodeArgs), c_void_p]),
     "fa_decode_attn_timed": (c_int, [POINTER(DecodeArgs), c_void_p, POINTER(c_float)]),
+    "fa_decode_attn_last_fused": (c_int, []),
     "fa_linear_pack": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "fa_linear_packed_ok": (c_int, [c_int, c_int, c_int]),
     "fa_linear_packed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -126,6 +128,9 @@ _SIGNATURES = {
 
 EXPORTED = tuple(_SIGNATURES)
 
+# bumped with every change of a prototype or of an argument struct (fa_abi_version in the library)
+ABI_VERSION = 2
+
 _lib = None
 
 
@@ -143,6 +148,9 @@ def load():
         fn = getattr(lib, name)  # AttributeError if the library does not export it
         fn.restype = res
         fn.argtypes = args
+    if lib.fa_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has ABI version {lib.fa_abi_version()}, this binding was written for {ABI_VERSION}: "
+                          "rebuild the library (`python -m fourierattention_amd.build`)")
     if lib.fa_stream_args_size() != ctypes.sizeof(StreamArgs):
         raise ImportError(f"fa_stream_args is {lib.fa_stream_args_size()} bytes in the library but "
                           f"{ctypes.sizeof(StreamArgs)} in the Python mirror")

@@ -9,6 +9,7 @@
 // per-token reconstruction, and the token loop only touches the stored dims.
 // All exponentials are base 2 (scores carry log2(e)).
 #include <stdlib.h>
+#include <string.h>
 
 #include "fa_common.h"
 #include <mutex>
@@ -20,6 +21,9 @@ constexpr int kGMax = 8;      // query heads per KV head handled by the generic 
 constexpr int kTile = 256;    // tokens per tile = threads per block
 constexpr int kFreqIters = 4; // frequencies per thread in the g accumulation (N <= 1024)
 constexpr float kLog2e = 1.4426950408889634f;
+// fused step: how long a workgroup waits for the rest of its team before it gives up and writes NaN rows, in ticks
+// of the 100 MHz wall clock (0.2 s; the wait normally lasts a few microseconds)
+constexpr unsigned kTeamWaitTicks = 20u * 1000u * 1000u;
 
 struct Seg {
   const void* k;
@@ -63,6 +67,8 @@ struct PrepArgs {
   E* q_stored;
   const int32_t* kn_list;
   const int32_t* kn_h;
+  // fused step: the two meeting counters of every (batch group, KV head), cleared here for the launch behind
+  unsigned* team_cnt;
 };
 
 // LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head
@@ -103,6 +109,7 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
     s_qa[g][j] = qa;
   }
   __syncthreads();
+  if (bx == 0 && tid < 2 && pa.team_cnt && b % pa.nbpg == 0) pa.team_cnt[((int64_t)(b / pa.nbpg) * Hkv + h) * 2 + tid] = 0u;
   if (bx == 0 && tid < 64) {
     for (int g = 0; g < G; ++g) {
       float v = fa_wave_sum(s_qa[g][tid] + s_qa[g][tid + 64]);
@@ -1446,22 +1453,6 @@ struct IlArgs {
   float sm_log2e;
 };
 
-// a . b of two pairs of 16-bit values plus c, in one instruction
-typedef __bf16 fa_bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 fa_f16x2 __attribute__((ext_vector_type(2)));
-template <typename E>
-__device__ __forceinline__ float fa_dot2(unsigned a, unsigned b, float c);
-template <>
-__device__ __forceinline__ float fa_dot2<bf16_t>(unsigned a, unsigned b, float c) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(fa_bf16x2, a), __builtin_bit_cast(fa_bf16x2, b), c, false);
-}
-template <>
-__device__ __forceinline__ float fa_dot2<f16_t>(unsigned a, unsigned b, float c) {
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(fa_f16x2, a), __builtin_bit_cast(fa_f16x2, b), c, false);
-}
-template <>
-__device__ __forceinline__ float fa_dot2<float>(unsigned, unsigned, float c) { return c; }   // never run: 16-bit rows only
-
 // LDS of a sink/window block: the four waves' maxima, denominators and outputs meet here
 template <int D, int GM>
 struct IlFastLds {
@@ -1723,7 +1714,9 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     p.n_groups = fa_cdiv(B, p.nbpg);
     p.ks = N / (16 * fa_mfma::table_slices(N));
     const int tiles = fa_cdiv(L_m, 32);
+    // one workgroup per compute unit; rounded down where rounding up would leave a second round of a few workgroups
     int want = fa_cdiv(device_cu_count(), (int64_t)Hkv * p.n_groups);
+    if ((int64_t)want * Hkv * p.n_groups > device_cu_count() && want > 1) --want;
     if (want < 1) want = 1;
     int ns = tiles < want ? tiles : want;
     p.tiles_per_split = ns > 0 ? fa_cdiv(tiles, ns) : 0;
@@ -1768,10 +1761,14 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   // two-pass mid rows (eight frequency slices): the scores of every page travel through memory
   p.off_scores = take(mfma && fa_mfma::table_slices(N) > 4 ? (size_t)p.n_groups * Hkv * fa_cdiv(L_m, 32) * 512 * 4 : 0);
   p.n_row_blocks = mfma ? N / (kMrTiles * 8) : 0;
-  p.off_pc = take(mfma ? (size_t)B * Hkv * p.n_row_blocks * (Hq / Hkv) * 128 * 4 : 0);
+  {
+    const size_t by_rows = (size_t)B * Hkv * p.n_row_blocks * (Hq / Hkv) * 128 * 4;
+    const size_t by_team = (size_t)p.n_groups * Hkv * p.n_mid_split * 16 * 128 * 4;   // fused step
+    p.off_pc = take(mfma ? (by_rows > by_team ? by_rows : by_team) : 0);
+  }
   p.off_sil = take(mfma ? rows * D * 4 : 0);
   p.off_son = take(mfma ? rows * D * 4 : 0);
-  p.off_cnt = take(mfma ? (size_t)B * Hkv * 4 : 0);
+  p.off_cnt = take(mfma ? ((size_t)B * Hkv + (size_t)p.n_groups * Hkv * 2) * 4 : 0);
   p.off_qn = take(mfma ? (size_t)p.n_groups * Hkv * 4 * 4 * 64 * 16 : 0);
   p.total = o;
   return p;
@@ -1812,12 +1809,97 @@ void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bo
 }
 
 template <typename E, int KS>
-void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
+void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, hipStream_t st) {
   dim3 grid(p.n_wg, p.n_groups);
-  if (wide)
+  if (fused) {
+    grid = dim3(p.n_wg * p.n_groups);   // numbered through wg_map
+    if (wide)
+      fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true><<<grid, 512, 0, st>>>(mp);
+    else
+      fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true><<<grid, 512, 0, st>>>(mp);
+  } else if (wide) {
     fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2><<<grid, 512, 0, st>>>(mp);
-  else
+  } else {
     fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2><<<grid, 512, 0, st>>>(mp);
+  }
+}
+
+// The fused merge relies on the workgroups of a launch being dealt out to the dies in turn (workgroup L on die
+// L % 8).  Checked once per device by a launch of the same shape that records the die of every workgroup; a device
+// (or partition mode) that deals them out differently keeps the merge in a launch of its own.
+static __device__ unsigned xcc_probe_out[fa_mfma::kFusedMaxWgs];
+__global__ __launch_bounds__(512) void xcc_probe_kernel(unsigned* out) {
+  if (threadIdx.x == 0) out[blockIdx.x] = fa_mfma::xcc_id();
+}
+bool fused_layout_ok(hipStream_t st) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static int known[kMaxDevices] = {};   // 0: not probed, 1: in turn, -1: not
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+  std::lock_guard<std::mutex> lock(mu);
+  if (known[dev] != 0) return known[dev] > 0;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return false;   // (ask again later)
+  void* out = nullptr;
+  unsigned host[fa_mfma::kFusedMaxWgs];
+  bool ok = hipGetSymbolAddress(&out, HIP_SYMBOL(xcc_probe_out)) == hipSuccess && out;
+  if (ok) {
+    xcc_probe_kernel<<<fa_mfma::kFusedMaxWgs, 512, 0, st>>>((unsigned*)out);
+    ok = hipMemcpyAsync(host, out, sizeof(host), hipMemcpyDeviceToHost, st) == hipSuccess &&
+         hipStreamSynchronize(st) == hipSuccess;
+  }
+  for (int l = 0; ok && l < fa_mfma::kFusedMaxWgs; ++l) ok = host[l] == host[l % fa_mfma::kFusedXcds];
+  for (int i = 0; ok && i < fa_mfma::kFusedXcds; ++i)
+    for (int j = 0; j < i; ++j) ok = ok && host[i] != host[j];
+  known[dev] = ok ? 1 : -1;
+  return ok;
+}
+
+thread_local int g_last_call_fused = 0;   // what the last fa_decode_attn call of this thread did (a measurement aid)
+
+// Whether the merge can run inside the mid-row launch (fa_decode_fused.h): the one-pass matrix-core pipeline, heads
+// of 128 dims with at most four query heads per KV head, every workgroup of the launch resident at once (the
+// workgroups of a team wait for each other), and the teams dealt out so that each sits on one die.  Fills wg_map.
+bool fused_merge_plan(const fa_decode_args& a, const Plan& p, uint16_t* wg_map, hipStream_t st) {
+  using namespace fa_mfma;
+  if (p.path != Path::Mfma || a.no_fuse || p.n_mid_split <= 0) return false;
+  if (table_slices(a.N) != 4 || a.D != kFusedD || a.Hq / a.Hkv > kFusedG) return false;
+  if (a.dtype != FA_BF16 && a.dtype != FA_FP16) return false;
+  const int total = p.n_wg * p.n_groups, n_teams = p.n_groups * a.Hkv;
+  if (total > device_cu_count() || total > kFusedMaxWgs || total % kFusedXcds != 0 || n_teams > (1 << (16 - kFusedSplitBits)))
+    return false;
+  if (p.n_mid_split + p.n_il_split > kFusedMaxParts || p.n_mid_split >= (1 << kFusedSplitBits)) return false;
+  // a workgroup finishes ceil(R / splits) columns of its team's R = nb * G: they must belong to one batch element
+  {
+    const int G = a.Hq / a.Hkv;
+    for (int h = 0; h < a.Hkv; ++h)
+      for (int nb = p.nbpg; nb > 0; nb = (nb == p.nbpg && a.B % p.nbpg) ? a.B % p.nbpg : 0) {   // full groups, the last one
+        const int per = fa_cdiv(nb * G, p.st.n[h]);
+        if (per > G || G % per != 0) return false;
+      }
+  }
+  if (!fused_layout_ok(st)) return false;
+  // Workgroup L of the launch runs on die L % 8.  Teams are placed largest first into the die with room; the
+  // workgroups of die c are L = c, c + 8, c + 16, ...
+  const int cap = total / kFusedXcds;
+  int order[kFusedMaxWgs], fill[kFusedXcds] = {};
+  for (int t = 0; t < n_teams; ++t) order[t] = t;
+  auto size_of = [&](int t) { return p.st.n[t % a.Hkv]; };
+  for (int i = 1; i < n_teams; ++i)   // insertion sort by size, descending, stable
+    for (int j = i; j > 0 && size_of(order[j]) > size_of(order[j - 1]); --j) {
+      const int tmp = order[j]; order[j] = order[j - 1]; order[j - 1] = tmp;
+    }
+  for (int i = 0; i < n_teams; ++i) {
+    const int t = order[i], n = size_of(t);
+    if (n <= 0) return false;
+    int c = 0;
+    while (c < kFusedXcds && fill[c] + n > cap) ++c;
+    if (c == kFusedXcds) return false;
+    for (int s = 0; s < n; ++s) wg_map[kFusedXcds * (fill[c] + s) + c] = (uint16_t)((t << kFusedSplitBits) | s);
+    fill[c] += n;
+  }
+  return true;
 }
 
 // bytes of LDS decode_merge_fast_kernel needs for this call, 0 where it does not apply (then decode_merge_kernel runs)
@@ -1855,11 +1937,16 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   IlArgs<E> ia{(const E*)a.q, s0, s1, ilm, ild, ilo, a.Hq, a.Hkv, p.n_il_split, sm_log2e};
   // sink/window tiles ride in the query-preparation launch when both exist and the fast tile kernel applies
   const bool fuse_il = sizeof(E) == 2 && p_il_fast && p.n_il_split > 0 && p.n_mid_split > 0;
+  uint16_t wg_map[fa_mfma::kFusedMaxWgs] = {};
+  // (the sink/window tiles must be in front of the mid rows for the merge to run inside that launch)
+  const bool fused = sizeof(E) == 2 && (fuse_il || p.n_il_split == 0) && fused_merge_plan(a, p, wg_map, st);
+  g_last_call_fused = fused ? 1 : 0;
   if (p.n_mid_split > 0) {
     PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
                    a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e,
                    p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks,
-                   p.path == Path::Mfma ? (E*)(ws + p.off_qn) : nullptr, a.kn_list, a.kn_h_list};
+                   p.path == Path::Mfma ? (E*)(ws + p.off_qn) : nullptr, a.kn_list, a.kn_h_list,
+                   fused ? (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv : nullptr};
     const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
@@ -1890,7 +1977,18 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.rot = (const float2v*)(mp.tabET + NSL * 2 * KS * 64);
         mp.pm = mm; mp.pd = md; mp.pg = mg; mp.pon = mon;
         mp.scores = (float*)(ws + p.off_scores);
-        mp.merge_count = (unsigned*)(ws + p.off_cnt);
+        mp.merge_count = fused ? nullptr : (unsigned*)(ws + p.off_cnt);
+        if (fused) {
+          auto& fz = mp.fz;
+          fz.il_m = ilm; fz.il_d = ild; fz.il_o = ilo; fz.n_il = p.n_il_split;
+          fz.part_c = (float*)(ws + p.off_pc); fz.stage_il = (float*)(ws + p.off_sil); fz.stage_on = (float*)(ws + p.off_son);
+          fz.cnt = (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv;
+          fz.v_mc = a.v_mc; fz.avg_u = a.avg_v_u; fz.avg_d = a.avg_v_d; fz.scale = a.scale_v;
+          fz.vc_list = a.vc_list; fz.vc_h = a.vc_h_list; fz.vn_list = a.vn_list;
+          fz.out = a.out; fz.out_cast = (E*)a.out_cast; fz.Cv = a.Cv;
+          fz.wait_ticks = kTeamWaitTicks;
+          memcpy(fz.wg_map, wg_map, sizeof(wg_map));
+        }
         mp.q_stored = (const E*)(ws + p.off_qn);
         mp.B = a.B; mp.Hq = a.Hq; mp.Hkv = a.Hkv; mp.D = a.D; mp.G = G; mp.nbpg = p.nbpg; mp.N = a.N;
         mp.L_m = a.L_m; mp.T = a.T; mp.n_split = p.n_mid_split; mp.st = p.st;
@@ -1899,9 +1997,9 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
         if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, st);
         else switch (KS) {
-          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, st); break;
-          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, st); break;
-          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, st); break;
+          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, fused, st); break;
+          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, fused, st); break;
+          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, fused, st); break;
         }
       }
     } else {
@@ -1928,6 +2026,13 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   }
   if (ev && (p.n_mid_split == 0 || p.path != Path::Mfma)) hipEventRecord(ev[1], st);
   if (ev) hipEventRecord(ev[2], st);
+  if (fused) {   // the launch above has written the output rows
+    if (ev) {
+      hipEventRecord(ev[3], st);
+      hipEventRecord(ev[4], st);
+    }
+    return fa_check_launch("fa_decode_attn");
+  }
   if (p.n_il_split > 0 && !fuse_il) {
     dim3 grid(p.n_il_split, a.Hkv, a.B);
     bool launched = false;
@@ -2155,6 +2260,8 @@ extern "C" int fa_decode_attn_noalloc(const fa_decode_args* a, fa_stream_t strea
   b.workspace_bytes = (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES;
   return decode_attn_impl(&b, stream, nullptr);
 }
+
+extern "C" int fa_decode_attn_last_fused(void) { return g_last_call_fused; }
 
 extern "C" int fa_decode_attn_timed(const fa_decode_args* a, fa_stream_t stream, float* ms_out) {
   FA_REQUIRE(ms_out, FA_ERR_NULL_POINTER, "fa_decode_attn_timed: ms_out null");

@@ -33,6 +33,7 @@
 #pragma once
 
 #include "fa_mfma_util.h"
+#include "fa_decode_fused.h"
 #include <type_traits>
 
 namespace fa_mfma {
@@ -249,6 +250,7 @@ struct MidParams {
   int n_split;   // splits the partial buffers have room for per head (the largest n[h])
   float sm_log2e;
   SplitTable st;
+  FusedParams<E> fz;   // the fused merge only (FUSE instances of the kernel)
 };
 
 // The workgroup is a two-stage pipeline over the pages of its split, one barrier per page:
@@ -270,9 +272,12 @@ struct MidParams {
 //         memory (2 KiB per page and workgroup, against 16 KiB of K/V);
 // MODE 2, values: every wave reads the page's scores back, runs the softmax and keeps its slice of the g
 //         history; waves 0-3 stream V.  No exchange between the waves at all.
-template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0>
+// FUSE (MODE 0 only): the launch merges its own partials and writes the output rows, see fa_decode_fused.h; the
+// workgroups are then numbered through p.fz.wg_map so that the splits of a (batch group, KV head) share one die.
+template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
+  static_assert(!FUSE || MODE == 0, "the fused merge runs behind the one-pass pipeline");
   constexpr int NSL = MODE == 0 ? kFreqWaves : 2 * kFreqWaves;   // frequency slices
   using M = Mma<E>;
   using vec8 = typename M::vec8;
@@ -290,21 +295,28 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // the frequencies 16 (u / 2) + 4 lg + 2 (u % 2) + 0 / 1, the rows 4 lg + 2 (u % 2) + 0 / 1 of tile pair u / 2
   __shared__ float4v s_rot[MODE == 2 ? 1 : NSL * 2 * KS * 4];
   __shared__ float4v s_rotv[MODE == 1 ? 1 : NSL * 2 * KS * 4];
-
+  __shared__ int s_team_flag;
   const int tid = threadIdx.x, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps role and page addressing scalar
   const bool score_wave = MODE == 0 ? w < kFreqWaves : MODE == 1;
   const int sl = MODE == 0 ? (w & 3) : w;  // frequency slice; below 4 also the batch element of the group
-  // workgroup -> (KV head, split of that head)
-  const int grp = blockIdx.y;
-  // (the first sixteen entries are compared at once: they arrive with one load of the argument block, where a
-  // scan waits for one dependent load per head)
-  int h = 0;
+  // workgroup -> (batch group, KV head, split of that head)
+  int grp = blockIdx.y, h = 0, split = 0;
+  if constexpr (FUSE) {
+    const int code = p.fz.wg_map[blockIdx.x];   // (a one-dimensional grid)
+    const int team = code >> kFusedSplitBits;
+    grp = team / p.Hkv;
+    h = team - grp * p.Hkv;
+    split = code & ((1 << kFusedSplitBits) - 1);
+  } else {
+    // (the first sixteen entries are compared at once: they arrive with one load of the argument block, where a
+    // scan waits for one dependent load per head)
 #pragma unroll
-  for (int i = 1; i < 16; ++i) h += (int)blockIdx.x >= p.st.first[i] ? 1 : 0;
-  if (p.Hkv > 16)
-    while (h + 1 < p.Hkv && (int)blockIdx.x >= p.st.first[h + 1]) ++h;
-  const int split = blockIdx.x - p.st.first[h];
+    for (int i = 1; i < 16; ++i) h += (int)blockIdx.x >= p.st.first[i] ? 1 : 0;
+    if (p.Hkv > 16)
+      while (h + 1 < p.Hkv && (int)blockIdx.x >= p.st.first[h + 1]) ++h;
+    split = blockIdx.x - p.st.first[h];
+  }
   const int G = p.G, N = p.N;
   const int b0 = grp * p.nbpg;
   const int nb = min(p.nbpg, p.B - b0);
@@ -323,6 +335,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int t_beg = split * tiles_per_split;
   const int t_end = min(n_tiles, t_beg + tiles_per_split);
   const int n_it = t_end > t_beg ? t_end - t_beg : 0;
+  // fused merge: the head's compressed V dims (offset into the lists, count), needed behind the page loop
+  int fz_vc0 = 0, fz_vc_len = 0;
+  if constexpr (FUSE) {
+    fz_vc0 = p.fz.vc_h[h];
+    fz_vc_len = p.fz.vc_h[h + 1] - fz_vc0;
+  }
 
   // Rotation constants of slice sl into LDS: one entry (unit, lane group) per lane, requested early and stored once
   // the other loads of the prologue are on their way.  Every wave stores the constants it reads itself (in the
@@ -872,6 +890,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           if (f < ndg) *(float4v*)&on[f * 16 + 4 * lg] = oacc[f];
       }
     }
+  }
+  if constexpr (FUSE) {
+    const FusedShare fs = fused_share(p, fz_vc0, fz_vc_len, split, p.st.n[h], b0, nb, KS, tid);
+    fused_merge_tail<E>(p, (float*)&s_stage[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb, KS);
   }
 }
 

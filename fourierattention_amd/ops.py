@@ -380,7 +380,7 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
                     T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None,
-                    no_alloc=False, balance_heads=True):
+                    no_alloc=False, balance_heads=True, no_fuse=False):
     """Thin call into ``fa_decode_attn``.  The result is float32 like the reference's (TRI:779) unless ``out_dtype``
     names the dtype of ``q``: then the merge launch rounds it to that type itself (the caller's ``.to(dtype)``).
 
@@ -391,7 +391,9 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     ``no_alloc``: call ``fa_decode_attn_noalloc`` (partial results in the library's own fixed buffer, no workspace
     tensor; pass ``out`` as well and nothing is allocated on the device at all).
     ``balance_heads``: hand the per-head padded dim counts of a paged store over on the host side too, so that heads
-    that store more dims get more splits (``False``: every head the same number, for comparison)."""
+    that store more dims get more splits (``False``: every head the same number, for comparison).
+    ``no_fuse``: keep the sink/window tiles, the mid rows and the merge as launches of their own where the library
+    would run them as one (for comparison)."""
     from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
@@ -440,6 +442,7 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
         if tables is not None:
             a.tables = tables.data_ptr()
     a.force_generic = int(bool(force_generic))
+    a.no_fuse = int(bool(no_fuse))
     a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()
     a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list = vc.data_ptr(), vc_h.data_ptr(), vn.data_ptr(), vn_h.data_ptr()
     if out is None:
