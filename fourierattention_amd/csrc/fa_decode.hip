@@ -1642,6 +1642,8 @@ struct Plan {
   int n_il_split, n_mid_split, tiles_per_split, nbpg, n_groups, ks;
   int n_wg;   // matrix-core mid rows: workgroups per batch group
   fa_mfma::SplitTable st;
+  int heads_per_bin;                        // > 0: the splits were shared out so that the teams fill the dies exactly
+  int bin_of_head[fa_mfma::kSplitHeads];
   int n_merge_chunks;
   size_t off_W, off_c0, off_ilm, off_ild, off_ilo, off_mm, off_md, off_mg, off_mon, off_tab, off_scores, total;
   // merge after the matrix-core mid rows: contributions per block of coefficient rows, staged sums, counters
@@ -1664,26 +1666,51 @@ bool mfma_shape_ok(int Hq, int Hkv, int D, int N, int dtype, int layout) {
 // Llama-3.1-8B), a workgroup takes ceil(pages / splits) pages, and single splits move from the head that finishes first to
 // the head that finishes last while that shortens the longest time.  No head gets more than `room` splits (half as
 // many again as the even share: the partial buffers are sized for that).  Returns the largest count.
-int share_out_splits(fa_mfma::SplitTable& st, int Hkv, int tiles, int ns, int room, const int32_t* kpad, const int32_t* vpad) {
+// heads_per_bin > 0 (the merge may run inside the mid-row launch, whose teams must fill the dies exactly): the heads
+// are put into bins of that many, expensive heads with cheap ones, and splits only move between the heads of a bin,
+// so that every bin keeps heads_per_bin * ns splits; bin_of_head[h] receives the bin.  Splits that no page is left
+// for are then kept (their workgroups find nothing to do).
+int share_out_splits(fa_mfma::SplitTable& st, int Hkv, int tiles, int ns, int room, const int32_t* kpad, const int32_t* vpad,
+                     int heads_per_bin = 0, int* bin_of_head = nullptr) {
   using fa_mfma::kSplitHeads;
   for (int h = 0; h < kSplitHeads; ++h) st.n[h] = ns;
+  const bool binned = heads_per_bin > 0 && bin_of_head && Hkv <= kSplitHeads && Hkv % heads_per_bin == 0;
+  if (bin_of_head)
+    for (int h = 0; h < Hkv && h < kSplitHeads; ++h) bin_of_head[h] = binned ? h / heads_per_bin : -1;
   if (kpad && vpad && ns > 1 && Hkv > 1 && Hkv <= kSplitHeads) {
     int cost[kSplitHeads];
     for (int h = 0; h < Hkv; ++h) cost[h] = 54 + 2 * ((kpad[h + 1] - kpad[h]) / 32) + 3 * ((vpad[h + 1] - vpad[h]) / 16);
     auto time_of = [&](int h, int n) { return (int64_t)cost[h] * fa_cdiv(tiles, n); };
-    for (int moves = 0; moves < ns * Hkv; ++moves) {
-      int slow = 0;
-      for (int h = 1; h < Hkv; ++h)
-        if (time_of(h, st.n[h]) > time_of(slow, st.n[slow])) slow = h;
-      if (st.n[slow] >= room) break;
-      const int64_t worst = time_of(slow, st.n[slow]);
-      int donor = -1;   // the head that is fastest even with one split fewer
-      for (int h = 0; h < Hkv; ++h)
-        if (h != slow && st.n[h] > 1 && (donor < 0 || time_of(h, st.n[h] - 1) < time_of(donor, st.n[donor] - 1))) donor = h;
-      if (donor < 0 || time_of(donor, st.n[donor] - 1) >= worst) break;   // nothing gained: the donor would be as slow
-      // the step must shorten the longest time or leave it to another head that is no slower than before
-      --st.n[donor];
-      ++st.n[slow];
+    const int n_bins = binned ? Hkv / heads_per_bin : 1;
+    if (binned) {   // heads by falling cost, dealt out to the bins there and back
+      int order[kSplitHeads];
+      for (int h = 0; h < Hkv; ++h) order[h] = h;
+      for (int i = 1; i < Hkv; ++i)
+        for (int j = i; j > 0 && cost[order[j]] > cost[order[j - 1]]; --j) {
+          const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t;
+        }
+      for (int i = 0; i < Hkv; ++i) {
+        const int pass = i / n_bins, at = i % n_bins;
+        bin_of_head[order[i]] = (pass & 1) ? n_bins - 1 - at : at;
+      }
+    }
+    for (int bin = 0; bin < n_bins; ++bin) {
+      auto in_bin = [&](int h) { return !binned || bin_of_head[h] == bin; };
+      for (int moves = 0; moves < ns * Hkv; ++moves) {
+        int slow = -1;
+        for (int h = 0; h < Hkv; ++h)
+          if (in_bin(h) && (slow < 0 || time_of(h, st.n[h]) > time_of(slow, st.n[slow]))) slow = h;
+        if (slow < 0 || st.n[slow] >= room) break;
+        const int64_t worst = time_of(slow, st.n[slow]);
+        int donor = -1;   // the head that is fastest even with one split fewer
+        for (int h = 0; h < Hkv; ++h)
+          if (in_bin(h) && h != slow && st.n[h] > 1 &&
+              (donor < 0 || time_of(h, st.n[h] - 1) < time_of(donor, st.n[donor] - 1))) donor = h;
+        if (donor < 0 || time_of(donor, st.n[donor] - 1) >= worst) break;   // nothing gained: the donor would be as slow
+        // the step must shorten the longest time or leave it to another head that is no slower than before
+        --st.n[donor];
+        ++st.n[slow];
+      }
     }
   }
   int largest = 0;
@@ -1692,7 +1719,7 @@ int share_out_splits(fa_mfma::SplitTable& st, int Hkv, int tiles, int ns, int ro
     if (h < Hkv) {
       // (as many splits as pages of the resulting length really fill)
       const int per = fa_cdiv(tiles, st.n[h] > 0 ? st.n[h] : 1);
-      st.n[h] = st.n[h] > 0 ? fa_cdiv(tiles, per) : 0;
+      if (!binned) st.n[h] = st.n[h] > 0 ? fa_cdiv(tiles, per) : 0;
       if (st.n[h] > largest) largest = st.n[h];
     }
     st.first[h + 1] = st.first[h] + (h < Hkv ? st.n[h] : 0);
@@ -1703,7 +1730,8 @@ int share_out_splits(fa_mfma::SplitTable& st, int Hkv, int tiles, int ns, int ro
 // kpad / vpad: see share_out_splits.  full_room: size the partial buffers for the most uneven share a call with those
 // lists could ask for (the workspace query, which does not see them).
 Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfma, bool il_fast,
-               const int32_t* kpad = nullptr, const int32_t* vpad = nullptr, bool full_room = false) {
+               const int32_t* kpad = nullptr, const int32_t* vpad = nullptr, bool full_room = false,
+               bool fill_dies = true) {
   Plan p{};
   p.path = mfma ? Path::Mfma : Path::Generic;
   p.n_il_split = fa_cdiv(n_il, il_fast ? kIlFastTile : kTile);
@@ -1723,7 +1751,16 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     const int even = ns > 0 ? fa_cdiv(tiles, p.tiles_per_split) : 0;
     int room = fa_cdiv(3 * even, 2);
     if (room > tiles) room = tiles;
-    const int largest = share_out_splits(p.st, Hkv, tiles, even, room, kpad, vpad);
+    // Teams of the launch per die, if the merge may run inside it (see fused_merge_plan): a whole number of heads of
+    // one batch group, or whole batch groups
+    p.heads_per_bin = 0;
+    {
+      const int teams = Hkv * p.n_groups;
+      if (fill_dies && fa_mfma::table_slices(N) == 4 && D == fa_mfma::kFusedD && G <= fa_mfma::kFusedG && teams % fa_mfma::kFusedXcds == 0 &&
+          teams / fa_mfma::kFusedXcds < Hkv && Hkv % (teams / fa_mfma::kFusedXcds) == 0 && even == ns)
+        p.heads_per_bin = teams / fa_mfma::kFusedXcds;
+    }
+    const int largest = share_out_splits(p.st, Hkv, tiles, even, room, kpad, vpad, p.heads_per_bin, p.bin_of_head);
     p.n_mid_split = full_room && Hkv > 1 && Hkv <= fa_mfma::kSplitHeads ? room : largest;
     p.n_wg = p.st.first[Hkv <= fa_mfma::kSplitHeads ? Hkv : fa_mfma::kSplitHeads];
   } else {
@@ -1880,22 +1917,29 @@ bool fused_merge_plan(const fa_decode_args& a, const Plan& p, uint16_t* wg_map, 
       }
   }
   if (!fused_layout_ok(st)) return false;
-  // Workgroup L of the launch runs on die L % 8.  Teams are placed largest first into the die with room; the
-  // workgroups of die c are L = c, c + 8, c + 16, ...
+  // Workgroup L of the launch runs on die L % 8; the workgroups of die c are L = c, c + 8, c + 16, ...  Teams go
+  // to the dies bin by bin (the bins the splits were shared out in, or whole batch groups), largest first otherwise.
   const int cap = total / kFusedXcds;
   int order[kFusedMaxWgs], fill[kFusedXcds] = {};
   for (int t = 0; t < n_teams; ++t) order[t] = t;
   auto size_of = [&](int t) { return p.st.n[t % a.Hkv]; };
-  for (int i = 1; i < n_teams; ++i)   // insertion sort by size, descending, stable
-    for (int j = i; j > 0 && size_of(order[j]) > size_of(order[j - 1]); --j) {
-      const int tmp = order[j]; order[j] = order[j - 1]; order[j - 1] = tmp;
-    }
+  if (p.heads_per_bin == 0) {
+    for (int i = 1; i < n_teams; ++i)   // insertion sort by size, descending, stable
+      for (int j = i; j > 0 && size_of(order[j]) > size_of(order[j - 1]); --j) {
+        const int tmp = order[j]; order[j] = order[j - 1]; order[j - 1] = tmp;
+      }
+  }
   for (int i = 0; i < n_teams; ++i) {
     const int t = order[i], n = size_of(t);
     if (n <= 0) return false;
     int c = 0;
-    while (c < kFusedXcds && fill[c] + n > cap) ++c;
-    if (c == kFusedXcds) return false;
+    if (p.heads_per_bin > 0) {
+      c = (t / a.Hkv) * (a.Hkv / p.heads_per_bin) + p.bin_of_head[t % a.Hkv];
+      if (c >= kFusedXcds || fill[c] + n > cap) return false;
+    } else {
+      while (c < kFusedXcds && fill[c] + n > cap) ++c;
+      if (c == kFusedXcds) return false;
+    }
     for (int s = 0; s < n; ++s) wg_map[kFusedXcds * (fill[c] + s) + c] = (uint16_t)((t << kFusedSplitBits) | s);
     fill[c] += n;
   }
@@ -2195,7 +2239,7 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
   const bool mfma = use_mfma(*a);
   const bool il_fast = il_fast_ok(*a);
   const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma,
-                           il_fast, a->k_pad_h_host, a->v_pad_h_host);
+                           il_fast, a->k_pad_h_host, a->v_pad_h_host, false, !a->no_fuse);
   FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
              a->workspace_bytes, p.total);
   FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");
