@@ -57,8 +57,8 @@ int fa_abi_version(void);
  * otherwise columns 0..Mc-1 are read.  c: (B, 2N, Mc) fp32 contiguous.
  * accumulate != 0 adds into c (the `base_input + ...` of TRI:856).
  * workspace (optional): with at least fa_mat_fourier_workspace_bytes(B, K, Mc, N)
- * bytes (256-byte aligned), 16-bit inputs of K >= 512 rows with N % 8 == 0 and
- * Mc even run on the matrix cores (basis rounded to fp16, fp32 accumulation);
+ * bytes (256-byte aligned), 16-bit inputs of K >= 512 rows with N % 8 == 0 (any
+ * number of columns Mc) run on the matrix cores (basis rounded to fp16, fp32 accumulation);
  * without it, and for every other shape, an fp32 vector kernel is used. */
 int fa_mat_fourier(const void* a, int a_dtype, int64_t a_batch_stride, int64_t a_row_stride,
                    const int32_t* cols, float* c, int B, int K, int Mc, int N, int T,
@@ -309,6 +309,15 @@ int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_s
  * the stream is being captured). */
 int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
 
+/* How fa_decode_attn would cut the mid rows of each KV head into splits on the matrix-core kernels (host-side
+ * arithmetic only, no GPU work; no counterpart in the reference): splits_out[h] for h < Hkv, given the host copies of
+ * the per-head padded dim counts (or NULL for both: every head the same), and in *room_out (optional) the number of
+ * splits per head that fa_decode_attn_workspace_bytes leaves room for.  FA_ERR_UNSUPPORTED for shapes that take the
+ * generic kernels. */
+int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m,
+                         const int32_t* k_pad_h_host, const int32_t* v_pad_h_host, int32_t* splits_out,
+                         int32_t* room_out);
+
 /* fa_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): no counterpart in the reference.  `args->workspace` and
  * `args->workspace_bytes` are ignored; the partial results live in a buffer of FA_DECODE_NOALLOC_SCRATCH_BYTES
@@ -320,15 +329,6 @@ int fa_decode_attn(const fa_decode_args* args, fa_stream_t stream);
  * overlap on one GPU (two streams, two threads) race and must be serialised by the caller; consecutive calls on
  * one stream are fine (every kernel writes what it later reads, nothing needs clearing).  The first call on a
  * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture. */
-/* How fa_decode_attn would cut the mid rows of each KV head into splits on the matrix-core kernels (host-side
- * arithmetic only, no GPU work; no counterpart in the reference): splits_out[h] for h < Hkv, given the host copies of
- * the per-head padded dim counts (or NULL for both: every head the same), and in *room_out (optional) the number of
- * splits per head that fa_decode_attn_workspace_bytes leaves room for.  FA_ERR_UNSUPPORTED for shapes that take the
- * generic kernels. */
-int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total, int L_m,
-                         const int32_t* k_pad_h_host, const int32_t* v_pad_h_host, int32_t* splits_out,
-                         int32_t* room_out);
-
 #define FA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
 int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
 
