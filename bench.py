@@ -44,6 +44,17 @@ _RAGGED = {
 }
 for _name, (_kc, _vc) in _RAGGED.items():
     WORKLOADS[f"config3_ragged_{_name}"] = dict(WORKLOADS["config3_decode_attn_8b_32k"], cper=None, kc_heads=_kc, vc_heads=_vc)
+# The settings the reference itself evaluates with (models/fourier.py:141-153, eval/eval_longbench_fourier.py:45-46,
+# 72, 86): batch 1, 4 sink tokens, a window of 1020, 512 / 1024 / 2048 states, with the head-by-head counts of its own
+# Llama-3.1-8B mask (layers 0, 15 and 31 at 1024 states; layer 15 at the other two)
+_REF_EVAL = dict(B=1, ctx=32768, Hq=32, Hkv=8, D=128, I=4, W=1020, cper=None, max_new=128)
+for _name, (_kc, _vc) in _RAGGED.items():
+    WORKLOADS[f"ref_eval_b1_32k_m1024_{_name}"] = dict(_REF_EVAL, M=1024, kc_heads=_kc, vc_heads=_vc)
+for _m in (512, 2048):
+    WORKLOADS[f"ref_eval_b1_32k_m{_m}_layer15"] = dict(_REF_EVAL, M=_m, kc_heads=_RAGGED["layer15"][0], vc_heads=_RAGGED["layer15"][1])
+# what the default run times besides its headline workload (one line each in "other_workloads")
+OTHER_WORKLOADS = ["config3_ragged_layer0", "config3_ragged_layer15", "config3_ragged_layer31", "config4_decode_attn_8b_64k",
+                   "config5_decode_attn_3b_128k"] + [n for n in WORKLOADS if n.startswith("ref_eval_")]
 
 
 def compressed_counts(w):
@@ -96,6 +107,29 @@ def build_cache(w, dtype, device, seed=0, layers=1):
     kn = synth.apply_rope(torch.randn((B, Hkv, 1, D), generator=g, device=device), cq.to(device), sq.to(device)).to(dtype)
     vn = torch.randn((B, Hkv, 1, D), generator=g, device=device).to(dtype)
     return cache, q, kn, vn
+
+
+def attn_step_bench(name, device, steps=100, warmup=10):
+    """Decode attention of one layer on workload ``name`` (cache built through its own prefill): time per step between
+    events around ``steps`` calls, the compulsory bytes and what fraction of the HBM peak that is."""
+    from fourierattention_amd import _lib
+    w = WORKLOADS[name]
+    cache, q, kn, vn = build_cache(w, torch.bfloat16, device)
+    for _ in range(warmup):
+        out = cache.decode_attention(q, 0, w["Hq"], w["Hkv"])
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        out = cache.decode_attention(q, 0, w["Hq"], w["Hkv"])
+    e1.record()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    ms = e0.elapsed_time(e1) / steps
+    nbytes = algorithmic_bytes(w)
+    return {"us_per_step": round(ms * 1e3, 2), "algorithmic_bytes": nbytes, "GB_s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "batch": w["B"], "context": w["ctx"],
+            "window": w["W"], "coeff_rows": w["M"], "merge_inside_mid_row_launch": bool(_lib.load().fa_decode_attn_last_fused())}
 
 
 def parity_check(device):
@@ -381,6 +415,8 @@ def main():
                     help="skip the leg that uses the CPU restatement: the parity check before the timed region and the "
                          "CPU baseline after it (for profiler runs)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end decodes of configs 4 and 5 in the default run")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the ragged-mask, config 4 / 5 and batch-1 workloads the default run times besides its headline")
     ap.add_argument("--layers", type=int, default=32, help="layers assumed for the attention-only tok/s figure")
     ap.add_argument("--even-splits", action="store_true",
                     help="give every KV head the same number of splits of the mid rows (default: heads that store more dims "
@@ -552,6 +588,16 @@ def main():
     result["stream_update"] = {"ms_per_step": round(upd_ms, 5), "wall_ms_per_step": round(upd_wall * 1e3, 5),
                                "algorithmic_bytes": upd_bytes, "GB_s": round(upd_bytes / (upd_ms * 1e-3) / 1e9, 1)}
     del cache, q, kn, vn, out
+    if args.workload == "config3_decode_attn_8b_32k" and not args.no_other_workloads:
+        # the same kernels on the reference's own ragged masks, on the per-layer attention of configs 4 and 5 and
+        # in the reference's evaluation settings (batch 1): latency and fraction of the HBM peak of the whole step
+        result["other_workloads"] = {}
+        for name in OTHER_WORKLOADS:
+            torch.cuda.empty_cache()
+            try:
+                result["other_workloads"][name] = attn_step_bench(name, device)
+            except Exception as exc:
+                result["other_workloads"][name] = {"error": f"{type(exc).__name__}: {exc}"}
     result["prefill_compress"] = compress_bench(device)
     result["prefill_attn"] = prefill_attn_bench(device)
     if not args.no_e2e and args.workload.startswith("config3"):

@@ -90,6 +90,21 @@ def test_config4_sequence_at_65536_tokens():
     assert np.isfinite(got).all() and err <= 2e-2, err
 
 
+@pytest.mark.parametrize("states", [1024, 512])
+def test_reference_evaluation_settings_batch_one(states):
+    """The settings the reference evaluates with (models/fourier.py:141-153, eval/eval_longbench_fourier.py:45-46):
+    batch 1, 4 sink tokens, a local window of 1020, 1024 (or 512) states, and layer 31 of the mask it ships for
+    Llama-3.1-8B at 32k (ragged heads, up to 127 stored dims: the wide kernel instance).  At batch 1 a workgroup's
+    sixteen matrix-core columns hold the four query heads of one KV head only."""
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "masks_extract.json")))
+    mask = {"Layer_0": fx["llama3.1-8b-fourier/compressed_dims_32k_1024states"]["layers"]["Layer_31"]["splithead"]}
+    gpu, cpu, got, want = _one_sequence(32768, 32, 8, 128, 1020, states, torch.bfloat16, mask, seed=9)
+    assert gpu._tables is not None and gpu.curr_tokennum == cpu.curr_tokennum == [32768 - 4 - 1020 + 1]
+    assert gpu.period_reconstruct == cpu._t_x()
+    err = np.abs(got - want).max()
+    assert np.isfinite(got).all() and err <= 2e-2, err
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_statistics_at_full_length_in_units_of_the_last_place(dtype):
     """The statistics the prefill freezes (CACHE:564-569), at 32768 tokens, on columns that differ in offset and in
