@@ -93,9 +93,57 @@ def audit_async_lds_reads(asm_text: str):
     return found
 
 
+# kernels in which one workgroup hands data to another inside a launch: it stores, waits for the stores, then counts
+# itself in with an atomic (decode_merge_rows_kernel; the instances of decode_mid_mfma_kernel that merge their own
+# partials, whose template argument list ends in `true`)
+HANDOVER_KERNELS = (re.compile(r"decode_merge_rows_kernel"), re.compile(r"decode_mid_mfma_kernel\S*Lb1EEEv"))
+_STORE_OPS = ("global_store", "buffer_store", "flat_store")
+
+
+def audit_handover_stores(asm_text: str, kernels=HANDOVER_KERNELS):
+    """In the kernels that hand data from one workgroup to another, every counting atomic must find the workgroup's
+    stores acknowledged: walking back from each ``global_atomic_add`` through the listing, an ``s_waitcnt`` with
+    ``vmcnt(0)`` has to come before any vector-memory store does.  The source guarantees it (``s_waitcnt(0)``, a
+    barrier, then the atomic), but nothing in the language ties the stores to that wait: a compiler that sank a store
+    below it would produce a hand-over that works most of the time.  Returns ``(violations, atomics_seen)``; the scan
+    follows the layout of the code backwards (labels and branches are passed over), which is conservative for the
+    straight-line sequences it is meant for."""
+    found, seen = [], 0
+    lines = asm_text.split("\n")
+    kernel, start = None, 0
+    for no, line in enumerate(lines):
+        mk = re.match(r"^(_Z\S+):", line)
+        if mk:
+            kernel, start = mk.group(1), no
+            continue
+        if kernel is None or not any(k.search(kernel) for k in kernels):
+            continue
+        s_ = line.strip().split(";")[0].strip()
+        if not s_.startswith("global_atomic_add"):
+            continue
+        seen += 1
+        ok = False
+        for back in range(no - 1, start, -1):
+            t = lines[back].strip().split(";")[0].strip()
+            if not t or t.startswith("."):
+                continue
+            if t.startswith("s_waitcnt") and re.search(r"vmcnt\(0\)", t):
+                ok = True
+                break
+            if t.startswith(_STORE_OPS):
+                found.append(f"{kernel}: the atomic at line {no + 1} follows `{t[:70]}` (line {back + 1}) with no "
+                             "s_waitcnt vmcnt(0) in between")
+                ok = True   # reported
+                break
+        if not ok:
+            found.append(f"{kernel}: no s_waitcnt vmcnt(0) in front of the atomic at line {no + 1}")
+    return found, seen
+
+
 # sources whose kernels issue LDS reads from inline asm (directly or through fa_decode_mfma.h): their assembly must
 # show such reads, or the audit above has looked at nothing
 ASYNC_LDS_SOURCES = ("fa_decode", "fa_prefill", "fa_spectral_mfma")
+HANDOVER_SOURCES = ("fa_decode",)
 
 
 def count_async_lds_reads(asm_text: str) -> int:
@@ -125,6 +173,15 @@ def audit_listings(base: str, listings) -> list:
     if base in ASYNC_LDS_SOURCES and reads == 0:
         found.append(f"{base}: no inline-asm LDS read found in the assembly of a source that issues them "
                      "(markers or spellings the scan relies on have changed)")
+    if base in HANDOVER_SOURCES:
+        atomics = 0
+        for text in listings:
+            bad, n = audit_handover_stores(text)
+            found += bad
+            atomics += n
+        if atomics == 0:
+            found.append(f"{base}: no counting atomic found in the kernels that hand data between workgroups "
+                         "(kernel names or spellings the scan relies on have changed)")
     return found
 
 
@@ -143,7 +200,7 @@ def _compile(src: str, obj_dir: str, extra) -> str:
         os.remove(tmp)   # intermediate files of the compile
     found = audit_listings(base, listings)
     if found:
-        raise RuntimeError(f"{src}: results of asynchronous LDS reads are used before their wait:\n" + "\n".join(found))
+        raise RuntimeError(f"{src}: the audit of the generated assembly failed:\n" + "\n".join(found))
     return obj
 
 

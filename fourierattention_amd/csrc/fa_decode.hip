@@ -1104,6 +1104,9 @@ __global__ __launch_bounds__(256) void decode_merge_rows_kernel(const MergeRowsA
   }
 
   // ---- the block that finishes last for this (b, KV head) puts the rows together ----------------------------
+  // Everything handed to that block went out through st_device (written through to memory) and is read back through
+  // ld_device (past the caches); a plain store or load on this path would be a hand-over that works most of the
+  // time.  The build checks in the generated assembly that no store follows the wait below in front of the counter.
   __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0) expcnt(0) lgkmcnt(0): this thread's stores have been acknowledged
   __syncthreads();
   if (tid == 0) s_last = atomicAdd(a.count + (int64_t)b * Hkv + h, 1u) == (unsigned)(R - 1);

@@ -287,8 +287,9 @@ def test_split_plan_of_the_mid_rows():
     """``fa_decode_split_plan`` (host-side arithmetic of the launch, runs without a GPU): how the mid rows of each KV
     head are cut into splits.  Same count for every head without the per-head lists or with a uniform mask; with a
     ragged mask the total stays the same, nobody gets more than the workspace query leaves room for, nobody gets
-    none, and a head that stores more dims never gets fewer splits (beyond one of rounding) than one that stores fewer
-    of both K and V."""
+    none, and the head with the widest pages gets more than the even share.  Where the merge may run inside the
+    mid-row launch (this geometry), the workgroups of a (batch group, KV head) must fill the dies of the device
+    exactly: heads are shared out in bins (here pairs, two heads per die and batch group) that keep their total."""
     import ctypes
     from fourierattention_amd import _lib
     lib = _lib.load()
@@ -308,13 +309,27 @@ def test_split_plan_of_the_mid_rows():
     for kp, vp in (([64, 32, 32, 32, 32, 64, 32, 64], [16, 0, 32, 32, 128, 16, 0, 48]),
                    ([96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16])):
         got, room2 = plan(31740, kp, vp)
-        assert room2 == room and sum(got) <= sum(even) and sum(got) >= sum(even) - len(got)
+        assert room2 == room and sum(got) == sum(even)
         assert min(got) >= 1 and max(got) <= room
-        for a in range(8):
-            for b in range(8):
-                if kp[a] >= kp[b] and vp[a] >= vp[b]:
-                    assert got[a] + 1 >= got[b], (a, b, got)             # (single splits move: equal heads may differ by one)
+        # the heads pair up into bins of twice the even share: B = 8 makes two batch groups of eight teams, sixteen
+        # teams on eight dies
+        left = sorted(got)
+        while left:
+            big = left.pop()
+            assert 2 * even[0] - big in left, (got, big)
+            left.remove(2 * even[0] - big)
         assert got[vp.index(max(vp))] > even[0]                          # the head with the widest V pages gets more
+    # one batch group (B <= 4): a team per die, nothing to share out
+    assert plan(31740, [96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16], B=4)[0] == [32] * 8
+    # a geometry the fused merge does not take (eight query heads per KV head): shared out freely, dominated heads
+    # never get more (beyond one of rounding)
+    kp, vp = [96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16]
+    got, _ = plan(31740, kp, vp, B=8, Hq=64)
+    assert len(set(got)) > 1
+    for a in range(8):
+        for b in range(8):
+            if kp[a] >= kp[b] and vp[a] >= vp[b]:
+                assert got[a] + 1 >= got[b], (a, b, got)                 # (single splits move: equal heads may differ by one)
     # fewer pages than workgroups: one page per split for everybody
     short, _ = plan(200, [96, 64, 96, 96, 64, 64, 64, 64], [48, 16, 16, 80, 16, 128, 48, 16])
     assert short == [7] * 8

@@ -1,7 +1,7 @@
 """The build's check of the generated assembly: an inline-asm LDS read whose registers are touched before the
 wait that covers it must be reported (the compiler may copy such registers when a conditional read is merged
 with the other path; nothing else would notice)."""
-from fourierattention_amd.build import audit_async_lds_reads
+from fourierattention_amd.build import audit_async_lds_reads, audit_handover_stores
 
 GOOD = """
 _Zkernel_a:
@@ -102,10 +102,78 @@ def test_audit_fails_closed():
     the audit, not a pass."""
     from fourierattention_amd.build import ASYNC_LDS_SOURCES, audit_listings, count_async_lds_reads
     assert count_async_lds_reads(GOOD) == 1 and count_async_lds_reads(PARTIAL) >= 2
-    assert audit_listings("fa_decode", [GOOD]) == []
+    assert audit_listings("fa_prefill", [GOOD]) == []
+    # fa_decode also holds the kernels that hand data between workgroups: without any of their counting atomics in
+    # the listing the audit has seen nothing and says so
+    assert any("no counting atomic" in m for m in audit_listings("fa_decode", [GOOD]))
     assert any("no gfx950 assembly" in m for m in audit_listings("fa_decode", []))
     plain = "_Zkernel_z:\n\tv_add_f32_e32 v1, v2, v3\n\ts_endpgm\n"
     assert "fa_decode" in ASYNC_LDS_SOURCES and "fa_stream" not in ASYNC_LDS_SOURCES
     assert any("no inline-asm LDS read" in m for m in audit_listings("fa_decode", [plain]))
     assert audit_listings("fa_stream", [plain]) == []          # a source without such reads passes on a plain listing
     assert audit_listings("fa_stream", [BAD_COPY]) != []       # but a violation is reported wherever it shows up
+
+
+# ---- hand-over between workgroups: stores, wait, counting atomic ----------------------------------------------------
+HANDOVER_GOOD = """
+_Z24decode_merge_rows_kernel13MergeRowsArgs:
+\tglobal_store_dword v[2:3], v4, off sc1
+\tglobal_store_dwordx4 v[6:7], v[8:11], off
+\ts_waitcnt vmcnt(0) expcnt(0) lgkmcnt(0)
+\ts_barrier
+\ts_cbranch_execz .LBB0_2
+; %bb.1:
+\tglobal_atomic_add v1, v[2:3], v1, off sc0
+.LBB0_2:
+\ts_endpgm
+"""
+
+# a store that was moved behind the wait
+HANDOVER_SUNK = """
+_Z24decode_merge_rows_kernel13MergeRowsArgs:
+\tglobal_store_dword v[2:3], v4, off sc1
+\ts_waitcnt vmcnt(0) lgkmcnt(0)
+\ts_barrier
+\tglobal_store_dword v[12:13], v14, off sc1
+\tglobal_atomic_add v1, v[2:3], v1, off sc0
+"""
+
+# a wait that does not cover vector memory
+HANDOVER_WRONG_WAIT = """
+_ZN7fa_mfma22decode_mid_mfma_kernelI6bf16_tLi8ELi2ELi4ELi2ELi0ELb1EEEvNS_9MidParamsIT_EE:
+\tglobal_store_dwordx4 v[6:7], v[8:11], off
+\ts_waitcnt lgkmcnt(0)
+\ts_barrier
+\tglobal_atomic_add v1, v[2:3], v1, off sc0
+"""
+
+# other kernels are not looked at
+HANDOVER_OTHER = """
+_Z19decode_merge_kernelPKf:
+\tglobal_store_dword v[2:3], v4, off
+\tglobal_atomic_add v1, v[2:3], v1, off sc0
+"""
+
+
+def test_handover_clean_sequence_passes():
+    assert audit_handover_stores(HANDOVER_GOOD) == ([], 1)
+
+
+def test_handover_store_behind_the_wait_is_reported():
+    found, seen = audit_handover_stores(HANDOVER_SUNK)
+    assert seen == 1 and len(found) == 1 and "global_store_dword v[12:13]" in found[0]
+
+
+def test_handover_wait_must_cover_vector_memory():
+    found, seen = audit_handover_stores(HANDOVER_WRONG_WAIT)
+    assert seen == 1 and len(found) == 1 and "decode_mid_mfma_kernel" in found[0]
+
+
+def test_handover_scan_only_covers_the_named_kernels():
+    assert audit_handover_stores(HANDOVER_OTHER) == ([], 0)
+
+
+def test_handover_audit_is_part_of_the_build_of_the_decode_kernels():
+    from fourierattention_amd.build import audit_listings
+    assert audit_listings("fa_decode", [GOOD + HANDOVER_GOOD]) == []
+    assert any("global_store_dword v[12:13]" in m for m in audit_listings("fa_decode", [GOOD + HANDOVER_SUNK]))
