@@ -36,7 +36,13 @@ def _exact_attention(query_states, k_local, v_local, num_kv_heads, head_dim):
     S = k_local.shape[1]
     if ops.prefill_attention_supported(query_states, k_local, head_dim) and v_local.stride() == k_local.stride():
         return ops.prefill_attention(query_states, k_local, v_local, num_kv_heads)   # (B, q_len, Hq, D)
-    # other shapes (float32 storage, odd head dims) and the host-only tests: the framework's attention
+    if query_states.is_cuda and query_states.dtype == torch.float32 and head_dim in (64, 128):
+        # float32 storage: the reference casts q, k and v to half for this call whatever the model's type
+        # (modeling_llama_fourier.py:633); the caller casts the result back
+        qh, kh, vh = query_states.half().contiguous(), k_local.half().contiguous(), v_local.half().contiguous()
+        if ops.prefill_attention_supported(qh, kh, head_dim):
+            return ops.prefill_attention(qh, kh, vh, num_kv_heads)
+    # other head dims and the host-only tests: the framework's attention
     k = k_local.view(B, S, num_kv_heads, head_dim).transpose(1, 2)
     v = v_local.view(B, S, num_kv_heads, head_dim).transpose(1, 2)
     if q_len == S:

@@ -29,7 +29,7 @@ struct PrefillParams {
   int64_t q_bs, q_hs, q_rs;
   const E* k;          // (B, S, Hkv * D) token-major
   int64_t k_bs, k_rs;
-  const E* vt;         // [B][Hkv][tiles][D / 16][64 lanes][8]: V^T fragments
+  const f16_t* vt;     // [B][Hkv][tiles][D / 16][64 lanes][8]: V^T fragments, always f16 (see prefill_vt_kernel)
   E* out;              // (B, q_len, Hq, D) contiguous
   int B, Hq, Hkv, S, q_len, n_tiles, HW, RW;
   float sm_log2e;
@@ -40,8 +40,12 @@ __device__ __forceinline__ int slot_key(int lg, int e) { return e < 4 ? 4 * lg +
 
 template <typename E, int D>
 __global__ __launch_bounds__(256) void prefill_vt_kernel(const E* __restrict__ v, int64_t v_bs, int64_t v_rs,
-                                                         E* __restrict__ vt, int S, int Hkv, int n_tiles) {
+                                                         f16_t* __restrict__ vt, int S, int Hkv, int n_tiles) {
+  // The second product runs in f16 whatever the storage type: the reference computes this attention as
+  // flash_attn_func(q.half(), k.half(), v.half()) (MODEL:633), with probabilities of 11 significant bits; a bf16
+  // operand would keep 8.  bf16 -> f16 is exact between 2^-14 and 65504 (larger magnitudes are clamped there).
   struct alignas(sizeof(E) * 8) Piece { E e[8]; };
+  struct alignas(16) PieceOut { f16_t e[8]; };
   __shared__ __attribute__((aligned(16))) E tile[kTileKeys][D + 8];
   const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
   const E* src = v + (int64_t)b * v_bs + (int64_t)h * D;
@@ -54,12 +58,15 @@ __global__ __launch_bounds__(256) void prefill_vt_kernel(const E* __restrict__ v
     *(Piece*)&tile[r][c * 8] = pc;
   }
   __syncthreads();
-  Piece* dst = (Piece*)(vt + (((int64_t)b * Hkv + h) * n_tiles + t) * (int64_t)(kTileKeys * D));
+  PieceOut* dst = (PieceOut*)(vt + (((int64_t)b * Hkv + h) * n_tiles + t) * (int64_t)(kTileKeys * D));
   for (int pidx = tid; pidx < (D / 16) * 64; pidx += 256) {
     const int dg = pidx >> 6, lane = pidx & 63, lg = lane >> 4, ld = lane & 15;
-    Piece o;
+    PieceOut o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o.e[e] = tile[slot_key(lg, e)][16 * dg + ld];
+    for (int e = 0; e < 8; ++e) {
+      const float x = fa_to_float(tile[slot_key(lg, e)][16 * dg + ld]);
+      o.e[e] = f16_t{(_Float16)fminf(fmaxf(x, -65504.f), 65504.f)};
+    }
     dst[pidx] = o;
   }
 }
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
 
   // this wave's share of a tile: fragments w, w + WAVES, ... (clamped to the last one: every wave issues OPS loads)
   const E* kb_base = p.k + (int64_t)b * p.k_bs + (int64_t)kvh * D + 8 * lg;
-  const E* vt_base = p.vt + ((int64_t)b * p.Hkv + kvh) * p.n_tiles * (int64_t)(kTileKeys * D) + lane * 8;
+  const f16_t* vt_base = p.vt + ((int64_t)b * p.Hkv + kvh) * p.n_tiles * (int64_t)(kTileKeys * D) + lane * 8;
   // The tiles are requested in order, so every load keeps a running pointer that moves on by one tile; only a last
   // tile that reaches past the keys computes its (clamped) rows afresh.
   const E* run[OPS];
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
   for (int i = 0; i < OPS; ++i) {
     const int f = min(w + i * WAVES, NF - 1);
     if (f < 2 * KS) run[i] = kb_base + (int64_t)(16 * (f / KS) + lc) * p.k_rs + 32 * (f % KS);
-    else run[i] = vt_base + (int64_t)(f - 2 * KS) * 512;
+    else run[i] = (const E*)(vt_base + (int64_t)(f - 2 * KS) * 512);   // (both 16-bit: the pointer only counts elements)
   }
   const int64_t k_step = (int64_t)kTileKeys * p.k_rs;
   const bool ragged_keys = (p.S % kTileKeys) != 0;
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
     vf[3] = lds_read_b128_async_at<3072>(vbase);
     // ---- softmax of the tile (base 2), per row = per lane column
     const bool edge = t * kTileKeys + 31 > r0 + offset || t * kTileKeys + 31 >= p.S;   // wave-uniform
-    vec8 pb[2];
+    half8 pb[2];   // probabilities as f16 operands
     float alpha[2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
       for (int e = 0; e < 8; ++e) {
         const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], p.sm_log2e, -m_use));
         psum += pv;
-        pb[rb][e] = (typename M::elem)pv;
+        pb[rb][e] = (_Float16)pv;
       }
       l_run[rb] = l_run[rb] * alpha[rb] + psum;
       m_run[rb] = m_new;
@@ -238,8 +245,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3, 3
     auto o_pair = [&](uint4v& f0, uint4v& f1, int dg) {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
-        oacc[dg][rb] = M::mma(__builtin_bit_cast(vec8, f0), pb[rb], oacc[dg][rb]);
-        oacc[dg + 1][rb] = M::mma(__builtin_bit_cast(vec8, f1), pb[rb], oacc[dg + 1][rb]);
+        oacc[dg][rb] = Mma<f16_t>::mma(__builtin_bit_cast(half8, f0), pb[rb], oacc[dg][rb]);
+        oacc[dg + 1][rb] = Mma<f16_t>::mma(__builtin_bit_cast(half8, f1), pb[rb], oacc[dg + 1][rb]);
       }
     };
     if constexpr (DG == 8) {
@@ -289,7 +296,7 @@ int launch_prefill(const void* q, int64_t q_bs, int64_t q_hs, int64_t q_rs, cons
                    const void* v, int64_t v_bs, int64_t v_rs, void* out, void* workspace, int B, int Hq, int Hkv, int S,
                    int q_len, float sm_scale, hipStream_t st) {
   const int n_tiles = fa_cdiv(S, kTileKeys);
-  E* vt = (E*)workspace;
+  f16_t* vt = (f16_t*)workspace;
   prefill_vt_kernel<E, D><<<dim3(n_tiles, Hkv, B), 256, 0, st>>>((const E*)v, v_bs, v_rs, vt, S, Hkv, n_tiles);
   const int G = Hq / Hkv;
   PrefillParams<E> p{};

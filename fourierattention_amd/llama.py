@@ -103,10 +103,20 @@ class LlamaDecoderLayer(nn.Module):
             if n_out % 16 or k % 1024:
                 continue
             fused = mods[0].weight.data if len(mods) == 1 else torch.cat([m.weight.data for m in mods], dim=0)
-            self._packed[name] = ops.PackedLinearWeight(fused.contiguous())
+            self._packed[name] = ops.PackedLinearWeight(fused.contiguous(), sources=[m.weight for m in mods])
+
+    def _packed_weight(self, name):
+        """The packed copy of a weight group, or ``None``: a copy whose source parameters have been written or
+        replaced since it was made (``load_state_dict``, ``.to()``, an in-place update) is dropped, and the layer goes
+        back to the modules' own weights until ``pack_projections`` is called again."""
+        w = self._packed.get(name)
+        if w is not None and w.stale():
+            del self._packed[name]
+            return None
+        return w
 
     def _linear(self, name, x, fallback):
-        w = self._packed.get(name)
+        w = self._packed_weight(name)
         return ops.linear_packed(x, w) if w is not None and w.covers(x) else fallback(x)
 
     def fuse_projections(self, max_rows: int = 16384):
@@ -144,7 +154,7 @@ class LlamaDecoderLayer(nn.Module):
         y = ops.add_rmsnorm(h, delta, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
         bsz, q_len, _ = y.shape
         nq, nk = at.num_heads * at.head_dim, at.num_key_value_heads * at.head_dim
-        pk = self._packed.get("qkv")
+        pk = self._packed_weight("qkv")
         if pk is not None and pk.covers(y):
             q, k, v = ops.linear_packed(y, pk).split((nq, nk, nk), dim=-1)
         elif self._qkv_weight is not None:
@@ -159,7 +169,7 @@ class LlamaDecoderLayer(nn.Module):
                               {"sin": sin, "cos": cos, "cache_position": cache_position})
         y = ops.add_rmsnorm(h, self._linear("o", o, at.o_proj), self.post_attention_layernorm.weight,
                             self.post_attention_layernorm.variance_epsilon)
-        pk = self._packed.get("gate_up")
+        pk = self._packed_weight("gate_up")
         if pk is not None and pk.covers(y):
             gate, up = ops.linear_packed(y, pk).chunk(2, dim=-1)
         elif self._gate_up_weight is not None:

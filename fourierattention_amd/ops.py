@@ -281,11 +281,25 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+class WeightStamp:
+    """Identity and version of the tensors a derived copy was made from: ``changed()`` once any of them has been
+    written in place (``load_state_dict``, an optimizer step) or replaced (``.to()``, re-assignment of ``.data``)."""
+
+    def __init__(self, tensors):
+        self._refs = list(tensors)
+        self._seen = [(t.data_ptr(), t._version) for t in self._refs]
+
+    def changed(self) -> bool:
+        return any((t.data_ptr(), t._version) != s for t, s in zip(self._refs, self._seen))
+
+
 class PackedLinearWeight:
     """A bias-free ``nn.Linear`` weight ``(n_out, K)`` re-laid for ``linear_packed``: the order in which the matrix
-    cores take it, so that a decode step (a handful of rows) streams it in contiguous KiB pieces."""
+    cores take it, so that a decode step (a handful of rows) streams it in contiguous KiB pieces.  ``sources``: the
+    parameters the weight was assembled from; ``stale()`` tells when the copy no longer matches them."""
 
-    def __init__(self, weight: torch.Tensor):
+    def __init__(self, weight: torch.Tensor, sources=None):
+        self.stamp = WeightStamp(sources if sources is not None else [weight])
         _require_gpu(weight, "weight")
         assert weight.dim() == 2 and weight.is_contiguous() and weight.dtype in (torch.bfloat16, torch.float16)
         self.n_out, self.k = int(weight.shape[0]), int(weight.shape[1])
@@ -293,6 +307,9 @@ class PackedLinearWeight:
         self.data = torch.empty_like(weight)
         check(_lib.load().fa_linear_pack(weight.data_ptr(), self.data.data_ptr(), self.n_out, self.k, dtype_code(weight.dtype),
                                          _stream(weight.device)))
+
+    def stale(self) -> bool:
+        return self.stamp.changed()
 
     def covers(self, x: torch.Tensor) -> bool:
         rows = x.numel() // max(x.shape[-1], 1)
@@ -443,6 +460,8 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
             a.tables = tables.data_ptr()
     a.force_generic = int(bool(force_generic))
     a.no_fuse = int(bool(no_fuse))
+    if seq_len_m >= _REPACK_MIN_ROWS and not force_generic:
+        _warn_if_off_the_matrix_cores(q.dtype, num_head_q, num_head_kv, D, N, isinstance(k_mn, MidStore))
     a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()
     a.vc_list, a.vc_h_list, a.vn_list, a.vn_h_list = vc.data_ptr(), vc_h.data_ptr(), vn.data_ptr(), vn_h.data_ptr()
     if out is None:
@@ -472,6 +491,28 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     else:
         check(lib.fa_decode_attn(ctypes.byref(a), _stream(q.device)))
     return out
+
+
+_warned_shapes = set()
+
+
+def _warn_if_off_the_matrix_cores(dtype, num_head_q, num_head_kv, head_dim, n_f, paged):
+    """Long contexts outside the shapes of the matrix-core kernels (16-bit paged storage, 128 / 256 / 512 / 1024
+    frequencies, heads of at most 128 dims, at most 8 query heads per KV head) run on vector-ALU kernels that take any
+    shape and are far slower (16.2 ms against 0.31 ms per layer at B=4, 131072 tokens, 24 / 8 heads): say so once
+    per shape instead of being silently slow."""
+    g = num_head_q // max(num_head_kv, 1)
+    ok = (dtype in (torch.bfloat16, torch.float16) and paged and n_f in (128, 256, 512, 1024) and head_dim <= 128 and g <= 8)
+    key = (dtype, num_head_q, num_head_kv, head_dim, n_f, paged)
+    if ok or key in _warned_shapes:
+        return
+    _warned_shapes.add(key)
+    import warnings
+    warnings.warn(
+        f"fourier decode attention: dtype={dtype}, {num_head_q}/{num_head_kv} heads of {head_dim} dims, {n_f} frequencies, "
+        f"{'paged' if paged else 'token-major'} mid rows run on the any-shape vector kernels, roughly 50x slower than the "
+        "matrix-core kernels (16-bit paged storage, 128/256/512/1024 frequencies, head_dim <= 128, <= 8 query heads per KV head)",
+        RuntimeWarning, stacklevel=3)
 
 
 def triton_fourier_attn(q, k_il, v_il, k_mc, v_mc, k_mn, v_mn,

@@ -72,3 +72,21 @@ def test_attention_forward_computes_rotary_tables_from_position_ids():
     assert torch.equal(a, b) and ca.get_seq_length() == cb.get_seq_length() == 9
     with pytest.raises(ValueError):
         attn(x, past_key_value=_cache())
+
+
+def test_shapes_off_the_matrix_cores_are_announced_once():
+    """Long contexts whose shape only the any-shape vector kernels take (e.g. float32 storage, 384 frequencies) are
+    about 50x slower: the operator says so, once per shape."""
+    import warnings
+    import torch
+    from fourierattention_amd import ops
+    ops._warned_shapes.clear()
+    with warnings.catch_warnings(record=True) as got:
+        warnings.simplefilter("always")
+        ops._warn_if_off_the_matrix_cores(torch.bfloat16, 32, 8, 128, 512, True)      # covered: silent
+        ops._warn_if_off_the_matrix_cores(torch.float32, 32, 8, 128, 512, True)
+        ops._warn_if_off_the_matrix_cores(torch.float32, 32, 8, 128, 512, True)       # the same shape again: silent
+        ops._warn_if_off_the_matrix_cores(torch.bfloat16, 32, 8, 128, 384, True)
+        ops._warn_if_off_the_matrix_cores(torch.bfloat16, 72, 8, 128, 512, True)      # nine query heads per KV head
+    assert len(got) == 3 and all(issubclass(w.category, RuntimeWarning) for w in got)
+    assert "vector kernels" in str(got[0].message)

@@ -27,9 +27,11 @@ def _oracle_rows(q, k, v, rows, Hq, Hkv, offset):
 
 def _tight(want, dtype):
     """What the arithmetic really leaves: the result is rounded to the storage type (half a unit in the last place of
-    the largest value) on top of 16-bit probabilities accumulated in fp32."""
-    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
-    return 0.5 * ulp * float(np.abs(want).max()) + (4e-3 if dtype == torch.bfloat16 else 1e-3)
+    the largest value) on top of f16 probabilities accumulated in fp32 - f16 for both storage types, as the reference
+    computes this attention in half precision whatever the model's type (modeling_llama_fourier.py:633)."""
+    top = float(np.abs(want).max())
+    ulp = 2.0 ** (np.floor(np.log2(top)) - (7 if dtype == torch.bfloat16 else 10))   # of the largest value's binade
+    return 0.5 * ulp + 1e-3
 
 
 def _case(seed, B, Hq, Hkv, D, S, q_len, dtype, rope=True):
@@ -102,6 +104,26 @@ def test_attention_forward_takes_the_kernel_for_the_prompt():
         assert torch.equal(out, direct)
         want = _oracle_rows(q, k, v, [0, S - 1], Hq, Hkv, 0).reshape(B, 2, Hq * D)
         assert np.abs(out[:, [0, S - 1]].float().cpu().numpy() - want).max() <= _tight(want, dtype)
+
+
+def test_float32_prompt_is_computed_in_half_like_the_reference():
+    """A float32 model: the reference casts q, k and v to half for the prompt attention whatever the model's type
+    (modeling_llama_fourier.py:633) and casts the result back.  Same here, on the matrix-core kernel."""
+    from fourierattention_amd import DynamicCache, fourier_attention, ops
+    from tests.test_gpu_cache import _cfg, _masks
+    B, Hq, Hkv, D, S = 1, 8, 2, 128, 200
+    masks = _masks(1, Hkv, D, [64, 64], [64, 64])
+    q, k, v = _case(5, B, Hq, Hkv, D, S, S, torch.float32)
+    cache = DynamicCache(_cfg(masks, num_key_value_heads=Hkv))
+    qg = H.to_gpu(q, torch.float32)
+    kg = H.to_gpu(k, torch.float32).view(B, S, Hkv, D).transpose(1, 2)
+    vg = H.to_gpu(v, torch.float32).view(B, S, Hkv, D).transpose(1, 2)
+    out = fourier_attention(qg, kg, vg, cache, 0, Hq, Hkv)
+    assert tuple(out.shape) == (B, S, Hq * D) and out.dtype == torch.float32
+    direct = ops.prefill_attention(qg.half(), H.to_gpu(k, torch.float32).half(), H.to_gpu(v, torch.float32).half(), Hkv)
+    assert torch.equal(out, direct.reshape(B, S, Hq * D).float())
+    want = _oracle_rows(q, k, v, [0, S // 2, S - 1], Hq, Hkv, 0).reshape(B, 3, Hq * D)
+    assert np.abs(out[:, [0, S // 2, S - 1]].cpu().numpy() - want).max() <= 4e-3      # inputs rounded to half
 
 
 def test_argument_errors():

@@ -73,6 +73,41 @@ def test_fused_projection_weights_keep_modules_and_state_dict():
     assert torch.equal(layer._gate_up_weight[:mlp.gate_proj.weight.shape[0]], other.model.layers[1].mlp.gate_proj.weight)
 
 
+def test_packed_copies_are_dropped_when_their_weights_change():
+    """A packed copy of a weight group (``pack_projections``) is a second tensor: once one of the parameters it was
+    made from is written in place (``load_state_dict``, an update) or replaced, decode steps must go back to the
+    modules' own weights instead of multiplying with the stale copy."""
+    from fourierattention_amd import ops
+    from fourierattention_amd.llama import LlamaDecoderLayer
+    w1, w2 = torch.nn.Parameter(torch.randn(8, 4)), torch.nn.Parameter(torch.randn(8, 4))
+    stamp = ops.WeightStamp([w1, w2])
+    assert not stamp.changed()
+    with torch.no_grad():
+        w2.mul_(2.0)                                    # in place
+    assert stamp.changed()
+    stamp = ops.WeightStamp([w1, w2])
+    w1.data = w1.data.clone()                           # replaced storage
+    assert stamp.changed()
+
+    class Copy:                                         # stands in for a packed weight (which needs the GPU)
+        def __init__(self, sources):
+            self.stamp = ops.WeightStamp(sources)
+
+        def stale(self):
+            return self.stamp.changed()
+
+        def covers(self, x):
+            return True
+
+    layer = LlamaDecoderLayer(_tiny(), 0)
+    layer._packed["o"] = Copy([layer.self_attn.o_proj.weight])
+    assert layer._packed_weight("o") is layer._packed["o"]
+    layer.load_state_dict(layer.state_dict())           # copies in place: every version moves on
+    assert layer._packed_weight("o") is None and "o" not in layer._packed
+    x = torch.randn(2, layer.self_attn.o_proj.weight.shape[1])
+    assert torch.equal(layer._linear("o", x, layer.self_attn.o_proj), layer.self_attn.o_proj(x))
+
+
 def test_model_requires_a_cache():
     from fourierattention_amd.llama import random_init
     model = random_init(_tiny(layers=1), dtype=torch.float32, device="cpu")
