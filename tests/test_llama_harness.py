@@ -149,10 +149,15 @@ def _oracle_forward(model, cfg, cache, ids, pos0, gpu_cache):
             S = kw["k_local"].shape[1]
             k = kw["k_local"].reshape(B, S, Hkv, D).transpose(0, 2, 1, 3).repeat(Hq // Hkv, axis=1)
             v = vw["v_local"].reshape(B, S, Hkv, D).transpose(0, 2, 1, 3).repeat(Hq // Hkv, axis=1)
-            s = np.einsum("bhqd,bhkd->bhqk", qh, k) / np.sqrt(D)
+            # the reference computes the prompt attention on half-precision copies whatever the model's type and
+            # casts the result back (flash_attn_func(q.half(), k.half(), v.half()), modeling_llama_fourier.py:633);
+            # the cache above was given the unrounded keys and values, as there
+            half = lambda a: a.astype(np.float16).astype(np.float64)
+            qa, k, v = half(qh), half(k), half(v)
+            s = np.einsum("bhqd,bhkd->bhqk", qa, k) / np.sqrt(D)
             s = np.where(np.arange(S)[None, :] <= np.arange(q_len)[:, None] + (S - q_len), s, -np.inf)
             p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
-            o = np.einsum("bhqk,bhkd->bhqd", p, v)
+            o = half(np.einsum("bhqk,bhkd->bhqd", p, v))
         else:
             for n in ("k_scale", "k_layer_average", "kd_layer_average", "v_scale", "v_layer_average", "vd_layer_average"):
                 getattr(cache, n)[li] = getattr(gpu_cache, n)[li].float().cpu().numpy()   # isolate the attention from the stats
@@ -182,7 +187,7 @@ def test_compressed_decode_steps_match_the_oracle_model():
     with torch.no_grad():
         got = model(input_ids=ids.cuda(), past_key_values=gpu, num_logits_to_keep=1).logits[:, -1].cpu().numpy()
         want = _oracle_forward(model, cfg, cpu, ids, 0, gpu)
-        np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)     # prompt pass: exact attention on both sides
+        np.testing.assert_allclose(got, want, rtol=3e-3, atol=3e-3)     # prompt pass: exact attention in half on both sides
         nxt = torch.from_numpy(want.argmax(-1))[:, None]
         for step in range(4):
             assert gpu.get_seq_length() == 300 + step == cpu.get_seq_length()
