@@ -216,7 +216,7 @@ def cpu_baseline():
                                   f"warm-ups = {med1 * 1e3:.2f} ms (min {t1[0] * 1e3:.2f} ms), {bytes1} algorithmic bytes"}}
 
 
-KERNEL_SOURCES = ("fa_decode.hip", "fa_decode_mfma.h", "fa_mfma_util.h", "fa_common.h")
+KERNEL_SOURCES = ("fa_decode.hip", "fa_decode_mfma.h", "fa_decode_fused.h", "fa_mfma_util.h", "fa_common.h")
 
 
 def kernel_source_digest():
@@ -424,6 +424,8 @@ def main():
     ap.add_argument("--no-fuse", action="store_true",
                     help="run sink/window tiles, mid rows and merge as launches of their own where the library would run the "
                          "merge inside the mid-row launch (for comparison)")
+    ap.add_argument("--no-sub-splits", action="store_true",
+                    help="a batch of one sequence: one page stream per workgroup instead of four sub-splits (comparison)")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
                     help="run the end-to-end decode of a random-init model instead (its own JSON line); --steps caps the "
                          "number of timed tokens per sequence")
@@ -472,6 +474,7 @@ def main():
     cache, q, kn, vn = build_cache(w, dtype, device)
     cache.balance_heads = not args.even_splits
     cache.fuse_decode = not args.no_fuse
+    cache.sub_splits = not args.no_sub_splits
     Hq, Hkv = w["Hq"], w["Hkv"]
     for _ in range(args.warmup):
         out = cache.decode_attention(q, 0, Hq, Hkv)
@@ -504,8 +507,11 @@ def main():
     # three launches: the coefficient-domain query shares one with the sink/window tiles (the third slot is the
     # gap left between the event pairs, a few microseconds of event overhead)
     # (with the merge inside the mid-row launch the step has two launches and the last slot is event overhead only)
-    kernel_ms = {"query_and_sink_window": per[0] + per[2], "mid_rows_and_merge" if merge_in_mid_rows else "mid_rows": per[1],
-                 "merge": per[3]}
+    kernel_ms = {"query_and_sink_window": per[0] + per[2], "mid_rows_and_merge" if merge_in_mid_rows else "mid_rows": per[1]}
+    if merge_in_mid_rows:
+        kernel_ms["empty_event_pair"] = per[3]
+    else:
+        kernel_ms["merge"] = per[3]
     # algorithmic bytes of each kernel's own launch
     kbytes = {
         "query_and_sink_window": w["B"] * w["M"] * ck * 4 + w["B"] * Hq * w["M"] * 4 + w["B"] * 2 * (w["I"] + w["W"]) * hd * 2,

@@ -204,7 +204,8 @@ class DynamicCache(Cache):
         self.force_generic = False                     # testing: keep decode attention off the MFMA kernels
         self.balance_heads = True                      # mid rows: more splits for heads that store more dims
         self.fuse_prefill = True                       # prefill: pages, coefficients and statistics from one read
-        self.fuse_decode = True                        # decode: sink/window, mid rows and merge as one launch where it applies
+        self.fuse_decode = True                        # decode: the merge inside the mid-row launch where it applies
+        self.sub_splits = True                         # ... and a batch of one as four sub-splits per workgroup
         self._book = CacheBook(self._num_layers, self.numinittokens, self.maxlocallen, self.maxmidstates,
                                self.maxnewtokens, self.maxtokens)
         self._layers: List[_Layer] = [_Layer() for _ in range(self._num_layers)]
@@ -461,4 +462,4 @@ class DynamicCache(Cache):
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
                                    sm_scale, tables=self._tables, force_generic=self.force_generic, timings=timings,
                                    out_dtype=out_dtype, out=out, no_alloc=no_alloc, balance_heads=self.balance_heads,
-                                   no_fuse=not self.fuse_decode)
+                                   no_fuse=(0 if self.fuse_decode else 1) | (0 if self.sub_splits else 2))

@@ -69,6 +69,9 @@ struct PrepArgs {
   const int32_t* kn_h;
   // fused step: the two meeting counters of every (batch group, KV head), cleared here for the launch behind
   unsigned* team_cnt;
+  // a batch of one sequence whose mid rows run as four sub-splits per workgroup (SUB instances of the mid-row kernel):
+  // the stored query dims go out four times, once for the columns of each sub-split
+  int sub;
 };
 
 // LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head
@@ -119,10 +122,11 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
   if constexpr (sizeof(E) == 2) if (bx == 1 && pa.q_stored) {
     const int kn0 = pa.kn_h[h], kn_len = pa.kn_h[h + 1] - kn0;
     const int s = tid >> 6, lane = tid & 63, lg = lane >> 4, lc = lane & 15;
-    const int grp = b / pa.nbpg, sl = b - grp * pa.nbpg;
-    const int g = lc - sl * G;   // the column's query head if the column is this batch element's
-    const bool mine = g >= 0 && g < G;
-    if (kn_len > 0) {   // (a head that stores no K dims has no entries in the list and nobody reads its operands)
+    const int grp = b / pa.nbpg;
+    // (a head that stores no K dims has no entries in the list and nobody reads its operands)
+    for (int sl = pa.sub ? 0 : b - grp * pa.nbpg, last = pa.sub ? 3 : sl; sl <= last && kn_len > 0; ++sl) {
+      const int g = lc - sl * G;   // the column's query head if the column is this batch element's (this sub-split's)
+      const bool mine = g >= 0 && g < G;
       const E* qr = q + ((int64_t)b * Hq + h * G + (mine ? g : 0)) * D - h * D;
       union { E e[8]; uint4 raw; } o;
 #pragma unroll
@@ -1760,7 +1764,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     {
       const int teams = Hkv * p.n_groups;
       if (fill_dies && fa_mfma::table_slices(N) == 4 && D == fa_mfma::kFusedD && G <= fa_mfma::kFusedG && teams % fa_mfma::kFusedXcds == 0 &&
-          teams / fa_mfma::kFusedXcds < Hkv && Hkv % (teams / fa_mfma::kFusedXcds) == 0 && even == ns)
+          teams / fa_mfma::kFusedXcds < Hkv && Hkv % (teams / fa_mfma::kFusedXcds) == 0)
         p.heads_per_bin = teams / fa_mfma::kFusedXcds;
     }
     const int largest = share_out_splits(p.st, Hkv, tiles, even, room, kpad, vpad, p.heads_per_bin, p.bin_of_head);
@@ -1789,11 +1793,13 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
   p.off_ilm = take(rows * p.n_il_split * 4);
   p.off_ild = take(rows * p.n_il_split * 4);
   p.off_ilo = take(rows * p.n_il_split * D * 4);
-  p.off_mm = take(rows * p.n_mid_split * 4);
-  p.off_md = take(rows * p.n_mid_split * 4);
+  // (a single sequence on the matrix-core path may run as four sub-splits per workgroup, each with partials of its own)
+  const size_t prows = mfma && B == 1 ? 4 * rows : rows;
+  p.off_mm = take(prows * p.n_mid_split * 4);
+  p.off_md = take(prows * p.n_mid_split * 4);
   // g partials: a row of 2N per (query head, split); the matrix-core path stores 16 columns per (batch group, KV head, split)
   p.off_mg = take((mfma ? (size_t)p.n_groups * Hkv * 16 : rows) * p.n_mid_split * 2 * N * 4);
-  p.off_mon = take(rows * p.n_mid_split * D * 4);
+  p.off_mon = take(prows * p.n_mid_split * D * 4);
   p.off_tab = take(mfma ? fa_mfma::tables_bytes(N) : 0);
   // merge: as many blocks per (b, KV head) as still run side by side on the device (a block fills one compute unit)
   p.n_merge_chunks = kMergeChunksMax;
@@ -1849,9 +1855,15 @@ void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bo
 }
 
 template <typename E, int KS>
-void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, hipStream_t st) {
+void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, bool sub, hipStream_t st) {
   dim3 grid(p.n_wg, p.n_groups);
-  if (fused) {
+  if (fused && sub) {
+    grid = dim3(p.n_wg * p.n_groups);
+    if (wide)
+      fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true, true><<<grid, 512, 0, st>>>(mp);
+    else
+      fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true, true><<<grid, 512, 0, st>>>(mp);
+  } else if (fused) {
     grid = dim3(p.n_wg * p.n_groups);   // numbered through wg_map
     if (wide)
       fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true><<<grid, 512, 0, st>>>(mp);
@@ -1903,7 +1915,7 @@ thread_local int g_last_call_fused = 0;   // what the last fa_decode_attn call o
 // workgroups of a team wait for each other), and the teams dealt out so that each sits on one die.  Fills wg_map.
 bool fused_merge_plan(const fa_decode_args& a, const Plan& p, uint16_t* wg_map, hipStream_t st) {
   using namespace fa_mfma;
-  if (p.path != Path::Mfma || a.no_fuse || p.n_mid_split <= 0) return false;
+  if (p.path != Path::Mfma || (a.no_fuse & 1) || p.n_mid_split <= 0) return false;
   if (table_slices(a.N) != 4 || a.D != kFusedD || a.Hq / a.Hkv > kFusedG) return false;
   if (a.dtype != FA_BF16 && a.dtype != FA_FP16) return false;
   const int total = p.n_wg * p.n_groups, n_teams = p.n_groups * a.Hkv;
@@ -1987,13 +1999,15 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   uint16_t wg_map[fa_mfma::kFusedMaxWgs] = {};
   // (the sink/window tiles must be in front of the mid rows for the merge to run inside that launch)
   const bool fused = sizeof(E) == 2 && (fuse_il || p.n_il_split == 0) && fused_merge_plan(a, p, wg_map, st);
-  g_last_call_fused = fused ? 1 : 0;
+  // one sequence: its mid rows as four sub-splits per workgroup in the places of four batch elements
+  const bool sub = fused && a.B == 1 && !(a.no_fuse & 2);
+  g_last_call_fused = fused ? (sub ? 2 : 1) : 0;
   if (p.n_mid_split > 0) {
     PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
                    a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e,
                    p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks,
                    p.path == Path::Mfma ? (E*)(ws + p.off_qn) : nullptr, a.kn_list, a.kn_h_list,
-                   fused ? (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv : nullptr};
+                   fused ? (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv : nullptr, sub ? 1 : 0};
     const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
@@ -2044,9 +2058,9 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
         if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, st);
         else switch (KS) {
-          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, fused, st); break;
-          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, fused, st); break;
-          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, fused, st); break;
+          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, fused, sub, st); break;
+          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, fused, sub, st); break;
+          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, fused, sub, st); break;
         }
       }
     } else {
@@ -2242,7 +2256,7 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
   const bool mfma = use_mfma(*a);
   const bool il_fast = il_fast_ok(*a);
   const Plan p = make_plan(a->B, a->Hq, a->Hkv, a->D, a->N > 0 ? a->N : 1, a->il_rows[0] + a->il_rows[1], a->L_m, mfma,
-                           il_fast, a->k_pad_h_host, a->v_pad_h_host, false, !a->no_fuse);
+                           il_fast, a->k_pad_h_host, a->v_pad_h_host, false, !(a->no_fuse & 1));
   FA_REQUIRE(a->workspace && a->workspace_bytes >= p.total, FA_ERR_WORKSPACE, "fa_decode_attn: workspace %zu < %zu",
              a->workspace_bytes, p.total);
   FA_REQUIRE(((uintptr_t)a->workspace & 255) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: workspace not 256-byte aligned");

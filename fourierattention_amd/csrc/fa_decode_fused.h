@@ -168,7 +168,11 @@ struct FusedShare {
 // split classes of the g sums and the sink/window sums), where each dim comes from, statistics of the compressed dims
 __host__ __device__ __forceinline__ int fused_tail_lds_floats(int n_parts) { return 2 * 16 * n_parts + 32 + 2048 + 8192 + 128 + 384; }
 
-template <typename P>
+// SUB: the team belongs to one batch element whose mid rows were cut into four sub-splits per workgroup (see the
+// mid-row kernel): the sixteen column slots are (sub-split, query head), all of them multiply with the V coefficients
+// of that one batch element, so the product first adds the four sub-splits of a head and the threads that would
+// have taken the other batch elements take further row classes instead.
+template <bool SUB, typename P>
 __device__ __forceinline__ FusedShare fused_share(const P& p, int vc0, int vc_len, int split, int n_s, int b0, int nb, int KS,
                                                   int tid) {
   FusedShare f;
@@ -187,9 +191,9 @@ __device__ __forceinline__ FusedShare fused_share(const P& p, int vc0, int vc_le
   f.nqp = nqp;
   f.lq = lq;
   f.q = tid & (nqp - 1);
-  f.bbslot = (tid >> lq) & 3;
-  f.rc = tid >> (lq + 2);
-  f.n_rc = 128 >> lq;
+  f.bbslot = SUB ? 0 : (tid >> lq) & 3;
+  f.rc = SUB ? tid >> lq : tid >> (lq + 2);
+  f.n_rc = (SUB ? 512 : 128) >> lq;
   f.v_on = f.vc_len > 0 && f.bbslot < nb && 4 * f.q < f.vc_len && f.t1 > f.t0;
   // every thread reads 16 bytes per row (4-byte aligned: the head's columns start anywhere); the group that would
   // reach past the head's columns starts early instead and its values are moved down when they are used
@@ -218,7 +222,7 @@ __device__ __forceinline__ float4v fused_v_place(float4v v, int back) {
 // waited for.  P: the mid-row kernel's parameter block (pm, pd, pg, pon, n_split, shape) with the FusedParams in
 // P::fz.  sm: LDS of at least fused_tail_lds_floats(n_split + n_il) floats that no wave uses any more.  KS: ksteps per
 // frequency slice.
-template <typename E, typename P>
+template <typename E, bool SUB, typename P>
 __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_flag, const FusedShare& f, int grp, int h,
                                                  int split, int n_s, int b0, int nb, int KS) {
   constexpr int D = kFusedD, GS = kFusedG;
@@ -235,8 +239,11 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
   float* s_stat = (float*)(s_src + 128);   // [3][128] scale, avg_u, avg_d of the compressed dims of the column share
   unsigned* cnt = p.fz.cnt + (int64_t)(grp * p.Hkv + h) * 2;
   const int vn0 = p.vn_h[h], vn_len = p.vn_h[h + 1] - vn0;
-  auto slot_ok = [&](int c16) { return (c16 >> 2) < nb && (c16 & 3) < G; };
-  auto qrow_of = [&](int c16) { return (int64_t)(b0 + (c16 >> 2)) * p.Hq + h * G + (c16 & 3); };
+  // column slot c16 = 4 * batch element of the group + query head; SUB: 4 * sub-split + query head, the partials of
+  // sub-split j being those of the virtual batch element 4 b0 + j and the sink/window tiles belonging to slot j = 0
+  auto slot_ok = [&](int c16) { return (SUB || (c16 >> 2) < nb) && (c16 & 3) < G; };
+  auto qrow_of = [&](int c16) { return (int64_t)(b0 + (SUB ? 0 : c16 >> 2)) * p.Hq + h * G + (c16 & 3); };   // the query row
+  auto prow_of = [&](int c16) { return (int64_t)((SUB ? 4 * b0 : b0) + (c16 >> 2)) * p.Hq + h * G + (c16 & 3); };   // its mid partials
   // column share: the columns are query heads g_lo .. g_lo + ncol - 1 of batch element cbb (the host only fuses when
   // the columns of a workgroup belong to one batch element)
   const int ncol = f.u_hi - f.u_lo, cbb = f.u_lo / G, g_lo = f.u_lo - cbb * G;
@@ -288,9 +295,9 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
     d_raw[u] = 0.f;
     if (idx < 16 * WS && slot_ok(c16)) {
       if (e < n_s) {
-        m_raw[u] = p.pm[qrow_of(c16) * NS + e];
-        d_raw[u] = p.pd[qrow_of(c16) * NS + e];
-      } else if (e >= NS) {
+        m_raw[u] = p.pm[prow_of(c16) * NS + e];
+        d_raw[u] = p.pd[prow_of(c16) * NS + e];
+      } else if (e >= NS && (!SUB || c16 < 4)) {
         m_raw[u] = p.fz.il_m[qrow_of(c16) * n_il + (e - NS)];
         d_raw[u] = p.fz.il_d[qrow_of(c16) * n_il + (e - NS)];
       }
@@ -303,7 +310,7 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
     const int ntb = min(kFusedTileBlock, f.t1 - f.t0);
     const int n_items = 64 * ntb, n_cls = 512 / n_items;
     const int item = tid % n_items, cls = tid / n_items;
-    if (cls < n_cls && ((item & 63) >> 2) < nb * G) {
+    if (cls < n_cls && ((item & 63) >> 2) < (SUB ? 4 : nb) * G) {
       const float* gp = g_team + (f.t0 + (item >> 6)) * 256 + (item & 63) * 4;
 #pragma unroll
       for (int u = 0; u < kFusedGPre; ++u) gv[u] = *(const float4v*)(gp + (int64_t)min(cls + u * n_cls, n_s - 1) * g_split_floats);
@@ -329,7 +336,12 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
     const int c16 = tid >> 5, e0 = tid & 31;
     const float* mrow = s_w + c16 * WS;
     float mstar = -INFINITY;
-    for (int e = 0; e < WS; ++e) mstar = fa_fmax(mstar, mrow[e]);
+    if constexpr (SUB) {   // one reference for the four sub-splits of the query head
+      for (int j = 0; j < 4; ++j)
+        for (int e = 0; e < WS; ++e) mstar = fa_fmax(mstar, s_w[(4 * j + (c16 & 3)) * WS + e]);
+    } else {
+      for (int e = 0; e < WS; ++e) mstar = fa_fmax(mstar, mrow[e]);
+    }
     float wgt[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -375,11 +387,14 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
 #pragma unroll
     for (int u = 0; u < kPre; ++u) il_pre[u] = *(const float4v*)(il_src + (int64_t)min(x_cls + 4 * u, n_il - 1) * D);
   }
+  // (SUB: class j takes all splits of sub-split j, whose partials are those of virtual batch element 4 b0 + j)
   const bool on_on = x_cl < ncol && 4 * x_d4 < vn_len;
-  const float* on_src = p.pon + (qrow0 + x_cl) * NS * D + 4 * x_d4;
+  const int on_first = SUB ? 0 : x_cls, on_step = SUB ? 1 : 4;
+  const int on_slot = SUB ? 4 * x_cls + c16_0 + x_cl : c16_0 + x_cl;
+  const float* on_src = p.pon + (SUB ? prow_of(on_slot) : qrow0 + x_cl) * NS * D + 4 * x_d4;
   if (on_on) {
 #pragma unroll
-    for (int u = 0; u < kPre; ++u) on_pre[u] = *(const float4v*)(on_src + (int64_t)min(x_cls + 4 * u, n_s - 1) * D);
+    for (int u = 0; u < kPre; ++u) on_pre[u] = *(const float4v*)(on_src + (int64_t)min(on_first + on_step * u, n_s - 1) * D);
   }
   // ---- row share: g over the team's splits, times the V coefficients -----------------------------------------------
   float4v acc[GS];
@@ -394,7 +409,7 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
       const int tl = item >> 6, rem = item & 63, lc = rem >> 2, lgp = rem & 3;
       const int c16 = (lc / G) * 4 + (lc % G);
       if (tb > f.t0) __syncthreads();   // the block before is done with s_g and s_red
-      const bool col_ok = lc < nb * G;   // (columns past the group hold nothing; their slots of s_g are never read)
+      const bool col_ok = lc < (SUB ? 4 : nb) * G;   // (columns past the group hold nothing; their slots of s_g are never read)
       auto put_g = [&](const float4v& a4) {
         const int rb = tl * 16 + 2 * lgp;
         s_g[rb * 16 + c16] = a4[0]; s_g[(rb + 8) * 16 + c16] = a4[1];
@@ -435,7 +450,9 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
         const int rows = 16 * ntb;
         auto fma_row = [&](int r, float4v v) {
           if (ragged) v = fused_v_place(v, f.v_back);
-          const float4v gq = *(const float4v*)(s_g + r * 16 + f.bbslot * 4);
+          float4v gq = *(const float4v*)(s_g + r * 16 + f.bbslot * 4);
+          if constexpr (SUB)   // the four sub-splits of a query head meet here
+            gq = (gq + *(const float4v*)(s_g + r * 16 + 4)) + (*(const float4v*)(s_g + r * 16 + 8) + *(const float4v*)(s_g + r * 16 + 12));
 #pragma unroll
           for (int g = 0; g < GS; ++g) acc[g] += v * gq[g];
         };
@@ -471,11 +488,11 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
     *(float4v*)(s_red + ((x_cls * 4 + x_cl) * 32 + x_d4) * 4) = a4;
     a4 = float4v{0.f, 0.f, 0.f, 0.f};
     if (on_on) {
-      const float* wg = s_w + (c16_0 + x_cl) * WS;
+      const float* wg = s_w + on_slot * WS;
 #pragma unroll
       for (int u = 0; u < kPre; ++u)
-        if (x_cls + 4 * u < n_s) a4 += on_pre[u] * wg[x_cls + 4 * u];
-      for (int sp = x_cls + 4 * kPre; sp < n_s; sp += 4) a4 += *(const float4v*)(on_src + (int64_t)sp * D) * wg[sp];
+        if (on_first + on_step * u < n_s) a4 += on_pre[u] * wg[on_first + on_step * u];
+      for (int sp = on_first + on_step * kPre; sp < n_s; sp += on_step) a4 += *(const float4v*)(on_src + (int64_t)sp * D) * wg[sp];
     }
     *(float4v*)(s_g + ((x_cls * 4 + x_cl) * 32 + x_d4) * 4) = a4;
   }
@@ -496,15 +513,17 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
   if (has_coef) {
     if (f.v_on) {
 #pragma unroll
-      for (int g = 0; g < GS; ++g) *(float4v*)(s_red + ((f.rc * 4 + f.bbslot) * GS + g) * 4 * f.nqp + 4 * f.q) = acc[g];
+      for (int g = 0; g < GS; ++g) *(float4v*)(s_red + ((f.rc * (SUB ? 1 : 4) + f.bbslot) * GS + g) * 4 * f.nqp + 4 * f.q) = acc[g];
     }
     __syncthreads();
     float* pc = pc_team + (int64_t)split * 16 * 128;
-    for (int idx = tid; idx < 16 * f.nqp; idx += 512) {
+    // (SUB: the row classes hold four slots each, those of the query heads)
+    constexpr int kSlots = SUB ? 4 : 16;
+    for (int idx = tid; idx < kSlots * f.nqp; idx += 512) {
       const int c16 = idx >> f.lq, q = idx & (f.nqp - 1);
       if (4 * q < f.vc_len && slot_ok(c16)) {
         float4v a4 = float4v{0.f, 0.f, 0.f, 0.f};
-        for (int rc = 0; rc < f.n_rc; ++rc) a4 += *(const float4v*)(s_red + (rc * 16 + c16) * 4 * f.nqp + 4 * q);
+        for (int rc = 0; rc < f.n_rc; ++rc) a4 += *(const float4v*)(s_red + (rc * kSlots + c16) * 4 * f.nqp + 4 * q);
         *(float4v*)(pc + c16 * 128 + 4 * q) = a4;
       }
     }
@@ -528,10 +547,13 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
         for (int u = 0; u < 8; ++u)
           if (z0 + u < n_blocks) sum += t[u];
       }
-      const float pmid = s_sc[16 + c16_0 + o_cl];
+      float pmid = s_sc[16 + c16_0 + o_cl];
+      if constexpr (SUB) pmid = (pmid + s_sc[20 + c16_0 + o_cl]) + (s_sc[24 + c16_0 + o_cl] + s_sc[28 + c16_0 + o_cl]);
       o_val += s_stat[o_src] * (sum * (1.0f / (float)N) - s_stat[256 + o_src] * pmid) + s_stat[128 + o_src] * pmid;
     }
-    o_val *= 1.0f / s_sc[c16_0 + o_cl];
+    float den = s_sc[c16_0 + o_cl];
+    if constexpr (SUB) den = (den + s_sc[4 + c16_0 + o_cl]) + (s_sc[8 + c16_0 + o_cl] + s_sc[12 + c16_0 + o_cl]);
+    o_val *= 1.0f / den;
     const int64_t at = (qrow0 + o_cl) * D + o_d;
     if (p.fz.out) p.fz.out[at] = o_val;
     if constexpr (sizeof(E) == 2) {

@@ -274,10 +274,19 @@ struct MidParams {
 //         history; waves 0-3 stream V.  No exchange between the waves at all.
 // FUSE (MODE 0 only): the launch merges its own partials and writes the output rows, see fa_decode_fused.h; the
 // workgroups are then numbered through p.fz.wg_map so that the splits of a (batch group, KV head) share one die.
-template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false>
+// SUB (FUSE only, a batch of one sequence, at most four query heads per KV head): a single batch element would
+// leave twelve of the sixteen matrix-core columns and three of the four page streams of a workgroup idle.  The
+// workgroup's pages are cut into four sub-splits instead, which take the places of four batch elements: wave i
+// streams the pages of sub-split i, column 4 j' + g (j' = sub-split, as a batch element would be) holds query head g
+// with its weights W' rotated to the first frame of sub-split j', and every column keeps its own softmax reference,
+// g history and outputs, i.e. each sub-split ends as a partial result of its own ("virtual batch element" j' of the
+// partial buffers).  The page loop has a quarter of the trips.  Pages past the end of a sub-split are fetched from a
+// valid page and masked.
+template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false, bool SUB = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
   static_assert(!FUSE || MODE == 0, "the fused merge runs behind the one-pass pipeline");
+  static_assert(!SUB || FUSE, "sub-splits end in the fused merge");
   constexpr int NSL = MODE == 0 ? kFreqWaves : 2 * kFreqWaves;   // frequency slices
   using M = Mma<E>;
   using vec8 = typename M::vec8;
@@ -319,22 +328,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   const int G = p.G, N = p.N;
   const int b0 = grp * p.nbpg;
-  const int nb = min(p.nbpg, p.B - b0);
+  const int nb_real = min(p.nbpg, p.B - b0);
+  const int nb = SUB ? 4 : nb_real;   // SUB: four sub-splits of the one batch element in the places of batch elements
   const int R = nb * G;
   const bool valid_r = lc < R;
   const int bb_r = lc / G, g_r = lc - bb_r * G;
-  const int64_t qrow = valid_r ? ((int64_t)(b0 + bb_r) * p.Hq + h * G + g_r) : 0;
-  if (MODE != 1 && split == 0 && tid < nb && p.merge_count) p.merge_count[(b0 + tid) * p.Hkv + h] = 0u;
+  // the query row of this lane's column; the row of its partial results (SUB: virtual batch element 4 b + sub-split)
+  const int64_t qrow = valid_r ? ((int64_t)(b0 + (SUB ? 0 : bb_r)) * p.Hq + h * G + g_r) : 0;
+  const int64_t prow = !SUB ? qrow : valid_r ? ((int64_t)(b0 * 4 + bb_r) * p.Hq + h * G + g_r) : 0;
+  if (MODE != 1 && split == 0 && tid < nb_real && p.merge_count) p.merge_count[(b0 + tid) * p.Hkv + h] = 0u;
   const int fbase = sl * 16 * KS;
   const bool has_mn = sl < nb && sl < kFreqWaves;
-  const int my_b = b0 + (has_mn ? sl : 0);
+  const int my_b = b0 + (has_mn && !SUB ? sl : 0);
   const int stw = has_mn ? w & 3 : 0;   // page stage of this wave
 
   const int n_tiles = (p.L_m + 31) >> 5;
   const int tiles_per_split = (n_tiles + p.st.n[h] - 1) / p.st.n[h];
   const int t_beg = split * tiles_per_split;
   const int t_end = min(n_tiles, t_beg + tiles_per_split);
-  const int n_it = t_end > t_beg ? t_end - t_beg : 0;
+  const int n_pages = t_end > t_beg ? t_end - t_beg : 0;
+  // trips of the page loop; SUB: a quarter of the pages per sub-split, the sub-split of this wave (wave-uniform) and
+  // of this lane's column start at page w_beg / c_beg of the split, and the column's has c_n pages
+  const int n_it = SUB ? (n_pages + 3) >> 2 : n_pages;
+  const int w_beg = SUB ? min(n_pages, (w & 3) * n_it) : 0;
+  const int c_beg = SUB ? min(n_pages, min(bb_r, 3) * n_it) : 0;
+  const int c_n = SUB ? min(n_pages, c_beg + n_it) - c_beg : n_pages;
+  const int t_beg_w = t_beg + w_beg;
   // fused merge: the head's compressed V dims (offset into the lists, count), needed behind the page loop
   int fz_vc0 = 0, fz_vc_len = 0;
   if constexpr (FUSE) {
@@ -375,9 +394,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool has_k = has_mn && nks > 0;
     // a page moves the fragments the head really has
     // (mirrored page: token 31 - i becomes row i, i.e. the blocks change places and their rows are reversed)
-    auto issue_k = [&](int t, bool mir) {   // page t -> stage (t - t_beg) % NST
-      const E* kp = kbase + (int64_t)t * dpk * 32 + (mir ? lane_krev : lane_nat);
-      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
+    auto issue_k = [&](int t, bool mir) {   // page t -> stage (t - t_beg_w) % NST
+      const int tp = SUB ? min(t, n_tiles - 1) : t;   // (a page past the sub-split: any valid page, masked later)
+      const E* kp = kbase + (int64_t)tp * dpk * 32 + (mir ? lane_krev : lane_nat);
+      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg_w) % NST][0];
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
@@ -395,7 +415,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // the lanes of other batch elements and past the head's count): requested behind the weights
     vec8 Qb[KMAX];
     {
-      const float2v* wl = (const float2v*)p.W + ((int64_t)((grp * p.Hkv + h) * NSL + sl) * 2 * KS * 2) * 64 + (lc * 4 + lg);
+      // (SUB: every sub-split starts from the weights of its query head, column g of the one batch element)
+      const float2v* wl = (const float2v*)p.W + ((int64_t)((grp * p.Hkv + h) * NSL + sl) * 2 * KS * 2) * 64 + ((SUB ? g_r : lc) * 4 + lg);
       float2v wc2[2 * KS], ws2[2 * KS];
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) {
@@ -418,7 +439,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (has_k) {
 #pragma unroll
         for (int i = 0; i < NST - 1; ++i)
-          if (i < n_it) issue_k(t_beg + i, (i & 1) == 0);
+          if (i < n_it) issue_k(t_beg_w + i, (i & 1) == 0);
       }
 #pragma unroll
       for (int rt = 0; rt < 2 * KS; ++rt) {
@@ -438,7 +459,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     {
       // phases of the first frame centre (token 32 (t_beg + 1) - 1/2, as a count of half tokens against 2T): exact
       // for row tile 0, then stepped by the (exact) phase of 8 frequencies
-      const int64_t c2 = (int64_t)64 * (t_beg + 1) - 1;
+      const int64_t c2 = (int64_t)64 * (t_beg + c_beg + 1) - 1;   // (SUB: of the column's sub-split)
       float sn[2], co[2], s8, c8;
       fast_sincos_phase(8, c2, 2 * p.T, &s8, &c8);
 #pragma unroll
@@ -481,7 +502,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     auto score_trip = [&](int it, auto mirrored_tag) {
       constexpr bool mirrored = decltype(mirrored_tag)::value;   // first page of its frame
       if (it < n_it) {
-        const int t = t_beg + it;
+        const int t = t_beg_w + it;
         uint4v kraw[4];   // two ksteps of both token blocks at a time
         const unsigned kst = lds_addr_of(&s_stage[MODE == 0 ? w : stw][it % NST][0]) + lane * 16;
         uint4v rc[2][4];
@@ -597,9 +618,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const E* vbase = p.v_mid + (int64_t)my_b * p.v_bs + (int64_t)vp0 * 32 * p.cap_pages;  // wave-uniform
     const bool streams_v = has_mn && ndg > 0;
     // (mirrored page: lane group lg takes the tokens of group 3 - lg; the probabilities follow, see below)
-    auto issue_v = [&](int t, bool mir) {   // page t -> stage (t - t_beg) % NST
-      const E* vp = vbase + (int64_t)t * dpv * 32 + (mir ? lane_vrev : lane_nat);
-      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg) % NST][0];
+    auto issue_v = [&](int t, bool mir) {   // page t -> stage (t - t_beg_w) % NST
+      const int tp = SUB ? min(t, n_tiles - 1) : t;
+      const E* vp = vbase + (int64_t)tp * dpv * 32 + (mir ? lane_vrev : lane_nat);
+      unsigned char* st = &s_stage[MODE == 0 ? w : stw][(t - t_beg_w) % NST][0];
 #pragma unroll
       for (int f = 0; f < VMAX; ++f)
         if (f < ndg) load_frag_to_lds<2>(vp + f * 512, st + f * 1024);
@@ -622,7 +644,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int i = 0; i < NST - 1; ++i)
       if (i < n_it) {
-        if (streams_v) issue_v(t_beg + i, (i & 1) == 0);
+        if (streams_v) issue_v(t_beg_w + i, (i & 1) == 0);
         issue_sc(i);
       }
     rot_store();
@@ -649,7 +671,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // (whether this wave streams V is fixed for the whole loop: a parameter of the body, not a branch in it)
     auto value_page = [&](int it, auto first_tag, auto stream_tag) {
         constexpr bool has_v = decltype(stream_tag)::value;
-        const int t = t_beg + it - 1, buf = (it - 1) & 1;
+        const int t = t_beg_w + it - 1, buf = (it - 1) & 1;
         const int pg = it - 1;   // page index within the split
         constexpr int RCB = VMAX > 4 ? 1 : 2;   // the wide variant has no registers to spare for a second batch
         constexpr bool first_of_frame = decltype(first_tag)::value;   // the mirrored page of a frame (rotates), or the second
@@ -737,7 +759,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             sc[e] = __builtin_bit_cast(float, u);
           }
         }
-        if (ragged_tail && t == n_tiles - 1) {
+        if constexpr (SUB) {
+          // this lane's column belongs to a sub-split of its own: past its last page nothing counts
+          const int tc = t_beg + c_beg + pg;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int tok = tc * 32 + (first_of_frame ? 31 - 8 * lg - e : 8 * lg + e);
+            if (pg >= c_n || tok >= p.L_m) sc[e] = -INFINITY;
+          }
+        } else if (ragged_tail && t == n_tiles - 1) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int tok = t * 32 + (first_of_frame ? 31 - 8 * lg - e : 8 * lg + e);
@@ -838,11 +868,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // ---- partials of this split ------------------------------------------------------
     const float dsum = fa_rows_sum(d_run);
+    // SUB: a column whose sub-split has no page has seen masked scores only; what it accumulated is not a number
+    const bool c_none = SUB && c_n == 0;
     if (valid_r) {
-      const int64_t base = qrow * p.n_split + split;
+      const int64_t base = prow * p.n_split + split;
       if (sl == 0 && lg == 0) {
-        p.pm[base] = m_run;
-        p.pd[base] = dsum;
+        p.pm[base] = c_none ? -INFINITY : m_run;
+        p.pd[base] = c_none ? 0.f : dsum;
       }
     }
     {
@@ -853,7 +885,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       // past the group store values that nobody reads.
       float4v* gl = (float4v*)p.pg + ((((int64_t)(grp * p.Hkv + h) * p.n_split + split) * NSL + sl) * 2 * KS) * 64 + lc * 4;
       // twice the centre of the last frame, in half tokens
-      const int64_t c2 = (int64_t)64 * (t_beg + (n_it > 0 ? ((n_it - 1) & ~1) : 0) + 1) - 1;
+      const int64_t c2 = (int64_t)64 * (t_beg + c_beg + (n_it > 0 ? ((n_it - 1) & ~1) : 0) + 1) - 1;
       float sn[4], co[4], s16, c16;   // stepped phases, as for the first frame of the score waves
       fast_sincos_phase(16, c2, 2 * p.T, &s16, &c16);
 #pragma unroll
@@ -870,6 +902,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             o[2 * f2] = co[v] * x - sn[v] * y;
             o[2 * f2 + 1] = sn[v] * x + co[v] * y;
           }
+          if (c_none) o = float4v{0.f, 0.f, 0.f, 0.f};
           gl[(2 * j + (lg >> 1)) * 64 + 2 * (lg & 1) + h2] = o;
         }
 #pragma unroll
@@ -881,19 +914,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
     if (valid_r) {
-      const int64_t base = qrow * p.n_split + split;
+      const int64_t base = prow * p.n_split + split;
       if (has_mn && bb_r == sl) {
         // rows of D floats: dims past the head's stored count are written too (zeros, never read)
         float* on = p.pon + base * p.D;
 #pragma unroll
         for (int f = 0; f < VMAX; ++f)
-          if (f < ndg) *(float4v*)&on[f * 16 + 4 * lg] = oacc[f];
+          if (f < ndg) *(float4v*)&on[f * 16 + 4 * lg] = c_none ? float4v{0.f, 0.f, 0.f, 0.f} : oacc[f];
       }
     }
   }
   if constexpr (FUSE) {
-    const FusedShare fs = fused_share(p, fz_vc0, fz_vc_len, split, p.st.n[h], b0, nb, KS, tid);
-    fused_merge_tail<E>(p, (float*)&s_stage[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb, KS);
+    const FusedShare fs = fused_share<SUB>(p, fz_vc0, fz_vc_len, split, p.st.n[h], b0, nb_real, KS, tid);
+    fused_merge_tail<E, SUB>(p, (float*)&s_stage[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb_real, KS);
   }
 }
 

@@ -410,7 +410,8 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     ``balance_heads``: hand the per-head padded dim counts of a paged store over on the host side too, so that heads
     that store more dims get more splits (``False``: every head the same number, for comparison).
     ``no_fuse``: keep the sink/window tiles, the mid rows and the merge as launches of their own where the library
-    would run them as one (for comparison)."""
+    would run them as one (for comparison); an int is passed on as the bits of ``fa_decode_args.no_fuse`` (2: fused,
+    but without the four sub-splits per workgroup that a batch of one sequence otherwise runs)."""
     from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
@@ -459,7 +460,7 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
         if tables is not None:
             a.tables = tables.data_ptr()
     a.force_generic = int(bool(force_generic))
-    a.no_fuse = int(bool(no_fuse))
+    a.no_fuse = int(no_fuse)   # False / True, or the bits of fa_decode_args.no_fuse
     if seq_len_m >= _REPACK_MIN_ROWS and not force_generic:
         _warn_if_off_the_matrix_cores(q.dtype, num_head_q, num_head_kv, D, N, isinstance(k_mn, MidStore))
     a.kc_list, a.kc_h_list, a.kn_list, a.kn_h_list = kc.data_ptr(), kc_h.data_ptr(), kn.data_ptr(), kn_h.data_ptr()

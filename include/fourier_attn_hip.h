@@ -211,8 +211,9 @@ typedef struct fa_decode_args {
   int32_t dtype;      /* fa_dtype of q, k_il, v_il, k_mn, v_mn */
   void* workspace;
   size_t workspace_bytes;
-  /* != 0: never run the step as one fused launch behind the query preparation (see fa_decode_attn); the sink/window
-   * tiles, the mid rows and the merge then run as launches of their own (testing, comparison) */
+  /* bit 0: never run the merge inside the mid-row launch (see fa_decode_attn); the mid rows and the merge then run as
+   * launches of their own.  bit 1: with a batch of one sequence, keep one page stream per workgroup instead of four
+   * sub-splits.  (Both for testing and comparison.) */
   int32_t no_fuse;
 } fa_decode_args;
 
@@ -303,7 +304,9 @@ int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_s
  * [sink ; local window ; mid rows (stored dims + dims rebuilt from coefficients)].
  * Launches: query preparation + sink/window tiles, mid rows, merge.  On the one-pass matrix-core path (16-bit
  * storage, head_dim 128, at most four query heads per KV head, up to 512 frequencies) the workgroups of the mid-row
- * launch merge their own partials and write the output rows (two launches); args->no_fuse != 0 keeps the three.
+ * launch merge their own partials and write the output rows (two launches); args->no_fuse bit 0 keeps the three.
+ * With a batch of one sequence every workgroup of that launch then runs four sub-splits of its pages side by side
+ * (in the matrix-core columns and page streams that further batch elements would use).
  * That needs the device to deal the workgroups of a launch out to its dies in turn, which the first call on a device
  * checks with a tiny launch and ONE synchronisation of `stream` (skipped, and asked again by the next call, while
  * the stream is being captured). */
@@ -333,7 +336,8 @@ int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total
 int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
 
 /* Whether the last fa_decode_attn / _noalloc / _timed call of the calling thread ran the merge inside the mid-row
- * launch (1) or as a launch of its own (0).  A measurement aid (the reference has no counterpart). */
+ * launch (1; 2: with the four sub-splits per workgroup of a batch of one) or as a launch of its own (0).  A
+ * measurement aid (the reference has no counterpart). */
 int fa_decode_attn_last_fused(void);
 
 /* Same call, bracketed by HIP events on `stream`; synchronises and returns in ms_out[0..3] the
