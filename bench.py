@@ -327,6 +327,7 @@ def e2e_bench(name, device, steps=None, warmup=3):
     if not os.environ.get("FA_BENCH_LIBRARY_GEMM"):   # (set to time the decode with the GEMM library's projections)
         model.model.pack_projections()
     cache = DynamicCache(ec, device=device)
+    cache.defer_coef_update = os.environ.get("FA_BENCH_UPDATE_INSIDE_ATTENTION", "0") == "1"   # (comparison)
     t0 = time.perf_counter()
     synthetic_prefill(cache, cfg, e["B"], e["prompt"], torch.bfloat16, device, seed=0)
     torch.cuda.synchronize()
@@ -424,6 +425,9 @@ def main():
     ap.add_argument("--no-fuse", action="store_true",
                     help="run sink/window tiles, mid rows and merge as launches of their own where the library would run the "
                          "merge inside the mid-row launch (for comparison)")
+    ap.add_argument("--update-inside-attention", action="store_true",
+                    help="update_plus_attn: the streaming update leaves the rank-1 coefficient update to the attention that "
+                         "follows, which applies it while it streams the coefficients (comparison; no faster, see DESIGN.md)")
     ap.add_argument("--no-sub-splits", action="store_true",
                     help="a batch of one sequence: one page stream per workgroup instead of four sub-splits (comparison)")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
@@ -555,6 +559,8 @@ def main():
     # (fewer streamed tokens in all than the workload's max_new_tokens: the page store is sized for those and would
     # be re-paged, a one-off of about a millisecond, inside one of the loops below)
     assert 3 + 40 + 30 + 3 + 50 <= w["max_new"] or w["max_new"] < 128
+    # (the update on its own, as one launch: what a caller pays who does not attend right after it)
+    cache.defer_coef_update = False
     for _ in range(3):
         cache.update(kn, vn, 0)
     torch.cuda.synchronize()
@@ -578,6 +584,8 @@ def main():
     upd_wall = (time.perf_counter() - t0) / 30
     upd_bytes = w["B"] * 2 * w["M"] * (ck + cv) * 4
     # a decode step in use: the streaming update, then the attention over the updated cache
+    # (--update-inside-attention: the attention applies the rank-1 update of the coefficients while it streams them)
+    cache.defer_coef_update = bool(args.update_inside_attention)
     for _ in range(3):
         cache.update(kn, vn, 0)
         cache.decode_attention(q, 0, Hq, Hkv)
@@ -588,7 +596,8 @@ def main():
     stop.record()
     torch.cuda.synchronize()
     both_ms = start.elapsed_time(stop) / 50
-    result["update_plus_attn"] = {"ms_per_step": round(both_ms, 5), "algorithmic_bytes": upd_bytes + nbytes,
+    result["update_plus_attn"] = {"ms_per_step": round(both_ms, 5), "coefficient_update_inside_attention": bool(cache.defer_coef_update),
+                                  "algorithmic_bytes": upd_bytes + nbytes,
                                   "GB_s": round((upd_bytes + nbytes) / (both_ms * 1e-3) / 1e9, 1),
                                   "pct_hbm_peak": round(100.0 * (upd_bytes + nbytes) / (both_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)}
     result["stream_update"] = {"ms_per_step": round(upd_ms, 5), "wall_ms_per_step": round(upd_wall * 1e3, 5),

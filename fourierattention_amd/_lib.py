@@ -57,6 +57,8 @@ class DecodeArgs(ctypes.Structure):
         ("sm_scale", c_float), ("dtype", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("no_fuse", c_int32),
+        ("upd_k_row", c_void_p), ("upd_v_row", c_void_p), ("upd_batch_stride", c_int64), ("upd_phase", c_int64),
+        ("upd_T", c_int32),
     ]
 
 
@@ -73,6 +75,7 @@ class StreamArgs(ctypes.Structure):
         ("kn_list", c_void_p), ("kn_h_list", c_void_p), ("k_pad_h_list", c_void_p),
         ("vn_list", c_void_p), ("vn_h_list", c_void_p), ("v_pad_h_list", c_void_p),
         ("Cnk", c_int32), ("Cnv", c_int32), ("B", c_int32), ("Hkv", c_int32), ("width", c_int32), ("dtype", c_int32),
+        ("skip_coef", c_int32),
     ]
 
 
@@ -129,7 +132,7 @@ _SIGNATURES = {
 EXPORTED = tuple(_SIGNATURES)
 
 # bumped with every change of a prototype or of an argument struct (fa_abi_version in the library)
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 

@@ -60,6 +60,7 @@ class _Layer:
         self.n_local = 0
         self.n_mid = 0
         self.version = 0        # bumped by every update; lets views detect staleness
+        self.owed = None        # (window slot, phase, period): a rank-1 update the coefficients have not taken yet
 
 
 class CacheParts(Mapping):
@@ -91,6 +92,7 @@ class CacheParts(Mapping):
         if part == "init":
             return t.init
         if part == "compressed":
+            self.cache._settle_coefficients(self.layer_idx)
             return t.coef
         if part == "uncompressed":
             return t.mid.dense(layer.n_mid)
@@ -206,6 +208,10 @@ class DynamicCache(Cache):
         self.fuse_prefill = True                       # prefill: pages, coefficients and statistics from one read
         self.fuse_decode = True                        # decode: the merge inside the mid-row launch where it applies
         self.sub_splits = True                         # ... and a batch of one as four sub-splits per workgroup
+        # streaming: leave the rank-1 update of the coefficients to the next decode_attention of the layer, which
+        # streams them anyway.  Off: measured, it is no faster than the update launch (whose reads mostly hit the
+        # last-level cache behind the attention of the step before), and two launches where the merge has its own
+        self.defer_coef_update = False
         self._book = CacheBook(self._num_layers, self.numinittokens, self.maxlocallen, self.maxmidstates,
                                self.maxnewtokens, self.maxtokens)
         self._layers: List[_Layer] = [_Layer() for _ in range(self._num_layers)]
@@ -327,6 +333,10 @@ class DynamicCache(Cache):
         v = value_states.permute(0, 2, 1, 3).reshape(bsz, q_len, heads * head_dim)
         layer = self._layers[layer_idx]
         lb = self._book.layers[layer_idx]
+        if step.action in (Action.PREFILL_COMPRESS, Action.PREFILL_LOCAL):
+            layer.owed = None                       # the coefficients are rebuilt from scratch
+        else:
+            self._settle_coefficients(layer_idx)    # the row they are owed sits in the window slot written next
         local_only = lambda kk, vv: ({"k_init": None, "k_compressed": None, "k_uncompressed": None, "k_local": kk},
                                      {"v_init": None, "v_compressed": None, "v_uncompressed": None, "v_local": vv})
 
@@ -412,14 +422,32 @@ class DynamicCache(Cache):
         for t in (layer.k, layer.v):
             if layer.n_mid >= t.mid.cap_tokens:
                 t.mid.grow(layer.n_mid, 2 * t.mid.cap_tokens)
-        # one launch: coefficients and page store take the oldest row, the new token takes the spare slot
+        # one launch: coefficients and page store take the oldest row, the new token takes the spare slot.  The
+        # attention that follows streams the coefficients anyway: where it can, it is left to apply their rank-1
+        # update on the way (the evicted row stays in its window slot until the next update of the layer writes there)
+        defer = bool(self.defer_coef_update and k.is_cuda and not torch.cuda.is_current_stream_capturing())
         ops.stream_update(k[:, 0, :], v[:, 0, :], layer.k.ring, layer.v.ring, oldest, sp, layer.k.coef, layer.v.coef,
-                          l32[0], l32[4], p, self._book.t_c, layer.k.mid, layer.v.mid, layer.n_mid)
+                          l32[0], l32[4], p, self._book.t_c, layer.k.mid, layer.v.mid, layer.n_mid, skip_coef=defer)
+        if defer:
+            layer.owed = (oldest, int(p), int(self._book.t_c))
         layer.n_mid += 1
         layer.spare = oldest
         kview, vview = CacheParts(self, layer_idx, "k"), CacheParts(self, layer_idx, "v")
         self.key_cache[layer_idx], self.value_cache[layer_idx] = kview, vview
         return kview, vview
+
+    def _settle_coefficients(self, layer_idx: int) -> None:
+        """Apply the rank-1 update a streaming ``update`` left to the next ``decode_attention`` of the layer, if it
+        is still owed (somebody reads the coefficients, or the layer is updated again, before that call came)."""
+        layer = self._layers[layer_idx]
+        owed, layer.owed = layer.owed, None
+        if owed is None:
+            return
+        slot, phase, t_c = owed
+        l32 = self._lists32[layer_idx]
+        for t, cols in ((layer.k, l32[0]), (layer.v, l32[4])):
+            if cols.numel():
+                ops.coeff_update_(t.coef, t.ring[:, slot, :], cols, phase, t_c)
 
     def _store_stats(self, layer_idx, ks, ku, kd, vs, vu, vd):
         lists = (self.k_scale, self.k_layer_average, self.kd_layer_average, self.v_scale, self.v_layer_average,
@@ -458,8 +486,16 @@ class DynamicCache(Cache):
                                        num_kv_heads, 0, 1, sm_scale, timings=timings, out_dtype=out_dtype, out=out,
                                        no_alloc=no_alloc)
         segs = self._il_segments(layer)
+        pending = None
+        if layer.owed is not None:
+            if q.is_cuda and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("a coefficient update is still owed to this layer: call update() inside the capture "
+                                   "as well, or settle it before (read the layer's *_compressed part)")
+            slot, phase, t_c = layer.owed
+            layer.owed = None
+            pending = (layer.k.ring[:, slot, :], layer.v.ring[:, slot, :], phase, t_c)
         return ops.decode_attn_raw(q, segs, layer.k.coef, layer.v.coef, layer.k.mid, layer.v.mid, layer.k.stats32,
                                    layer.v.stats32, l32, num_heads, num_kv_heads, layer.n_mid, self.period_reconstruct,
                                    sm_scale, tables=self._tables, force_generic=self.force_generic, timings=timings,
                                    out_dtype=out_dtype, out=out, no_alloc=no_alloc, balance_heads=self.balance_heads,
-                                   no_fuse=(0 if self.fuse_decode else 1) | (0 if self.sub_splits else 2))
+                                   no_fuse=(0 if self.fuse_decode else 1) | (0 if self.sub_splits else 2), pending=pending)

@@ -72,10 +72,17 @@ struct PrepArgs {
   // a batch of one sequence whose mid rows run as four sub-splits per workgroup (SUB instances of the mid-row kernel):
   // the stored query dims go out four times, once for the columns of each sub-split
   int sub;
+  // A rank-1 update the K coefficients are still owed (the row that left the window, see fa_decode_args.upd_*): every
+  // coefficient is read here by exactly one thread, which adds the row's term, writes the coefficient back and goes
+  // on with the new value.  upd_row == nullptr: nothing pending.
+  const E* upd_row;
+  int64_t upd_bs, upd_phase;
+  int upd_T;
 };
 
-// LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head
-constexpr int kPrepLdsBytes = 2 * kGMax * 128 * (int)sizeof(float);
+// LDS of the query preparation: the gathered query dims times the scale / the mean terms, per query head; the
+// compressed dims of a row the coefficients are still owed
+constexpr int kPrepLdsBytes = (2 * kGMax * 128 + 128) * (int)sizeof(float);
 
 // bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx; lds: kPrepLdsBytes
 template <typename E>
@@ -93,6 +100,7 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
   const float sm_log2e = pa.sm_log2e;
   float (&s_qs)[kGMax][128] = *reinterpret_cast<float (*)[kGMax][128]>(lds);
   float (&s_qa)[kGMax][128] = *reinterpret_cast<float (*)[kGMax][128]>((float*)lds + kGMax * 128);
+  float* s_ue = (float*)lds + 2 * kGMax * 128;
   const int tid = threadIdx.x;
   const int h = blockIdx.y, b = blockIdx.z;
   const int G = Hq / Hkv;
@@ -110,6 +118,7 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
     }
     s_qs[g][j] = qs;
     s_qa[g][j] = qa;
+    if (g == 0) s_ue[j] = (pa.upd_row && j < kc_len) ? fa_to_float(pa.upd_row[(int64_t)b * pa.upd_bs + kc_list[kc0 + j]]) : 0.f;
   }
   __syncthreads();
   if (bx == 0 && tid < 2 && pa.team_cnt && b % pa.nbpg == 0) pa.team_cnt[((int64_t)(b / pa.nbpg) * Hkv + h) * 2 + tid] = 0u;
@@ -146,6 +155,21 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
   for (int i = 0; i < 32; ++i) {
     const int j = jq + 4 * i;
     v[i] = j < kc_len ? row[j] : 0.f;
+  }
+  if (pa.upd_row) {
+    // the pending rank-1 update of this row (the arithmetic of fa_stream_update / fa_coeff_update)
+    float sn, co;
+    fa_sincos_phase(n >= N ? n - N : n, pa.upd_phase, pa.upd_T, &sn, &co);
+    const float f = n >= N ? sn : co;
+    float* wrow = const_cast<float*>(row);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int j = jq + 4 * i;
+      if (j < kc_len) {
+        v[i] = v[i] + f * s_ue[j];
+        wrow[j] = v[i];
+      }
+    }
   }
   const float mul = sm_log2e / (float)N;
 #pragma unroll
@@ -2002,12 +2026,27 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   // one sequence: its mid rows as four sub-splits per workgroup in the places of four batch elements
   const bool sub = fused && a.B == 1 && !(a.no_fuse & 2);
   g_last_call_fused = fused ? (sub ? 2 : 1) : 0;
+  // A rank-1 update the coefficients are still owed: the query preparation applies it to the K coefficients it streams,
+  // the merge inside the mid-row launch to the V coefficients; where those do not run it gets a launch of its own
+  if (a.upd_k_row && a.Ck > 0 && p.n_mid_split <= 0) {
+    const int rc = fa_coeff_update(const_cast<float*>(a.k_mc), a.upd_k_row, a.dtype, a.upd_batch_stride, a.kc_list, a.B, a.N,
+                                   a.Ck, a.upd_phase, a.upd_T, (fa_stream_t)st);
+    if (rc != FA_OK) return rc;
+  }
+  // (the tail of the mid-row launch reduces its phases in 32 bits)
+  const bool upd_v_in_tail = fused && a.upd_v_row && (uint64_t)a.N * (uint64_t)a.upd_T < (1ull << 32);
+  if (a.upd_v_row && a.Cv > 0 && !upd_v_in_tail) {
+    const int rc = fa_coeff_update(const_cast<float*>(a.v_mc), a.upd_v_row, a.dtype, a.upd_batch_stride, a.vc_list, a.B, a.N,
+                                   a.Cv, a.upd_phase, a.upd_T, (fa_stream_t)st);
+    if (rc != FA_OK) return rc;
+  }
   if (p.n_mid_split > 0) {
     PrepArgs<E> pa{(const E*)a.q, a.k_mc, a.avg_k_u, a.avg_k_d, a.scale_k, a.kc_list, a.kc_h_list, W, c0,
                    a.Hq, a.Hkv, a.D, a.N, a.Ck, sm_log2e,
                    p.path == Path::Mfma ? W : nullptr, p.nbpg, p.path == Path::Mfma ? fa_mfma::table_slices(a.N) : 0, p.ks,
                    p.path == Path::Mfma ? (E*)(ws + p.off_qn) : nullptr, a.kn_list, a.kn_h_list,
-                   fused ? (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv : nullptr, sub ? 1 : 0};
+                   fused ? (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv : nullptr, sub ? 1 : 0,
+                   a.Ck > 0 ? (const E*)a.upd_k_row : nullptr, a.upd_batch_stride, a.upd_phase, a.upd_T};
     const int n_prep = fa_cdiv(2 * a.N, kPrepRows);
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
@@ -2047,6 +2086,9 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
           fz.v_mc = a.v_mc; fz.avg_u = a.avg_v_u; fz.avg_d = a.avg_v_d; fz.scale = a.scale_v;
           fz.vc_list = a.vc_list; fz.vc_h = a.vc_h_list; fz.vn_list = a.vn_list;
           fz.out = a.out; fz.out_cast = (E*)a.out_cast; fz.Cv = a.Cv;
+          fz.upd_row = a.Cv > 0 && upd_v_in_tail ? (const E*)a.upd_v_row : nullptr;
+          fz.upd_bs = a.upd_batch_stride; fz.upd_T = a.upd_T;
+          fz.upd_phase = a.upd_T > 0 ? (unsigned)(a.upd_phase % a.upd_T) : 0u;
           fz.wait_ticks = kTeamWaitTicks;
           memcpy(fz.wg_map, wg_map, sizeof(wg_map));
         }
@@ -2252,6 +2294,13 @@ static int decode_attn_impl(const fa_decode_args* a, fa_stream_t stream, hipEven
       FA_REQUIRE((((uintptr_t)a->k_mn | (uintptr_t)a->v_mn) & 15) == 0 && (a->k_mn_batch_stride & 7) == 0 &&
                      (a->v_mn_batch_stride & 7) == 0, FA_ERR_MISALIGNED, "fa_decode_attn: paged store not 16-byte aligned");
     }
+  }
+  if (a->upd_k_row || a->upd_v_row) {
+    FA_REQUIRE(a->upd_T > 0 && a->upd_phase >= 0 && a->N > 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: pending update with N=%d T=%d phase=%lld",
+               a->N, a->upd_T, (long long)a->upd_phase);
+    FA_REQUIRE(a->Ck >= 0 && a->Cv >= 0, FA_ERR_BAD_SHAPE, "fa_decode_attn: negative dim count");
+    FA_REQUIRE((a->Ck == 0 || !a->upd_k_row || (a->k_mc && a->kc_list)) && (a->Cv == 0 || !a->upd_v_row || (a->v_mc && a->vc_list)),
+               FA_ERR_NULL_POINTER, "fa_decode_attn: pending update without coefficients / column list");
   }
   const bool mfma = use_mfma(*a);
   const bool il_fast = il_fast_ok(*a);

@@ -88,6 +88,13 @@ struct FusedParams {
   float* out;         // fp32 rows and / or rows of the storage type
   E* out_cast;
   int Cv;
+  // A rank-1 update the V coefficients are still owed (the row that left the window, see fa_decode_args.upd_*): the
+  // thread that reads a coefficient for the row share - exactly one per coefficient - adds the row's term, writes the
+  // coefficient back and multiplies with the new value.  upd_row == nullptr: nothing pending.
+  const E* upd_row;
+  int64_t upd_bs;
+  unsigned upd_phase;   // already reduced modulo upd_T
+  int upd_T;
   unsigned wait_ticks;   // bound of a meeting's wait, in ticks of the 100 MHz wall clock
   // workgroup of the launch (linear index) -> team << 6 | split, numbered so that a team shares its index modulo 8
   uint16_t wg_map[kFusedMaxWgs];
@@ -221,10 +228,10 @@ __device__ __forceinline__ float4v fused_v_place(float4v v, int back) {
 // Called by every thread of the workgroup behind the page loops, with the workgroup's partials stored but not yet
 // waited for.  P: the mid-row kernel's parameter block (pm, pd, pg, pon, n_split, shape) with the FusedParams in
 // P::fz.  sm: LDS of at least fused_tail_lds_floats(n_split + n_il) floats that no wave uses any more.  KS: ksteps per
-// frequency slice.
+// frequency slice.  s_own: four more floats of LDS per thread (free behind the page loops as well).
 template <typename E, bool SUB, typename P>
-__device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_flag, const FusedShare& f, int grp, int h,
-                                                 int split, int n_s, int b0, int nb, int KS) {
+__device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s_own, int* s_flag, const FusedShare& f, int grp,
+                                                 int h, int split, int n_s, int b0, int nb, int KS) {
   constexpr int D = kFusedD, GS = kFusedG;
   const int tid = threadIdx.x;
   const int G = p.G, N = p.N, NS = p.n_split, n_il = p.fz.n_il, WS = NS + n_il;
@@ -259,6 +266,48 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
 #pragma unroll
     for (int u = 0; u < kFusedVPre; ++u) v_pre[u] = fused_v_load(p, f, f.t0, min(f.rc + u * f.n_rc, rows - 1));
   }
+  // a pending rank-1 update of the V coefficients: this thread's four dims of the row that left the window, which of
+  // the four loaded values are its own (a group that started early overlaps its neighbour's; a head with one to
+  // three such dims repeats its last), and the update itself for local row r of the tile block at tb
+  const bool upd = p.fz.upd_row != nullptr;   // (uniform)
+  int ue_own = 0;
+  if (upd && f.v_on) {
+    const E* ur = p.fz.upd_row + (int64_t)(b0 + f.bbslot) * p.fz.upd_bs;
+    const int d0 = 4 * f.q - f.v_back;
+    float4v ue;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      ue[c] = fa_to_float(ur[p.fz.vc_list[f.vc0 + min(d0 + c, f.vc_len - 1)]]);
+      if (c >= f.v_back && d0 + c < f.vc_len) ue_own |= 1 << c;
+    }
+    *(float4v*)(s_own + 4 * tid) = ue;   // (kept in LDS until the row share: registers are scarce in between)
+  }
+  // (the host hands over the phase reduced modulo the period and only when N * period fits 32 bits)
+  // cos or sin(2 pi n p / T) for local row r of the tile block at tb, by the hardware's sine / cosine of revolutions
+  // (within 1e-7 of the library routine that fa_coeff_update calls)
+  auto owed_factor = [&](int tb, int r) -> float {
+    const int grow = fused_v_row(tb, r, N), fr = grow >= N ? grow - N : grow;
+    const float x = (float)(((unsigned)fr * p.fz.upd_phase) % (unsigned)p.fz.upd_T) / (float)p.fz.upd_T;
+    return grow >= N ? __builtin_amdgcn_sinf(x) : __builtin_amdgcn_cosf(x);
+  };
+  // the coefficient with the row's term added, written back where the thread owns it (no wait: nobody reads it again
+  // in this launch).  Applied where the row is used, behind the meeting: the wait for the team does not start behind
+  // the arrival of the rows requested ahead.
+  auto owed = [&](int tb, int r, float4v v, float fct, const float4v& ue) -> float4v {
+    float* wp = const_cast<float*>(f.vp) + (int64_t)fused_v_row(tb, r, N) * p.fz.Cv;
+    if (ue_own == 15) {
+      v = v + fct * ue;
+      *(float4u*)wp = v;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if ((ue_own >> c) & 1) {
+          v[c] = v[c] + fct * ue[c];
+          wp[c] = v[c];
+        }
+    }
+    return v;
+  };
   // where the dims of the head come from, and the statistics of the compressed dims of the column share
   int src_dim = -1;
   float st_scale = 0.f, st_au = 0.f, st_ad = 0.f;
@@ -402,6 +451,8 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
   for (int g = 0; g < GS; ++g) acc[g] = float4v{0.f, 0.f, 0.f, 0.f};
   if (has_coef) {
     const bool ragged = (f.vc_len & 3) != 0;   // (uniform: only then some group of four started early)
+    float4v ue = float4v{0.f, 0.f, 0.f, 0.f};
+    if (upd && f.v_on) ue = *(const float4v*)(s_own + 4 * tid);
     for (int tb = f.t0; tb < f.t1; tb += kFusedTileBlock) {
       const int ntb = min(kFusedTileBlock, f.t1 - tb);
       const int n_items = 64 * ntb, n_cls = 512 / n_items;
@@ -460,7 +511,17 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
         if (tb == f.t0) {   // the rows requested ahead
 #pragma unroll
           for (int u = 0; u < kFusedVPre; ++u)
-            if (f.rc + u * f.n_rc < rows) fma_row(f.rc + u * f.n_rc, v_pre[u]);
+            if (f.rc + u * f.n_rc < rows) {
+              // (opaque here: otherwise every way fused_v_place can move these rows is worked out ahead of the loop
+              // and held in registers)
+              asm volatile("" : "+v"(v_pre[u]));
+              if (upd) {
+                int tbo = tb;   // (opaque as well: the factors are not to be worked out ahead of the loop either)
+                asm volatile("" : "+s"(tbo));
+                v_pre[u] = owed(tbo, f.rc + u * f.n_rc, v_pre[u], owed_factor(tbo, f.rc + u * f.n_rc), ue);
+              }
+              fma_row(f.rc + u * f.n_rc, v_pre[u]);
+            }
           r = f.rc + kFusedVPre * f.n_rc;
         }
         for (; r < rows; r += 4 * f.n_rc) {
@@ -469,7 +530,10 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, int* s_f
           for (int u = 0; u < 4; ++u) v[u] = fused_v_load(p, f, tb, min(r + u * f.n_rc, rows - 1));
 #pragma unroll
           for (int u = 0; u < 4; ++u)
-            if (r + u * f.n_rc < rows) fma_row(r + u * f.n_rc, v[u]);
+            if (r + u * f.n_rc < rows) {
+              if (upd) v[u] = owed(tb, r + u * f.n_rc, v[u], owed_factor(tb, r + u * f.n_rc), ue);
+              fma_row(r + u * f.n_rc, v[u]);
+            }
         }
       }
     }

@@ -926,7 +926,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   if constexpr (FUSE) {
     const FusedShare fs = fused_share<SUB>(p, fz_vc0, fz_vc_len, split, p.st.n[h], b0, nb_real, KS, tid);
-    fused_merge_tail<E, SUB>(p, (float*)&s_stage[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb_real, KS);
+    fused_merge_tail<E, SUB>(p, (float*)&s_stage[0][0][0], &s_part[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb_real, KS);
   }
 }
 

@@ -24,5 +24,5 @@ int fa_check_launch(const char* what) {
 }
 
 extern "C" const char* fa_last_error_string(void) { return g_last_error; }
-extern "C" int fa_abi_version(void) { return 2; }
+extern "C" int fa_abi_version(void) { return 3; }
 extern "C" size_t fa_decode_args_size(void) { return sizeof(fa_decode_args); }

@@ -162,8 +162,9 @@ extern "C" int fa_stream_update(const fa_stream_args* a, fa_stream_t stream) {
   p.N = a->N; p.T = a->T; p.Hkv = a->Hkv; p.width = a->width; p.cap_pages = a->cap_pages;
   p.phase = a->phase; p.mid_pos = a->mid_pos;
   p.cblk_n = fa_cdiv(a->N, 64);
-  p.c_end[0] = fa_cdiv(C[0], 64) * p.cblk_n;
-  p.c_end[1] = p.c_end[0] + fa_cdiv(C[1], 64) * p.cblk_n;
+  // (skip_coef: the launch has no coefficient blocks; the caller applies the rank-1 update elsewhere)
+  p.c_end[0] = a->skip_coef ? 0 : fa_cdiv(C[0], 64) * p.cblk_n;
+  p.c_end[1] = p.c_end[0] + (a->skip_coef ? 0 : fa_cdiv(C[1], 64) * p.cblk_n);
   p.a_end[0] = p.c_end[1] + fa_cdiv(Cn[0], 256);
   p.a_end[1] = p.a_end[0] + fa_cdiv(Cn[1], 256);
   const int total = p.a_end[1] + fa_cdiv(a->width, 256);

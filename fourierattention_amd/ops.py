@@ -190,11 +190,13 @@ def coeff_update_(c: torch.Tensor, row: torch.Tensor, cols: Optional[torch.Tenso
 
 def stream_update(k_new: torch.Tensor, v_new: torch.Tensor, k_ring: torch.Tensor, v_ring: torch.Tensor, evict_slot: int,
                   write_slot: int, k_coef: torch.Tensor, v_coef: torch.Tensor, kc_list: torch.Tensor, vc_list: torch.Tensor,
-                  phase: int, T: int, k_mid, v_mid, mid_pos: int) -> None:
+                  phase: int, T: int, k_mid, v_mid, mid_pos: int, skip_coef: bool = False) -> None:
     """One streaming step of one layer in one launch (the body of cache_utils_fourier.py:731-748 for K and V):
     the rows in window slot ``evict_slot`` enter the coefficients (rank-1 update at ``phase``) and the page
     stores (at token ``mid_pos``); ``k_new, v_new (B, width)`` are written to window slot ``write_slot``.
-    ``k_ring, v_ring (B, slots, width)`` share their strides; ``k_mid, v_mid`` are ``MidStore`` objects."""
+    ``k_ring, v_ring (B, slots, width)`` share their strides; ``k_mid, v_mid`` are ``MidStore`` objects.
+    ``skip_coef``: leave the coefficients alone; the caller owes them the update (``coeff_update_``, or the
+    ``pending`` argument of the layer's next ``decode_attn_raw``) before that window slot is written again."""
     _require_gpu(k_ring, "k_ring")
     assert k_new.dim() == 2 and k_new.stride(1) == 1 and v_new.stride() == k_new.stride()
     assert k_ring.stride(2) == 1 and v_ring.stride() == k_ring.stride() and k_ring.shape == v_ring.shape
@@ -215,6 +217,7 @@ def stream_update(k_new: torch.Tensor, v_new: torch.Tensor, k_ring: torch.Tensor
     a.vn_list, a.vn_h_list, a.v_pad_h_list = _ptr(v_mid.n_list32), v_mid.n_h32.data_ptr(), v_mid.pad_h32.data_ptr()
     a.Cnk, a.Cnv = int(k_mid.Cn), int(v_mid.Cn)
     a.B, a.Hkv, a.width, a.dtype = int(k_ring.shape[0]), int(k_mid.Hkv), int(k_ring.shape[2]), dtype_code(k_ring.dtype)
+    a.skip_coef = int(bool(skip_coef))
     import ctypes
     check(_lib.load().fa_stream_update(ctypes.byref(a), _stream(k_ring.device)))
 
@@ -397,7 +400,7 @@ def decode_tables(n_f: int, period: int, device) -> Optional[torch.Tensor]:
 
 def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, lists, num_head_q, num_head_kv, seq_len_m,
                     T, sm_scale=-1.0, out=None, tables=None, force_generic=False, timings=None, out_dtype=None,
-                    no_alloc=False, balance_heads=True, no_fuse=False):
+                    no_alloc=False, balance_heads=True, no_fuse=False, pending=None):
     """Thin call into ``fa_decode_attn``.  The result is float32 like the reference's (TRI:779) unless ``out_dtype``
     names the dtype of ``q``: then the merge launch rounds it to that type itself (the caller's ``.to(dtype)``).
 
@@ -411,7 +414,10 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
     that store more dims get more splits (``False``: every head the same number, for comparison).
     ``no_fuse``: keep the sink/window tiles, the mid rows and the merge as launches of their own where the library
     would run them as one (for comparison); an int is passed on as the bits of ``fa_decode_args.no_fuse`` (2: fused,
-    but without the four sub-splits per workgroup that a batch of one sequence otherwise runs)."""
+    but without the four sub-splits per workgroup that a batch of one sequence otherwise runs).
+    ``pending``: ``(k_row, v_row, phase, T_c)``, a rank-1 update the coefficients are still owed (``stream_update``
+    with ``skip_coef``): ``k_row, v_row (B, Hkv*D)`` are the rows that left the window (same strides).  The call
+    applies it to ``k_mc`` / ``v_mc`` IN PLACE while it streams them, once; pass it to one call only."""
     from .midstore import MidStore
     _require_gpu(q, "q")
     B, q_len, feat = q.shape
@@ -459,6 +465,12 @@ def decode_attn_raw(q, il_segments, k_mc, v_mc, k_mn, v_mn, stats_k, stats_v, li
             assert t.dtype == torch.float32 and t.is_contiguous()
         if tables is not None:
             a.tables = tables.data_ptr()
+    if pending is not None:
+        uk, uv, phase, t_c = pending
+        assert seq_len_m > 0, "a layer without mid rows has no coefficients to update"
+        assert uk.dim() == 2 and uk.stride(1) == 1 and uv.stride() == uk.stride() and uk.dtype == q.dtype == uv.dtype
+        a.upd_k_row, a.upd_v_row, a.upd_batch_stride = uk.data_ptr(), uv.data_ptr(), uk.stride(0)
+        a.upd_phase, a.upd_T = int(phase), int(t_c)
     a.force_generic = int(bool(force_generic))
     a.no_fuse = int(no_fuse)   # False / True, or the bits of fa_decode_args.no_fuse
     if seq_len_m >= _REPACK_MIN_ROWS and not force_generic:

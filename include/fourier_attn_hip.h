@@ -137,6 +137,11 @@ typedef struct fa_stream_args {
   const int32_t* vn_list; const int32_t* vn_h_list; const int32_t* v_pad_h_list;
   int32_t Cnk, Cnv;
   int32_t B, Hkv, width, dtype;
+  /* != 0: leave the coefficients alone (page stores and window are updated as always).  The caller owes them the
+   * rank-1 update of the row in `evict_slot` at `phase`: fa_coeff_update, or the next fa_decode_attn of the layer
+   * through its upd_* arguments, which applies it while it streams the coefficients anyway.  The row stays in its
+   * window slot until the next fa_stream_update of the layer writes there. */
+  int32_t skip_coef;
 } fa_stream_args;
 
 int fa_stream_update(const fa_stream_args* args, fa_stream_t stream);
@@ -215,6 +220,18 @@ typedef struct fa_decode_args {
    * launches of their own.  bit 1: with a batch of one sequence, keep one page stream per workgroup instead of four
    * sub-splits.  (Both for testing and comparison.) */
   int32_t no_fuse;
+  /* A rank-1 update that the coefficients are still owed (fa_stream_update with skip_coef), applied by this call
+   * before it uses them: k_mc[b, n, j] += cos(2 pi n p / upd_T) x_k[b, kc_list[j]] and k_mc[b, N + n, j] += sin(...),
+   * likewise v_mc with x_v and vc_list (CACHE:731-748 with TRI:853-856, K = 1).  upd_k_row / upd_v_row: the rows
+   * x_k, x_v (B, Hkv*D) of `dtype` that left the window, batch stride upd_batch_stride elements; p = upd_phase.
+   * Both NULL: nothing pending.  k_mc and v_mc are WRITTEN then, once: a second call with the same upd_* arguments
+   * would apply the update again.  No counterpart in the reference, which updates in `update` (a launch of its
+   * own) what the attention that follows reads again. */
+  const void* upd_k_row;
+  const void* upd_v_row;
+  int64_t upd_batch_stride;
+  int64_t upd_phase;
+  int32_t upd_T;
 } fa_decode_args;
 
 /* sizeof(fa_decode_args) as this library was built: lets a foreign-language binding
