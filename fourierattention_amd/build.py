@@ -95,8 +95,8 @@ def audit_async_lds_reads(asm_text: str):
 
 # kernels in which one workgroup hands data to another inside a launch: it stores, waits for the stores, then counts
 # itself in with an atomic (decode_merge_rows_kernel; the instances of decode_mid_mfma_kernel that merge their own
-# partials, whose template argument list ends in `true`)
-HANDOVER_KERNELS = (re.compile(r"decode_merge_rows_kernel"), re.compile(r"decode_mid_mfma_kernel\S*Lb1EEEv"))
+# partials: the third from last of their template arguments, FUSE, is `true`)
+HANDOVER_KERNELS = (re.compile(r"decode_merge_rows_kernel"), re.compile(r"decode_mid_mfma_kernel\S*Lb1ELb[01]ELb[01]EEEv"))
 _STORE_OPS = ("global_store", "buffer_store", "flat_store")
 
 
@@ -142,6 +142,21 @@ def audit_handover_stores(asm_text: str, kernels=HANDOVER_KERNELS):
 
 # sources whose kernels issue LDS reads from inline asm (directly or through fa_decode_mfma.h): their assembly must
 # show such reads, or the audit above has looked at nothing
+def kernels_with_atomics_outside(asm_text: str, kernels=HANDOVER_KERNELS):
+    """Kernels of a listing that issue a ``global_atomic_add`` but are not among the kernels ``audit_handover_stores``
+    looks at: a hand-over the audit does not know of (a new kernel, or a kernel whose name no longer matches)."""
+    out, kernel = [], None
+    for line in asm_text.split("\n"):
+        mk = re.match(r"^(_Z\S+):", line)
+        if mk:
+            kernel = mk.group(1)
+            continue
+        if kernel and line.strip().startswith("global_atomic_add") and not any(k.search(kernel) for k in kernels):
+            if kernel not in out:
+                out.append(kernel)
+    return out
+
+
 ASYNC_LDS_SOURCES = ("fa_decode", "fa_prefill", "fa_spectral_mfma")
 HANDOVER_SOURCES = ("fa_decode",)
 
@@ -182,6 +197,9 @@ def audit_listings(base: str, listings) -> list:
         if atomics == 0:
             found.append(f"{base}: no counting atomic found in the kernels that hand data between workgroups "
                          "(kernel names or spellings the scan relies on have changed)")
+        for text in listings:
+            for k in kernels_with_atomics_outside(text):
+                found.append(f"{base}: {k} issues a counting atomic but is not among the kernels whose hand-over is audited")
     return found
 
 

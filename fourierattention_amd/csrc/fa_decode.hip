@@ -85,7 +85,9 @@ struct PrepArgs {
 constexpr int kPrepLdsBytes = (2 * kGMax * 128 + 128) * (int)sizeof(float);
 
 // bx: block index along x (row chunk of kPrepRows coefficient rows); y, z come from blockIdx; lds: kPrepLdsBytes
-template <typename E>
+// UPD: a rank-1 update of the K coefficients is pending (an instance of its own: the code for it costs the launch
+// 2 us even when it does not run)
+template <typename E, bool UPD>
 __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, void* lds) {
   const E* __restrict__ q = pa.q;
   const float* __restrict__ k_mc = pa.k_mc;
@@ -118,7 +120,8 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
     }
     s_qs[g][j] = qs;
     s_qa[g][j] = qa;
-    if (g == 0) s_ue[j] = (pa.upd_row && j < kc_len) ? fa_to_float(pa.upd_row[(int64_t)b * pa.upd_bs + kc_list[kc0 + j]]) : 0.f;
+    if constexpr (UPD)
+      if (g == 0) s_ue[j] = j < kc_len ? fa_to_float(pa.upd_row[(int64_t)b * pa.upd_bs + kc_list[kc0 + j]]) : 0.f;
   }
   __syncthreads();
   if (bx == 0 && tid < 2 && pa.team_cnt && b % pa.nbpg == 0) pa.team_cnt[((int64_t)(b / pa.nbpg) * Hkv + h) * 2 + tid] = 0u;
@@ -156,7 +159,7 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
     const int j = jq + 4 * i;
     v[i] = j < kc_len ? row[j] : 0.f;
   }
-  if (pa.upd_row) {
+  if constexpr (UPD) {
     // the pending rank-1 update of this row (the arithmetic of fa_stream_update / fa_coeff_update)
     float sn, co;
     fa_sincos_phase(n >= N ? n - N : n, pa.upd_phase, pa.upd_T, &sn, &co);
@@ -194,10 +197,10 @@ __device__ __forceinline__ void decode_prep_body(const PrepArgs<E>& pa, int bx, 
   }
 }
 
-template <typename E>
+template <typename E, bool UPD>
 __global__ __launch_bounds__(256) void decode_prep_kernel(const PrepArgs<E> pa) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[kPrepLdsBytes];
-  decode_prep_body<E>(pa, blockIdx.x, lds);
+  decode_prep_body<E, UPD>(pa, blockIdx.x, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -1637,13 +1640,13 @@ __global__ __launch_bounds__(256) void decode_il_fast_kernel(const IlArgs<E> ia)
 // The coefficient-domain query and the sink/window rows do not depend on each other and are both short,
 // latency-bound pieces of work: one launch runs them side by side (blocks [0, n_prep) prepare the query,
 // the rest attend over sink/window tiles).
-template <typename E, int D, int GM>
+template <typename E, int D, int GM, bool UPD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GM <= 4 ? 6 : 4, GM <= 4 ? 6 : 4)))
 void decode_prep_il_kernel(const PrepArgs<E> pa, const IlArgs<E> ia, int n_prep) {
   // one buffer for whichever piece the block runs: what a block holds in LDS decides how many run side by side
   constexpr int kLds = (int)sizeof(IlFastLds<D, GM>) > kPrepLdsBytes ? (int)sizeof(IlFastLds<D, GM>) : kPrepLdsBytes;
   __shared__ __attribute__((aligned(16))) unsigned char lds[kLds];
-  if ((int)blockIdx.x < n_prep) decode_prep_body<E>(pa, blockIdx.x, lds);
+  if ((int)blockIdx.x < n_prep) decode_prep_body<E, UPD>(pa, blockIdx.x, lds);
   else decode_il_fast_body<E, D, GM>(ia, blockIdx.x - n_prep, lds);
 }
 
@@ -1881,18 +1884,20 @@ void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bo
 template <typename E, int KS>
 void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, bool sub, hipStream_t st) {
   dim3 grid(p.n_wg, p.n_groups);
-  if (fused && sub) {
-    grid = dim3(p.n_wg * p.n_groups);
-    if (wide)
-      fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true, true><<<grid, 512, 0, st>>>(mp);
-    else
-      fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true, true><<<grid, 512, 0, st>>>(mp);
-  } else if (fused) {
+  if (fused) {
     grid = dim3(p.n_wg * p.n_groups);   // numbered through wg_map
-    if (wide)
-      fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true><<<grid, 512, 0, st>>>(mp);
-    else
-      fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true><<<grid, 512, 0, st>>>(mp);
+    const bool upd = mp.fz.upd_row != nullptr;   // (instances of their own, like the query preparation's)
+    auto go = [&](auto sub_tag, auto upd_tag) {
+      constexpr bool S = decltype(sub_tag)::value, U = decltype(upd_tag)::value;
+      if (wide)
+        fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true, S, U><<<grid, 512, 0, st>>>(mp);
+      else
+        fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true, S, U><<<grid, 512, 0, st>>>(mp);
+    };
+    if (sub && upd) go(std::true_type{}, std::true_type{});
+    else if (sub) go(std::true_type{}, std::false_type{});
+    else if (upd) go(std::false_type{}, std::true_type{});
+    else go(std::false_type{}, std::false_type{});
   } else if (wide) {
     fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2><<<grid, 512, 0, st>>>(mp);
   } else {
@@ -2051,13 +2056,22 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     if (fuse_il) {
       if constexpr (sizeof(E) == 2) {
         dim3 grid(n_prep + p.n_il_split, a.Hkv, a.B);
-        if (a.D == 128 && G <= 4) decode_prep_il_kernel<E, 128, 4><<<grid, 256, 0, st>>>(pa, ia, n_prep);
-        else if (a.D == 128) decode_prep_il_kernel<E, 128, kGMax><<<grid, 256, 0, st>>>(pa, ia, n_prep);
-        else if (G <= 4) decode_prep_il_kernel<E, 64, 4><<<grid, 256, 0, st>>>(pa, ia, n_prep);
-        else decode_prep_il_kernel<E, 64, kGMax><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        if (pa.upd_row) {
+          if (a.D == 128 && G <= 4) decode_prep_il_kernel<E, 128, 4, true><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else if (a.D == 128) decode_prep_il_kernel<E, 128, kGMax, true><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else if (G <= 4) decode_prep_il_kernel<E, 64, 4, true><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else decode_prep_il_kernel<E, 64, kGMax, true><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        } else {
+          if (a.D == 128 && G <= 4) decode_prep_il_kernel<E, 128, 4, false><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else if (a.D == 128) decode_prep_il_kernel<E, 128, kGMax, false><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else if (G <= 4) decode_prep_il_kernel<E, 64, 4, false><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+          else decode_prep_il_kernel<E, 64, kGMax, false><<<grid, 256, 0, st>>>(pa, ia, n_prep);
+        }
       }
+    } else if (pa.upd_row) {
+      decode_prep_kernel<E, true><<<dim3(n_prep, a.Hkv, a.B), 256, 0, st>>>(pa);
     } else {
-      decode_prep_kernel<E><<<dim3(n_prep, a.Hkv, a.B), 256, 0, st>>>(pa);
+      decode_prep_kernel<E, false><<<dim3(n_prep, a.Hkv, a.B), 256, 0, st>>>(pa);
     }
     if (p.path == Path::Mfma) {
       if constexpr (sizeof(E) == 2) {

@@ -229,7 +229,7 @@ __device__ __forceinline__ float4v fused_v_place(float4v v, int back) {
 // waited for.  P: the mid-row kernel's parameter block (pm, pd, pg, pon, n_split, shape) with the FusedParams in
 // P::fz.  sm: LDS of at least fused_tail_lds_floats(n_split + n_il) floats that no wave uses any more.  KS: ksteps per
 // frequency slice.  s_own: four more floats of LDS per thread (free behind the page loops as well).
-template <typename E, bool SUB, typename P>
+template <typename E, bool SUB, bool UPD, typename P>
 __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s_own, int* s_flag, const FusedShare& f, int grp,
                                                  int h, int split, int n_s, int b0, int nb, int KS) {
   constexpr int D = kFusedD, GS = kFusedG;
@@ -269,7 +269,7 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
   // a pending rank-1 update of the V coefficients: this thread's four dims of the row that left the window, which of
   // the four loaded values are its own (a group that started early overlaps its neighbour's; a head with one to
   // three such dims repeats its last), and the update itself for local row r of the tile block at tb
-  const bool upd = p.fz.upd_row != nullptr;   // (uniform)
+  constexpr bool upd = UPD;   // (an instance of its own: p.fz.upd_row is set)
   int ue_own = 0;
   if (upd && f.v_on) {
     const E* ur = p.fz.upd_row + (int64_t)(b0 + f.bbslot) * p.fz.upd_bs;

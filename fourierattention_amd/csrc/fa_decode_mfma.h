@@ -282,11 +282,13 @@ struct MidParams {
 // g history and outputs, i.e. each sub-split ends as a partial result of its own ("virtual batch element" j' of the
 // partial buffers).  The page loop has a quarter of the trips.  Pages past the end of a sub-split are fetched from a
 // valid page and masked.
-template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false, bool SUB = false>
+// UPD (FUSE only): the tail also applies a pending rank-1 update to the V coefficients of its row share.
+template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false, bool SUB = false, bool UPD = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
   static_assert(!FUSE || MODE == 0, "the fused merge runs behind the one-pass pipeline");
   static_assert(!SUB || FUSE, "sub-splits end in the fused merge");
+  static_assert(!UPD || FUSE, "the pending update rides in the fused merge");
   constexpr int NSL = MODE == 0 ? kFreqWaves : 2 * kFreqWaves;   // frequency slices
   using M = Mma<E>;
   using vec8 = typename M::vec8;
@@ -926,7 +928,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   if constexpr (FUSE) {
     const FusedShare fs = fused_share<SUB>(p, fz_vc0, fz_vc_len, split, p.st.n[h], b0, nb_real, KS, tid);
-    fused_merge_tail<E, SUB>(p, (float*)&s_stage[0][0][0], &s_part[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb_real, KS);
+    fused_merge_tail<E, SUB, UPD>(p, (float*)&s_stage[0][0][0], &s_part[0][0][0], &s_team_flag, fs, grp, h, split, p.st.n[h], b0, nb_real, KS);
   }
 }
 
