@@ -379,17 +379,33 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
     s_stat[128 + tid] = st_au;
     s_stat[256 + tid] = st_ad;
   }
-  // Weights of the parts: thread (column slot, e), e + 32, ... finds the column's maximum itself (every thread of a
-  // column reads the same LDS words: broadcasts, no lane exchanges) and turns its own entries into weights in place
+  // Weights of the parts: thread (column slot, e), e + 32, ... takes the maximum of its own entries, the 32 lanes of
+  // the column find the column's maximum with lane exchanges (a loop over all entries in every thread is a chain of
+  // dependent LDS reads: 1.4 us at config 3), and each thread turns its entries into weights in place
   {
     const int c16 = tid >> 5, e0 = tid & 31;
     const float* mrow = s_w + c16 * WS;
     float mstar = -INFINITY;
-    if constexpr (SUB) {   // one reference for the four sub-splits of the query head
-      for (int j = 0; j < 4; ++j)
-        for (int e = 0; e < WS; ++e) mstar = fa_fmax(mstar, s_w[(4 * j + (c16 & 3)) * WS + e]);
-    } else {
-      for (int e = 0; e < WS; ++e) mstar = fa_fmax(mstar, mrow[e]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = e0 + 32 * u;
+      if (e < WS) {
+        if constexpr (SUB) {   // one reference for the four sub-splits of the query head
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mstar = fa_fmax(mstar, s_w[(4 * j + (c16 & 3)) * WS + e]);
+        } else {
+          mstar = fa_fmax(mstar, mrow[e]);
+        }
+      }
+    }
+    mstar = fa_fmax(mstar, fa_dpp<FA_DPP_XOR1>(mstar));
+    mstar = fa_fmax(mstar, fa_dpp<FA_DPP_XOR2>(mstar));
+    mstar = fa_fmax(mstar, fa_dpp<FA_DPP_HALF_MIRROR>(mstar));
+    mstar = fa_fmax(mstar, fa_dpp<FA_DPP_MIRROR>(mstar));
+    {
+      float lo, hi;
+      fa_swap16(mstar, &lo, &hi);
+      mstar = fa_fmax(lo, hi);
     }
     float wgt[4];
 #pragma unroll
@@ -587,7 +603,12 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
       const int c16 = idx >> f.lq, q = idx & (f.nqp - 1);
       if (4 * q < f.vc_len && slot_ok(c16)) {
         float4v a4 = float4v{0.f, 0.f, 0.f, 0.f};
-        for (int rc = 0; rc < f.n_rc; ++rc) a4 += *(const float4v*)(s_red + (rc * kSlots + c16) * 4 * f.nqp + 4 * q);
+        for (int rc = 0; rc < f.n_rc; rc += 4) {   // (a power of two, at least four; four reads in flight, fixed order)
+          float4v t[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) t[u] = *(const float4v*)(s_red + ((rc + u) * kSlots + c16) * 4 * f.nqp + 4 * q);
+          a4 += (t[0] + t[1]) + (t[2] + t[3]);
+        }
         *(float4v*)(pc + c16 * 128 + 4 * q) = a4;
       }
     }
@@ -603,12 +624,12 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
       const int n_blocks = (NT + tper - 1) / tper;   // workgroups of the team that own coefficient rows
       const float* src = pc_team + (c16_0 + o_cl) * 128 + o_src;
       float sum = 0.f;
-      for (int z0 = 0; z0 < n_blocks; z0 += 8) {   // eight loads in flight, added in the order of the workgroups
-        float t[8];
+      for (int z0 = 0; z0 < n_blocks; z0 += 16) {   // sixteen loads in flight, added in the order of the workgroups
+        float t[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) t[u] = src[(int64_t)min(z0 + u, n_blocks - 1) * 16 * 128];
+        for (int u = 0; u < 16; ++u) t[u] = src[(int64_t)min(z0 + u, n_blocks - 1) * 16 * 128];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < 16; ++u)
           if (z0 + u < n_blocks) sum += t[u];
       }
       float pmid = s_sc[16 + c16_0 + o_cl];
