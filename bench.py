@@ -366,7 +366,11 @@ def e2e_bench(name, device, steps=None, warmup=3):
                        "max_position_embeddings": MODEL_MAX_POSITIONS},
             "kv_cache_bytes": {"full_bf16": full, "fourier_in_use": used, "fourier_allocated": held,
                                "reduction_in_use": round(full / used, 3)},
-            "synthetic_prefill_s": round(fill_s, 2)}
+            "synthetic_prefill_s": round(fill_s, 2),
+            # the decode projections run on a second copy of the layer weights in matrix-core order
+            # (LlamaModel.pack_projections): what that copy costs in memory
+            "packed_projection_weights_bytes": sum(w.data.numel() * w.data.element_size()
+                                                   for layer in model.model.layers for w in layer._packed.values())}
 
 
 def prefill_e2e_bench(device, preset="llama-3.1-8b", prompt=32768, reps=2):
