@@ -635,7 +635,8 @@ def main():
                     "tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "steps": r["steps"], "warmup": r["warmup"],
                     "batch": r["config"]["batch"], "prompt": r["config"]["prompt"], "model": r["config"]["model"],
                     "T_x": r["config"]["T_x"], "T_c": r["config"]["T_c"], "max_position_embeddings": MODEL_MAX_POSITIONS,
-                    "kv_cache_bytes": r["kv_cache_bytes"], "synthetic_prefill_s": r["synthetic_prefill_s"]}
+                    "kv_cache_bytes": r["kv_cache_bytes"], "synthetic_prefill_s": r["synthetic_prefill_s"],
+                    "packed_projection_weights_bytes": r["packed_projection_weights_bytes"]}
             except Exception as exc:   # the headline figure above stands on its own; say what happened here
                 result["e2e"][name.split("_")[0]] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_cpu_baseline:
