@@ -431,7 +431,7 @@ def main():
                          "merge inside the mid-row launch (for comparison)")
     ap.add_argument("--update-inside-attention", action="store_true",
                     help="update_plus_attn: the streaming update leaves the rank-1 coefficient update to the attention that "
-                         "follows, which applies it while it streams the coefficients (comparison; no faster, see DESIGN.md)")
+                         "follows, which applies it while it streams the coefficients (comparison: measured no faster than the update launch)")
     ap.add_argument("--no-sub-splits", action="store_true",
                     help="a batch of one sequence: one page stream per workgroup instead of four sub-splits (comparison)")
     ap.add_argument("--e2e", choices=list(E2E), default=None,
