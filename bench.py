@@ -328,6 +328,7 @@ def e2e_bench(name, device, steps=None, warmup=3):
         model.model.pack_projections()
     cache = DynamicCache(ec, device=device)
     cache.defer_coef_update = os.environ.get("FA_BENCH_UPDATE_INSIDE_ATTENTION", "0") == "1"   # (comparison)
+    cache.fuse_decode = os.environ.get("FA_BENCH_NO_FUSE", "0") != "1"                         # (comparison)
     t0 = time.perf_counter()
     synthetic_prefill(cache, cfg, e["B"], e["prompt"], torch.bfloat16, device, seed=0)
     torch.cuda.synchronize()

@@ -1790,7 +1790,7 @@ Plan make_plan(int B, int Hq, int Hkv, int D, int N, int n_il, int L_m, bool mfm
     p.heads_per_bin = 0;
     {
       const int teams = Hkv * p.n_groups;
-      if (fill_dies && fa_mfma::table_slices(N) == 4 && D == fa_mfma::kFusedD && G <= fa_mfma::kFusedG && teams % fa_mfma::kFusedXcds == 0 &&
+      if (fill_dies && D == fa_mfma::kFusedD && G <= fa_mfma::kFusedG && teams % fa_mfma::kFusedXcds == 0 &&
           teams / fa_mfma::kFusedXcds < Hkv && Hkv % (teams / fa_mfma::kFusedXcds) == 0)
         p.heads_per_bin = teams / fa_mfma::kFusedXcds;
     }
@@ -1869,15 +1869,19 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
 }
 
 // eight frequency slices: a score pass, then a value pass over the same pages
+// (fused: the value pass merges its own partials; its workgroups are then numbered through wg_map, those of the score
+// pass, which hands over whole pages of scores, keep the plain numbering)
 template <typename E>
-void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, hipStream_t st) {
-  dim3 grid(p.n_wg, p.n_groups);
+void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, hipStream_t st) {
+  dim3 grid(p.n_wg, p.n_groups), flat(p.n_wg * p.n_groups);
   if (wide) {
     fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2><<<grid, 512, 0, st>>>(mp);
+    if (fused) fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2, true><<<flat, 512, 0, st>>>(mp);
+    else fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2><<<grid, 512, 0, st>>>(mp);
   } else {
     fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 1><<<grid, 512, 0, st>>>(mp);
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2><<<grid, 512, 0, st>>>(mp);
+    if (fused) fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2, true><<<flat, 512, 0, st>>>(mp);
+    else fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2><<<grid, 512, 0, st>>>(mp);
   }
 }
 
@@ -1945,7 +1949,7 @@ thread_local int g_last_call_fused = 0;   // what the last fa_decode_attn call o
 bool fused_merge_plan(const fa_decode_args& a, const Plan& p, uint16_t* wg_map, hipStream_t st) {
   using namespace fa_mfma;
   if (p.path != Path::Mfma || (a.no_fuse & 1) || p.n_mid_split <= 0) return false;
-  if (table_slices(a.N) != 4 || a.D != kFusedD || a.Hq / a.Hkv > kFusedG) return false;
+  if (a.D != kFusedD || a.Hq / a.Hkv > kFusedG) return false;
   if (a.dtype != FA_BF16 && a.dtype != FA_FP16) return false;
   const int total = p.n_wg * p.n_groups, n_teams = p.n_groups * a.Hkv;
   if (total > device_cu_count() || total > kFusedMaxWgs || total % kFusedXcds != 0 || n_teams > (1 << (16 - kFusedSplitBits)))
@@ -2029,7 +2033,8 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
   // (the sink/window tiles must be in front of the mid rows for the merge to run inside that launch)
   const bool fused = sizeof(E) == 2 && (fuse_il || p.n_il_split == 0) && fused_merge_plan(a, p, wg_map, st);
   // one sequence: its mid rows as four sub-splits per workgroup in the places of four batch elements
-  const bool sub = fused && a.B == 1 && !(a.no_fuse & 2);
+  const bool one_pass = p.path == Path::Mfma && fa_mfma::table_slices(a.N) == 4;
+  const bool sub = fused && one_pass && a.B == 1 && !(a.no_fuse & 2);
   g_last_call_fused = fused ? (sub ? 2 : 1) : 0;
   // A rank-1 update the coefficients are still owed: the query preparation applies it to the K coefficients it streams,
   // the merge inside the mid-row launch to the V coefficients; where those do not run it gets a launch of its own
@@ -2039,7 +2044,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
     if (rc != FA_OK) return rc;
   }
   // (the tail of the mid-row launch reduces its phases in 32 bits)
-  const bool upd_v_in_tail = fused && a.upd_v_row && (uint64_t)a.N * (uint64_t)a.upd_T < (1ull << 32);
+  const bool upd_v_in_tail = fused && one_pass && a.upd_v_row && (uint64_t)a.N * (uint64_t)a.upd_T < (1ull << 32);
   if (a.upd_v_row && a.Cv > 0 && !upd_v_in_tail) {
     const int rc = fa_coeff_update(const_cast<float*>(a.v_mc), a.upd_v_row, a.dtype, a.upd_batch_stride, a.vc_list, a.B, a.N,
                                    a.Cv, a.upd_phase, a.upd_T, (fa_stream_t)st);
@@ -2112,7 +2117,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.sm_log2e = sm_log2e;
         if (ev) hipEventRecord(ev[1], st);
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
-        if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, st);
+        if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, fused, st);
         else switch (KS) {
           case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, fused, sub, st); break;
           case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, fused, sub, st); break;

@@ -152,7 +152,7 @@ __device__ __forceinline__ float4v fused_sum_lane_classes(float4v v, int nqp) {
 }
 
 // What a workgroup of a team does behind the first meeting.  Two shares, each an even cut of the team's work:
-//   rows     its tiles [t0, t1) of the 8 KS tiles of 8 frequencies (8 cosine + 8 sine coefficient rows each): g of
+//   rows     its tiles [t0, t1) of the N / 8 tiles of 8 frequencies (8 cosine + 8 sine coefficient rows each): g of
 //            those rows summed over the team's splits, times those rows of the V coefficients of every batch element
 //            of the group -> one partial output per column (every byte of g and of the V coefficients is read by
 //            exactly one workgroup);
@@ -183,7 +183,7 @@ template <bool SUB, typename P>
 __device__ __forceinline__ FusedShare fused_share(const P& p, int vc0, int vc_len, int split, int n_s, int b0, int nb, int KS,
                                                   int tid) {
   FusedShare f;
-  const int NT = 8 * KS;
+  const int NT = p.N / 8;   // tiles of 8 frequencies (2 KS per frequency slice)
   const int tper = (NT + n_s - 1) / n_s;
   f.t0 = min(NT, split * tper);
   f.t1 = min(NT, f.t0 + tper);
@@ -620,7 +620,7 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
   // ---- column share: the output element -------------------------------------------------------------------------------
   if (o_cl < ncol) {
     if (o_src < 128) {
-      const int NT = 8 * KS, tper = (NT + n_s - 1) / n_s;
+      const int NT = N / 8, tper = (NT + n_s - 1) / n_s;
       const int n_blocks = (NT + tper - 1) / tper;   // workgroups of the team that own coefficient rows
       const float* src = pc_team + (c16_0 + o_cl) * 128 + o_src;
       float sum = 0.f;

@@ -272,7 +272,7 @@ struct MidParams {
 //         memory (2 KiB per page and workgroup, against 16 KiB of K/V);
 // MODE 2, values: every wave reads the page's scores back, runs the softmax and keeps its slice of the g
 //         history; waves 0-3 stream V.  No exchange between the waves at all.
-// FUSE (MODE 0 only): the launch merges its own partials and writes the output rows, see fa_decode_fused.h; the
+// FUSE (MODE 0 and the value pass, MODE 2): the launch merges its own partials and writes the output rows, see fa_decode_fused.h; the
 // workgroups are then numbered through p.fz.wg_map so that the splits of a (batch group, KV head) share one die.
 // SUB (FUSE only, a batch of one sequence, at most four query heads per KV head): a single batch element would
 // leave twelve of the sixteen matrix-core columns and three of the four page streams of a workgroup idle.  The
@@ -286,7 +286,9 @@ struct MidParams {
 template <typename E, int KS, int KMAX, int VMAX, int NST, int MODE = 0, bool FUSE = false, bool SUB = false, bool UPD = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_mid_mfma_kernel(
     const MidParams<E> p) {
-  static_assert(!FUSE || MODE == 0, "the fused merge runs behind the one-pass pipeline");
+  static_assert(!FUSE || MODE == 0 || MODE == 2, "the fused merge runs behind the one-pass pipeline or behind the value pass");
+  static_assert(!SUB || MODE == 0, "sub-splits belong to the one-pass pipeline");
+  static_assert(!UPD || MODE == 0, "the pending update keeps its row in the LDS of the score partials");
   static_assert(!SUB || FUSE, "sub-splits end in the fused merge");
   static_assert(!UPD || FUSE, "the pending update rides in the fused merge");
   constexpr int NSL = MODE == 0 ? kFreqWaves : 2 * kFreqWaves;   // frequency slices

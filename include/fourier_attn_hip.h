@@ -319,11 +319,12 @@ int fa_decode_tables_build(void* tables, size_t tables_bytes, int N, int T, fa_s
 
 /* One decode step of Fourier attention over
  * [sink ; local window ; mid rows (stored dims + dims rebuilt from coefficients)].
- * Launches: query preparation + sink/window tiles, mid rows, merge.  On the one-pass matrix-core path (16-bit
- * storage, head_dim 128, at most four query heads per KV head, up to 512 frequencies) the workgroups of the mid-row
- * launch merge their own partials and write the output rows (two launches); args->no_fuse bit 0 keeps the three.
- * With a batch of one sequence every workgroup of that launch then runs four sub-splits of its pages side by side
- * (in the matrix-core columns and page streams that further batch elements would use).
+ * Launches: query preparation + sink/window tiles, mid rows (two passes with 1024 frequencies), merge.  On the
+ * matrix-core path with 16-bit storage, head_dim 128 and at most four query heads per KV head the workgroups of the
+ * last mid-row launch merge their own partials and write the output rows (one launch fewer); args->no_fuse bit 0
+ * keeps the merge launch.  With a batch of one sequence and up to 512 frequencies every workgroup of that launch then
+ * runs four sub-splits of its pages side by side (in the matrix-core columns and page streams that further batch
+ * elements would use).
  * That needs the device to deal the workgroups of a launch out to its dies in turn, which the first call on a device
  * checks with a tiny launch and ONE synchronisation of `stream` (skipped, and asked again by the next call, while
  * the stream is being captured). */

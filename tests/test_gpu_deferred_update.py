@@ -20,6 +20,7 @@ CASES = [
     (torch.float16, 8, 16, 8, 128, 4, 40, 512, 1500, [64, 0, 128, 30, 64, 64, 100, 64], [1, 64, 2, 3, 128, 64, 0, 64]),
     (torch.bfloat16, 3, 8, 2, 128, 4, 32, 256, 700, [64, 40], [64, 96]),         # matrix cores, merge as a launch of its own
     (torch.bfloat16, 2, 16, 4, 128, 4, 32, 2048, 4500, [64] * 4, [30, 64, 0, 100]),   # 1024 frequencies, two passes
+    (torch.bfloat16, 4, 24, 8, 128, 4, 40, 2048, 6000, U, U),                    # ... whose value pass merges (V: own launch)
     (torch.float32, 2, 8, 2, 64, 4, 16, 256, 420, [10, 30], [3, 64]),            # fp32 storage: the any-shape kernels
 ]
 

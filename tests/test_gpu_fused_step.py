@@ -5,8 +5,8 @@ elements.  Every case is also held against the CPU restatement (bound 2e-2 for 1
 
 Geometries: eight KV heads so that the teams of a launch fill the eight dies (what the fused merge needs), one to
 four query heads per KV head, batches that fill a group of four, leave it ragged or consist of one sequence, heads
-that compress everything, nothing, or one to three dims, mid rows from a single page to a few hundred, 128 to 512
-frequencies."""
+that compress everything, nothing, or one to three dims, mid rows from a single page to a few hundred, 128 to 1024
+frequencies (the last as two passes over the pages, the second of which then merges)."""
 import numpy as np
 import pytest
 import torch
@@ -31,6 +31,10 @@ CASES = [
     (torch.bfloat16, 4, 32, 4, 64, 1024, 3000, U, U, 1),                                   # a full group of four
     (torch.bfloat16, 8, 32, 4, 64, 512, 1500, [64, 0, 128, 30, 64, 64, 100, 64], [1, 64, 2, 3, 128, 64, 0, 64], 1),
     (torch.float16, 2, 16, 4, 40, 512, 2500, U, U, 1),                                     # two sequences: no sub-splits
+    # 1024 frequencies: the value pass of the two merges its own partials
+    (torch.bfloat16, 4, 24, 4, 40, 2048, 6000, U, U, 1),
+    (torch.float16, 2, 32, 4, 64, 2048, 5000, [64, 0, 128, 30, 64, 64, 100, 64], [1, 64, 2, 3, 128, 64, 0, 64], 1),
+    (torch.bfloat16, 1, 32, 4, 64, 2048, 7000, U, U, 1),                                   # one sequence there: no sub-splits either
 ]
 
 
