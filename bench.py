@@ -592,6 +592,32 @@ def main():
                      "algorithmic_bytes_per_launch": kbytes[dom], "kernel_ms": round(float(kernel_ms[dom]), 5),
                      "whole_step_frac": round(gbs / HBM_PEAK_GBS, 4)},
     }
+    if merge_in_mid_rows:
+        # The dominant launch now ends with the merge and the output rows, so its time is not comparable with the
+        # mid-row kernel of a step whose merge is a launch of its own: the same step that way, timed beside it
+        cache.fuse_decode = False
+        for _ in range(5):
+            cache.decode_attention(q, 0, Hq, Hkv)
+        start.record()
+        for _ in range(reps):
+            cache.decode_attention(q, 0, Hq, Hkv)
+        stop.record()
+        torch.cuda.synchronize()
+        ms_sep = start.elapsed_time(stop) / reps
+        per_sep = np.zeros(4)
+        for _ in range(reps):
+            tm = []
+            cache.decode_attention(q, 0, Hq, Hkv, timings=tm)
+            per_sep += np.array(tm)
+        per_sep /= reps
+        cache.fuse_decode = not args.no_fuse
+        sep_gbs = kbytes["mid_rows"] / (per_sep[1] * 1e-3) / 1e9
+        result["roofline"]["merge_as_a_launch_of_its_own"] = {
+            "ms_per_step": round(ms_sep, 5), "whole_step_frac": round(nbytes / (ms_sep * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "kernel_ms": {"query_and_sink_window": round(float(per_sep[0] + per_sep[2]), 5), "mid_rows": round(float(per_sep[1]), 5),
+                          "merge": round(float(per_sep[3]), 5)},
+            "mid_rows_achieved": round(sep_gbs, 2), "mid_rows_frac": round(sep_gbs / HBM_PEAK_GBS, 4),
+            "mid_rows_algorithmic_bytes_per_launch": kbytes["mid_rows"]}
     # the streaming update that precedes every decode-attention pass in use (one launch: rank-1 coefficient
     # update, evicted row into the page store, new token into the window); read + write of the coefficients
     # (fewer streamed tokens in all than the workload's max_new_tokens: the page store is sized for those and would
