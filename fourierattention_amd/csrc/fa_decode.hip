@@ -2100,7 +2100,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         if (fused) {
           auto& fz = mp.fz;
           fz.il_m = ilm; fz.il_d = ild; fz.il_o = ilo; fz.n_il = p.n_il_split;
-          fz.part_c = (float*)(ws + p.off_pc); fz.stage_il = (float*)(ws + p.off_sil); fz.stage_on = (float*)(ws + p.off_son);
+          fz.part_c = (float*)(ws + p.off_pc);
           fz.cnt = (unsigned*)(ws + p.off_cnt) + (size_t)a.B * a.Hkv;
           fz.v_mc = a.v_mc; fz.avg_u = a.avg_v_u; fz.avg_d = a.avg_v_d; fz.scale = a.scale_v;
           fz.vc_list = a.vc_list; fz.vc_h = a.vc_h_list; fz.vn_list = a.vn_list;

@@ -11,8 +11,9 @@
 //   merge share   split weights; the workgroup's share of the coefficient rows: g summed over the team's splits
 //                 times those rows of the V coefficients (requested before the meeting) -> a partial output per
 //                 column; its share of the dims of the sink/window and stored-dim partial outputs
-//   meeting 2     the workgroup that counts itself in last adds the shares up in a fixed order, applies the column
-//                 statistics, normalises and writes the output rows
+//   meeting 2     every workgroup of the team has stored its partial output
+//   column share  for its share of the team's columns the workgroup adds those partial outputs up in a fixed order,
+//                 applies the column statistics, normalises and writes the output rows
 //
 // The workgroups of a team all run on ONE accelerator die (XCD): the hardware deals the workgroups of a launch out to
 // the eight dies in turn (linear workgroup index modulo 8), and the host numbers the workgroups so that a team's
@@ -21,7 +22,7 @@
 // in the L2; plain loads behind the meeting (nothing of these buffers can be in the reader's L1: it is empty when
 // the launch starts and the reader touches them here for the first time).  A round trip through memory with
 // device scope (`sc1`) takes about 3 us on a loaded device against well under 1 us through the L2, and the tail is
-// a chain of eight such trips.  Every workgroup adds the number of its die to the upper half of the meeting
+// a chain of eight such trips.  (With 1024 frequencies the same tail runs behind the value pass of the two passes.)  Every workgroup adds the number of its die to the upper half of the meeting
 // counter and checks the sum: a team that does not sit on one die (or a workgroup that never arrives) ends the
 // wait without a result and leaves NaN rows, never plausible numbers.
 #pragma once
@@ -75,8 +76,6 @@ struct FusedParams {
   const float* il_o;  // [B * Hq][n_il][D]
   int n_il;
   float* part_c;      // [groups][Hkv][n_split][16 column slots][128]  g . V_coef of a workgroup's coefficient rows
-  float* stage_il;    // [B * Hq][D]  sink/window outputs summed over the tiles
-  float* stage_on;    // [B * Hq][D]  stored-dim outputs summed over the team (by position in the head's list)
   unsigned* cnt;      // [groups][Hkv][2]  the two meetings; zero when the launch starts
   const float* v_mc;
   const float* avg_u;
@@ -129,28 +128,6 @@ __device__ __forceinline__ bool team_wait(unsigned* counter, unsigned n, unsigne
 }
 
 // ---- the merge share (see the head of this file) -----------------------------------------------------------------
-// sum over the lanes q, q + nqp, q + 2 nqp, ... of a wave (nqp a power of two up to 32, uniform over the wave); every
-// lane gets the sum of its class
-template <int CTRL>
-__device__ __forceinline__ float4v fused_dpp4_add(float4v v) {
-  v[0] += fa_dpp<CTRL>(v[0]); v[1] += fa_dpp<CTRL>(v[1]); v[2] += fa_dpp<CTRL>(v[2]); v[3] += fa_dpp<CTRL>(v[3]);
-  return v;
-}
-__device__ __forceinline__ float4v fused_sum_lane_classes(float4v v, int nqp) {
-  if (nqp <= 1) v = fused_dpp4_add<0x121>(v);   // row_ror:1
-  if (nqp <= 2) v = fused_dpp4_add<0x122>(v);   // row_ror:2
-  if (nqp <= 4) v = fused_dpp4_add<0x124>(v);   // row_ror:4
-  if (nqp <= 8) v = fused_dpp4_add<0x128>(v);   // row_ror:8
-  float lo, hi;
-  if (nqp <= 16) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) { fa_swap16(v[e], &lo, &hi); v[e] = lo + hi; }
-  }
-#pragma unroll
-  for (int e = 0; e < 4; ++e) { fa_swap32(v[e], &lo, &hi); v[e] = lo + hi; }
-  return v;
-}
-
 // What a workgroup of a team does behind the first meeting.  Two shares, each an even cut of the team's work:
 //   rows     its tiles [t0, t1) of the N / 8 tiles of 8 frequencies (8 cosine + 8 sine coefficient rows each): g of
 //            those rows summed over the team's splits, times those rows of the V coefficients of every batch element
