@@ -1916,6 +1916,10 @@ static __device__ unsigned xcc_probe_out[fa_mfma::kFusedMaxWgs];
 __global__ __launch_bounds__(512) void xcc_probe_kernel(unsigned* out) {
   if (threadIdx.x == 0) out[blockIdx.x] = fa_mfma::xcc_id();
 }
+// (set around the call by the entry point that must not allocate: the probe copies its result to pageable host memory,
+// for which the runtime may set up a staging buffer; that entry point keeps the merge launch until another call has
+// probed the device)
+thread_local bool g_no_layout_probe = false;
 bool fused_layout_ok(hipStream_t st) {
   constexpr int kMaxDevices = 64;
   static std::mutex mu;
@@ -1924,6 +1928,7 @@ bool fused_layout_ok(hipStream_t st) {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
   std::lock_guard<std::mutex> lock(mu);
   if (known[dev] != 0) return known[dev] > 0;
+  if (g_no_layout_probe) return false;
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return false;   // (ask again later)
   void* out = nullptr;
@@ -2387,7 +2392,10 @@ extern "C" int fa_decode_attn_noalloc(const fa_decode_args* a, fa_stream_t strea
   b.k_pad_h_host = b.v_pad_h_host = nullptr;
   b.workspace = ptr;
   b.workspace_bytes = (size_t)FA_DECODE_NOALLOC_SCRATCH_BYTES;
-  return decode_attn_impl(&b, stream, nullptr);
+  g_no_layout_probe = true;
+  rc = decode_attn_impl(&b, stream, nullptr);
+  g_no_layout_probe = false;
+  return rc;
 }
 
 extern "C" int fa_decode_attn_last_fused(void) { return g_last_call_fused; }

@@ -349,7 +349,10 @@ int fa_decode_split_plan(int B, int Hq, int Hkv, int D, int N, int il_rows_total
  * FA_ERR_WORKSPACE.  Every call on one GPU shares that GPU's buffer: calls that may
  * overlap on one GPU (two streams, two threads) race and must be serialised by the caller; consecutive calls on
  * one stream are fine (every kernel writes what it later reads, nothing needs clearing).  The first call on a
- * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture. */
+ * device looks the buffer's address up (hipGetSymbolAddress): make it outside any stream capture.  This entry
+ * point never runs fa_decode_attn's one-off check of the device's workgroup placement (its copy to the host could
+ * make the runtime set up a staging buffer): until a fa_decode_attn call has run that check on the device, the merge
+ * stays a launch of its own here. */
 #define FA_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
 int fa_decode_attn_noalloc(const fa_decode_args* args, fa_stream_t stream);
 

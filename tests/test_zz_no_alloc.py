@@ -93,6 +93,29 @@ def test_two_calls_in_a_row_match_the_entry_point_with_a_workspace(dtype, tol):
 
 
 @pytest.mark.gpu
+def test_calls_whose_mid_row_launch_merges_its_own_partials():
+    """Eight KV heads: the teams of the mid-row launch fill the dies, so the merge runs inside that launch and its
+    meeting counters live in the buffer too (cleared by the launch in front, every call).  A batch of four, then a
+    single sequence (four sub-splits per workgroup), then the batch again: bit for bit as with a workspace.  (This
+    entry point does not probe the device's workgroup placement itself, see the header: the calls with a workspace
+    in front of it have.)"""
+    from fourierattention_amd import _lib
+    Hq, Hkv, D = 32, 8, 128
+    big = _cache_case(torch.bfloat16, 4, Hq, Hkv, D, 64, 1024, 3000, [64] * 8, [64, 0, 128, 30, 64, 64, 100, 64], seed=5)
+    one = _cache_case(torch.bfloat16, 1, Hq, Hkv, D, 32, 512, 1500, [64] * 8, [64] * 8, seed=6)
+    for (gpu, q, want), mode in ((big, 1), (one, 2), (big, 1)):
+        gpu.balance_heads = False
+        ref = gpu.decode_attention(q, 0, Hq, Hkv)
+        assert _lib.load().fa_decode_attn_last_fused() == mode
+        out = torch.full_like(ref, float("nan"))
+        got = gpu.decode_attention(q, 0, Hq, Hkv, out=out, no_alloc=True)
+        assert _lib.load().fa_decode_attn_last_fused() == mode
+        assert got is out and torch.equal(got, ref)
+        err = np.abs(got.cpu().numpy() - want).max()
+        assert err <= 2e-3, err
+
+
+@pytest.mark.gpu
 def test_two_calls_with_1024_frequencies():
     """1024 frequencies take the two-pass mid rows and the merge whose blocks hand over through counters in the
     buffer (cleared by the launch in front): two calls in a row, the second smaller, bit for bit as with a workspace."""
