@@ -98,3 +98,52 @@ def test_fused_step_with_converted_output_rows():
         f32 = gpu.decode_attention(q, 0, Hq, Hkv)
         cast = gpu.decode_attention(q, 0, Hq, Hkv, out_dtype=q.dtype)
         assert cast.dtype == q.dtype and torch.equal(cast, f32.to(q.dtype))
+
+
+def test_random_geometries_with_the_merge_inside_the_launch_agree_with_the_generic_kernels():
+    """Seeded random geometry on eight or sixteen KV heads (whole teams per die, so the merge runs inside the mid-row
+    launch wherever the shape allows it): batches of 1 to 9 (groups of four, a last group that is not full, a single
+    sequence with its sub-splits), one to four query heads per KV head, 128 to 1024 frequencies, ragged per-head
+    masks, odd sink / window / prompt lengths, with and without a pending coefficient update; against the plain
+    kernels on the same cache.  At least half of the cases must have taken the launch that merges."""
+    from fourierattention_amd import DynamicCache, _lib
+    rng = np.random.default_rng(4711)
+    lib = _lib.load()
+    merged = 0
+    n_cases = 14
+    for case in range(n_cases):
+        dtype = [torch.bfloat16, torch.float16][rng.integers(2)]
+        D = 128
+        Hkv = int([8, 8, 8, 16][rng.integers(4)]); G = int(rng.integers(1, 5)); Hq = Hkv * G
+        B = int([1, 1, 2, 3, 4, 5, 8, 9][rng.integers(8)]); I = int(rng.integers(0, 6)); W = int(rng.integers(1, 130))
+        M = int([256, 512, 1024, 1024, 2048][rng.integers(5)])
+        prompt = int(I + W + M + rng.integers(1, 4000))
+        kc = [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)]
+        vc = [int(rng.integers(1 if h == 0 else 0, D + 1)) for h in range(Hkv)]
+        defer = bool(rng.integers(2))
+        tag = (f"case {case}: {dtype} B={B} Hq={Hq} Hkv={Hkv} I={I} W={W} M={M} prompt={prompt} defer={defer} "
+               f"k={kc} v={vc}")
+        print(tag, flush=True)
+        masks = _masks(1, Hkv, D, kc, vc, seed=case)
+        cfg = _cfg(masks, numinittokens=I, maxlocallen=W, maxmidstates=M, num_key_value_heads=Hkv, max_new_tokens=8,
+                   max_position_embeddings=1 << 20)
+        gpu = DynamicCache(cfg)
+        gpu.defer_coef_update = defer
+        g = torch.Generator(device="cuda").manual_seed(case)
+        rn = lambda *sh: torch.randn(*sh, generator=g, device="cuda")
+        gpu.update(rn(B, Hkv, prompt, D).to(dtype), rn(B, Hkv, prompt, D).to(dtype), 0)
+        assert gpu._tables is not None, tag
+        for _ in range(2):
+            gpu.update(rn(B, Hkv, 1, D).to(dtype), rn(B, Hkv, 1, D).to(dtype), 0)
+            q = (rn(B, Hq, 1, D) * 1.5).to(dtype)
+            got = gpu.decode_attention(q, 0, Hq, Hkv)
+            ran = lib.fa_decode_attn_last_fused()
+            gpu.force_generic = True
+            ref = gpu.decode_attention(q, 0, Hq, Hkv)
+            gpu.force_generic = False
+            assert torch.isfinite(got).all(), tag
+            err = (got - ref).abs().max().item()
+            assert err <= 5e-3, (tag, err, ran)
+        merged += ran > 0
+        assert ran != 2 or B == 1, tag
+    assert merged >= n_cases // 2, merged
