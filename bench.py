@@ -216,7 +216,7 @@ def cpu_baseline():
                                   f"warm-ups = {med1 * 1e3:.2f} ms (min {t1[0] * 1e3:.2f} ms), {bytes1} algorithmic bytes"}}
 
 
-KERNEL_SOURCES = ("fa_decode.hip", "fa_decode_mfma.h", "fa_decode_fused.h", "fa_mfma_util.h", "fa_common.h")
+KERNEL_SOURCES = ("fa_decode.hip", "fa_decode_mfma.h", "fa_decode_fused.h", "fa_decode_mid_launch.h", "fa_mfma_util.h", "fa_common.h")
 
 
 def kernel_source_digest():

@@ -157,8 +157,8 @@ def kernels_with_atomics_outside(asm_text: str, kernels=HANDOVER_KERNELS):
     return out
 
 
-ASYNC_LDS_SOURCES = ("fa_decode", "fa_prefill", "fa_spectral_mfma")
-HANDOVER_SOURCES = ("fa_decode",)
+ASYNC_LDS_SOURCES = ("fa_decode_mid_bf16", "fa_decode_mid_f16", "fa_prefill", "fa_spectral_mfma")
+HANDOVER_SOURCES = ("fa_decode", "fa_decode_mid_bf16", "fa_decode_mid_f16")
 
 
 def count_async_lds_reads(asm_text: str) -> int:

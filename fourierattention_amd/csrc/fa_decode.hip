@@ -13,7 +13,7 @@
 
 #include "fa_common.h"
 #include <mutex>
-#include "fa_decode_mfma.h"
+#include "fa_decode_mid_launch.h"
 
 namespace {
 
@@ -1868,47 +1868,6 @@ void launch_tables(void* tables, int N, int T, hipStream_t st) {
   decode_tables_kernel<<<fa_cdiv(total, 256), 256, 0, st>>>(tabE, tabET, rot, KS, T, N, NSL);
 }
 
-// eight frequency slices: a score pass, then a value pass over the same pages
-// (fused: the value pass merges its own partials; its workgroups are then numbered through wg_map, those of the score
-// pass, which hands over whole pages of scores, keep the plain numbering)
-template <typename E>
-void launch_mid_mfma_two_pass(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, hipStream_t st) {
-  dim3 grid(p.n_wg, p.n_groups), flat(p.n_wg * p.n_groups);
-  if (wide) {
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
-    if (fused) fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2, true><<<flat, 512, 0, st>>>(mp);
-    else fa_mfma::decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2><<<grid, 512, 0, st>>>(mp);
-  } else {
-    fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 2, 1><<<grid, 512, 0, st>>>(mp);
-    if (fused) fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2, true><<<flat, 512, 0, st>>>(mp);
-    else fa_mfma::decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2><<<grid, 512, 0, st>>>(mp);
-  }
-}
-
-template <typename E, int KS>
-void launch_mid_mfma_ks(const fa_mfma::MidParams<E>& mp, const Plan& p, bool wide, bool fused, bool sub, hipStream_t st) {
-  dim3 grid(p.n_wg, p.n_groups);
-  if (fused) {
-    grid = dim3(p.n_wg * p.n_groups);   // numbered through wg_map
-    const bool upd = mp.fz.upd_row != nullptr;   // (instances of their own, like the query preparation's)
-    auto go = [&](auto sub_tag, auto upd_tag) {
-      constexpr bool S = decltype(sub_tag)::value, U = decltype(upd_tag)::value;
-      if (wide)
-        fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2, 0, true, S, U><<<grid, 512, 0, st>>>(mp);
-      else
-        fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2, 0, true, S, U><<<grid, 512, 0, st>>>(mp);
-    };
-    if (sub && upd) go(std::true_type{}, std::true_type{});
-    else if (sub) go(std::true_type{}, std::false_type{});
-    else if (upd) go(std::false_type{}, std::true_type{});
-    else go(std::false_type{}, std::false_type{});
-  } else if (wide) {
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 4, 8, 2><<<grid, 512, 0, st>>>(mp);
-  } else {
-    fa_mfma::decode_mid_mfma_kernel<E, KS, 2, 4, 2><<<grid, 512, 0, st>>>(mp);
-  }
-}
-
 // The fused merge relies on the workgroups of a launch being dealt out to the dies in turn (workgroup L on die
 // L % 8).  Checked once per device by a launch of the same shape that records the die of every workgroup; a device
 // (or partition mode) that deals them out differently keeps the merge in a launch of its own.
@@ -2122,12 +2081,7 @@ int launch_all(const fa_decode_args& a, const Plan& p, bool p_il_fast, float sm_
         mp.sm_log2e = sm_log2e;
         if (ev) hipEventRecord(ev[1], st);
         const bool wide = a.mid_max_k_pad > 64 || a.mid_max_v_pad > 64;
-        if (NSL > 4) launch_mid_mfma_two_pass<E>(mp, p, wide, fused, st);
-        else switch (KS) {
-          case 2: launch_mid_mfma_ks<E, 2>(mp, p, wide, fused, sub, st); break;
-          case 4: launch_mid_mfma_ks<E, 4>(mp, p, wide, fused, sub, st); break;
-          default: launch_mid_mfma_ks<E, 8>(mp, p, wide, fused, sub, st); break;
-        }
+        launch_mid_rows<E>(mp, MidLaunch{p.n_wg, p.n_groups, KS, wide, NSL > 4, fused, sub}, st);
       }
     } else {
       size_t lds = ((size_t)G * 2 * a.N + 2 * (size_t)G * a.D + (size_t)G * kTile + 4 * kGMax) * sizeof(float);

@@ -57,7 +57,7 @@ constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one 
 //   rot   [N] float2 : (cos, sin)(2 pi f 64 / T), the rotation from one frame to the next
 // Half-token offsets: phase f (2i + 1) / (2T), reduced exactly in integers.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ tabE, half8* __restrict__ tabET,
+static __global__ __launch_bounds__(256) void decode_tables_kernel(half8* __restrict__ tabE, half8* __restrict__ tabET,
                                                             float2v* __restrict__ rot, int KS, int T, int N, int NSL) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   const int nE = NSL * 2 * KS * 64, nET = NSL * 2 * KS * 64;

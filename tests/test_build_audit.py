@@ -108,8 +108,8 @@ def test_audit_fails_closed():
     assert any("no counting atomic" in m for m in audit_listings("fa_decode", [GOOD]))
     assert any("no gfx950 assembly" in m for m in audit_listings("fa_decode", []))
     plain = "_Zkernel_z:\n\tv_add_f32_e32 v1, v2, v3\n\ts_endpgm\n"
-    assert "fa_decode" in ASYNC_LDS_SOURCES and "fa_stream" not in ASYNC_LDS_SOURCES
-    assert any("no inline-asm LDS read" in m for m in audit_listings("fa_decode", [plain]))
+    assert "fa_decode_mid_bf16" in ASYNC_LDS_SOURCES and "fa_stream" not in ASYNC_LDS_SOURCES
+    assert any("no inline-asm LDS read" in m for m in audit_listings("fa_decode_mid_bf16", [plain]))
     assert audit_listings("fa_stream", [plain]) == []          # a source without such reads passes on a plain listing
     assert audit_listings("fa_stream", [BAD_COPY]) != []       # but a violation is reported wherever it shows up
 
