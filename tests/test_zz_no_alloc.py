@@ -137,9 +137,16 @@ def test_captured_in_a_graph_and_replayed():
     """``fa_decode_attn_noalloc`` recorded into a graph (no allocation, no clearing of memory by the runtime: the
     counters of the merge are cleared by the launch in front of it) and replayed on new queries in the same buffers:
     every replay bit for bit what the eager call returns."""
-    Hq, Hkv, D = 8, 2, 128
-    for M, prompt in ((512, 2000), (2048, 4300)):     # the fused mid rows / the two passes of 1024 frequencies
-        gpu, q, want = _cache_case(torch.bfloat16, 3, Hq, Hkv, D, 64, M, prompt, [64, 40], [64, 96], seed=5)
+    # the one-pass mid rows / the two passes of 1024 frequencies with the merge as a launch of its own (two KV heads);
+    # the merge inside the mid-row launch (eight KV heads: its meeting counters are cleared by the launch in front on
+    # every replay), for a batch and for a single sequence with its sub-splits.  (1024 frequencies on eight KV heads
+    # need more than the built-in buffer holds.)
+    shapes = [(3, 8, 2, 512, 2000, [64, 40], [64, 96], 0), (3, 8, 2, 2048, 4300, [64, 40], [64, 96], 0),
+              (4, 32, 8, 1024, 3000, [64] * 8, [64, 0, 128, 30, 64, 64, 100, 64], 1), (1, 32, 8, 512, 1500, [64] * 8, [64] * 8, 2)]
+    D = 128
+    from fourierattention_amd import _lib
+    for B, Hq, Hkv, M, prompt, kc, vc, mode in shapes:
+        gpu, q, want = _cache_case(torch.bfloat16, B, Hq, Hkv, D, 64, M, prompt, kc, vc, seed=5)
         gpu.balance_heads = False
         ref = gpu.decode_attention(q, 0, Hq, Hkv)
         out = torch.full_like(ref, float("nan"))
@@ -150,6 +157,7 @@ def test_captured_in_a_graph_and_replayed():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             gpu.decode_attention(qbuf, 0, Hq, Hkv, out=out, no_alloc=True)
+        assert _lib.load().fa_decode_attn_last_fused() == mode     # (what the recorded call runs)
         gen = torch.Generator(device="cuda").manual_seed(7)
         for _ in range(3):
             qk = (torch.randn(q.shape, generator=gen, device="cuda") * 1.5).to(q.dtype)
