@@ -337,6 +337,9 @@ E2E = {
     # BASELINE configs 4 and 5: a random-init decoder with the Fourier cache on every layer
     "config4_e2e_8b_64k": dict(preset="llama-3.1-8b", B=16, prompt=65536, new=128, I=4, W=1024, M=1024, cper=64),
     "config5_e2e_3b_128k": dict(preset="llama-3.2-3b", B=4, prompt=131072, new=512, I=4, W=1024, M=2048, cper=64),
+    # the reference's evaluation settings (one sequence, window 1020, 1024 states; about three quarters of the dims
+    # compressed, as in its mask for this model)
+    "refeval_e2e_8b_32k": dict(preset="llama-3.1-8b", B=1, prompt=32768, new=128, I=4, W=1020, M=1024, cper=96),
 }
 
 

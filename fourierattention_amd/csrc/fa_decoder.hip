@@ -275,7 +275,8 @@ extern "C" int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, vo
              "fa_rope_qk: rows=%d Hq=%d Hkv=%d D=%d", rows, Hq, Hkv, D);
   FA_REQUIRE(q_in_stride >= (int64_t)Hq * D && k_stride >= (int64_t)Hkv * D, FA_ERR_BAD_SHAPE,
              "fa_rope_qk: row strides %lld, %lld shorter than the rows", (long long)q_in_stride, (long long)k_stride);
-  FA_REQUIRE(q_out != q_in || q_in_stride == (int64_t)Hq * D, FA_ERR_BAD_SHAPE,
+  // (a single row is dense whatever stride its view reports: the q slice of one token's fused q/k/v projection)
+  FA_REQUIRE(q_out != q_in || rows <= 1 || q_in_stride == (int64_t)Hq * D, FA_ERR_BAD_SHAPE,
              "fa_rope_qk: in place needs densely packed q rows");
   if (rows == 0) return FA_OK;
   hipStream_t st = fa_hip_stream(stream);

@@ -253,6 +253,8 @@ def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tens
     q_out = q if q.is_contiguous() else torch.empty(q.shape, dtype=q.dtype, device=q.device)
     qs = q.stride(1) if q.shape[1] > 1 else q.stride(0)
     ks = k.stride(1) if k.shape[1] > 1 else k.stride(0)
+    if rows == 1:                      # a single row has no spacing, whatever its view reports
+        qs, ks = q.shape[2], k.shape[2]
     check(_lib.load().fa_rope_qk(q.data_ptr(), qs, q_out.data_ptr(), k.data_ptr(), ks, cos.data_ptr(), sin.data_ptr(), rows,
                                  q.shape[2] // head_dim, k.shape[2] // head_dim, head_dim, dtype_code(q.dtype),
                                  _stream(q.device)))

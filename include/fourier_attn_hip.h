@@ -402,7 +402,8 @@ int fa_add_rmsnorm(void* h, const void* delta, const void* weight, void* y, int 
  * `dtype` one by one like the tensor ops.  Row r of q is read at q_in + r * q_in_stride
  * (Hq * D elements; the rows may be slices of a wider fused projection output) and
  * written to q_out as (rows, Hq * D) densely packed; q_out may be q_in when q_in is
- * densely packed itself.  k: row r at k + r * k_stride, Hkv * D elements, in place.
+ * densely packed itself (a single row always is, whatever q_in_stride says).  k: row r
+ * at k + r * k_stride, Hkv * D elements, in place.
  * Strides in elements. */
 int fa_rope_qk(const void* q_in, int64_t q_in_stride, void* q_out, void* k, int64_t k_stride,
                const void* cos, const void* sin, int rows, int Hq, int Hkv, int D, int dtype,

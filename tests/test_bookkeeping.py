@@ -244,7 +244,7 @@ def test_argument_validation_returns_codes_without_a_gpu():
     assert lib.fa_rope_qk(p, 256, p, None, 128, p, p, 1, 4, 2, 64, 0, None) == -1
     assert lib.fa_rope_qk(p, 252, p, p, 126, p, p, 1, 4, 2, 63, 0, None) == -2    # odd head_dim
     assert lib.fa_rope_qk(p, 255, p, p, 128, p, p, 1, 4, 2, 64, 0, None) == -2    # stride shorter than a row
-    assert lib.fa_rope_qk(p, 512, p, p, 128, p, p, 1, 4, 2, 64, 0, None) == -2    # in place on sliced rows
+    assert lib.fa_rope_qk(p, 512, p, p, 128, p, p, 2, 4, 2, 64, 0, None) == -2    # in place on sliced rows (more than one)
     assert lib.fa_silu_mul(p, p, None, 1, 8, 8, 0, None) == -1
     assert lib.fa_silu_mul(p, p, p, -1, 8, 8, 0, None) == -2
     assert lib.fa_silu_mul(p, p, p, 2, 8, 4, 0, None) == -2                        # stride shorter than a row

@@ -224,8 +224,10 @@ def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
         assert torch.equal(h2, want_h) and torch.equal(y0, y)
     # rotary embedding: no reduction anywhere, so bit for bit (head dims of 64 and at least 64 rows: 16 bytes per
     # thread with 16-bit storage; otherwise the element-wise variant)
-    for D, q_len in ((64, 40), (64, 2), (40, 2)):   # 120 rows; a few rows (one block per head); odd head dim
-        B, Hq, Hkv = 3, 6, 2
+    # 120 rows; a few rows (one block per head); odd head dim; one row (one token of one sequence: the slice of a
+    # wider row is then "contiguous" and still reports the wider row's stride)
+    for D, q_len, B in ((64, 40, 3), (64, 2, 3), (40, 2, 3), (64, 1, 1)):
+        Hq, Hkv = 6, 2
         q, k = rn(B, q_len, Hq * D).to(dtype), rn(B, q_len, Hkv * D).to(dtype)
         ang = rn(B, q_len, D) * 3
         cos, sin = ang.cos().to(dtype), ang.sin().to(dtype)
@@ -251,8 +253,10 @@ def test_fused_elementwise_kernels_match_the_tensor_op_chains(dtype):
 
 
 @pytest.mark.gpu
-def test_fused_decoder_path_matches_the_module_chain():
-    """The same bf16 model stepped with and without the fused elementwise launches."""
+@pytest.mark.parametrize("batch", [2, 1])
+def test_fused_decoder_path_matches_the_module_chain(batch):
+    """The same bf16 model stepped with and without the fused elementwise launches. With one sequence the q slice of
+    a step's fused q/k/v row is a single row whose view still reports the stride of the wider row."""
     from fourierattention_amd import DynamicCache
     from fourierattention_amd.llama import LlamaConfig, random_init
     cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=3, num_attention_heads=4,
@@ -261,7 +265,7 @@ def test_fused_decoder_path_matches_the_module_chain():
     masks = _masks(3, 2, 64, [32, 32], [32, 32], seed=4)
     ec = lambda: _cfg(masks, numinittokens=4, maxlocallen=32, maxmidstates=64, num_key_value_heads=2, max_new_tokens=8,
                       max_position_embeddings=1024)
-    ids = torch.randint(0, cfg.vocab_size, (2, 200), generator=torch.Generator().manual_seed(3)).cuda()
+    ids = torch.randint(0, cfg.vocab_size, (batch, 200), generator=torch.Generator().manual_seed(3)).cuda()
     outs = []
     with torch.no_grad():
         for fused in (True, False, "projections"):
