@@ -284,11 +284,12 @@ def test_fused_decoder_path_matches_the_module_chain(batch):
                 tok = logits[-1].argmax(-1, keepdim=True)
             outs.append(torch.stack(logits))
     # identical rounding points; only reduction order (norm) and the exponential differ in the last place of bf16
+    # (logits of magnitude 0.5 - 1.5: one place of bf16 there is 0.004 - 0.008; the mean difference stays below one)
     torch.testing.assert_close(outs[0], outs[1], rtol=3e-2, atol=3e-2)
-    assert (outs[0] - outs[1]).abs().mean().item() < 3e-3
+    assert (outs[0] - outs[1]).abs().mean().item() < 5e-3
     # a wider GEMM may pick another tiling, hence another summation order inside the dot products
     torch.testing.assert_close(outs[2], outs[0], rtol=3e-2, atol=3e-2)
-    assert (outs[2] - outs[0]).abs().mean().item() < 3e-3
+    assert (outs[2] - outs[0]).abs().mean().item() < 5e-3
 
 
 @pytest.mark.gpu
