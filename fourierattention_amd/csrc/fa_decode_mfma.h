@@ -18,9 +18,8 @@
 // with C = E_cos . W'_cos and S = E_sin . W'_sin (cosine and sine ksteps in separate accumulators) the scores of
 // the second page are C + S and those of the first ("mirrored") page C - S, row i being token 31 - i there; g of
 // the frame takes E_cos^T (P2 + P1) and E_sin^T (P2 - P1), P1 / P2 being the probabilities of the first and of
-// the second page.  The coefficient-domain products are thus issued once per frame (the score pass of the two-pass
-// mode, which lacks the registers for C and S, still runs them per page with the sine rows of W' negated on the
-// mirrored page).  W' and the g history are rotated once per frame (64 tokens), not once per page.  On a mirrored page every
+// the second page.  The coefficient-domain products are thus issued once per frame, and W' and the g history are
+// rotated once per frame (64 tokens), not once per page.  On a mirrored page every
 // position-indexed quantity (score partials in LDS, probabilities) is held in the mirrored order; the K and V
 // pages come into LDS through per-lane addresses, so fetching a K fragment with its 16 rows reversed (and the two
 // 16-token blocks exchanged) or a V fragment with its four groups of 8 tokens exchanged costs nothing.
@@ -296,7 +295,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   using vec8 = typename M::vec8;
   constexpr int kFragsMax = (2 * KMAX > VMAX ? 2 * KMAX : VMAX);   // fragments (1 KiB) of one page of one wave
   // in the two-pass modes only waves 0-3 stream pages
-  static_assert(MODE != 1 || NST == 2, "the score pass waits for every outstanding access at the top of a page");
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[MODE == 0 ? 8 : 4][NST][kFragsMax * 1024];
   __shared__ float s_part[MODE == 2 ? 1 : 2][MODE == 2 ? 1 : NSL][16 * kPart];
   // value pass: the scores of a page travel like its V fragments, memory -> LDS without registers, every wave its own
@@ -489,13 +487,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(Ea[rb][ks]));
     rot_store();
     const unsigned rot_lane = lds_addr_of(&s_rot[(MODE == 2 ? 0 : sl * 2 * KS) * 4 + lg]);
-    // score pass: the complete scores of page pg of the split (sum of the eight partials; thread = (column,
-    // token)) go to memory.  Called one page late, behind that page's barrier.
+    // score pass: the complete scores of page pg of the split (sum of the eight partials; index = (column, token))
+    // go to memory.  Called one page late, behind that page's barrier, and carried out by waves 4-7 alone, two
+    // values per thread: they stream no pages, so waves 0-3 have nothing but page requests in flight and can count
+    // them (loads and stores do not complete in one order).
     auto flush_scores = [&](int pg) {
       if constexpr (MODE == 1) {
-        constexpr int kW = 16 * kPart * 4;   // bytes between the partials of two waves
-        const float sum = lds_sum8_b32<kW>(lds_addr_of(&s_part[pg & 1][0][(tid >> 5) * kPart + (tid & 31)]));
-        p.scores[((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pg) * 512 + tid] = sum;
+        if (w >= 4) {
+          constexpr int kW = 16 * kPart * 4;   // bytes between the partials of two waves
+          const int i0 = tid - 256;            // columns 0 .. 7; the second value belongs to column + 8
+          const unsigned at = lds_addr_of(&s_part[pg & 1][0][(i0 >> 5) * kPart + (i0 & 31)]);
+          const float sum0 = lds_sum8_b32<kW>(at);
+          const float sum1 = lds_sum8_b32<kW>(at + 8 * kPart * 4);
+          float* dst = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pg) * 512 + i0;
+          dst[0] = sum0;
+          dst[256] = sum1;
+        }
       }
     };
 
@@ -528,55 +535,38 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           kraw[2] = lds_read_b128_async_at<KMAX * 1024>(kst);
           kraw[3] = lds_read_b128_async_at<(KMAX + 1) * 1024>(kst);
         }
-        if (it > 0) flush_scores(it - 1);   // behind the page wait: the store has a whole page to complete
+        {
+          // (the trip number goes through an empty asm statement: a condition the compiler can resolve for the
+          // first trip makes it peel that trip, and the peeled copy of the loop body costs registers)
+          int it_seen = it;
+          asm volatile("" : "+s"(it_seen));
+          if (it_seen > 0) flush_scores(it - 1);   // behind the page wait: the store has a whole page to complete
+        }
         if constexpr (!mirrored) {
           rot_issue<0>(rot_lane, rc[0]);
           if (2 * KS > 4) rot_issue<1>(rot_lane, rc[1]);
         }
         float4v cd[2];   // coefficient-domain part of this page's scores, scaled, with the constant term
-        if constexpr (MODE == 1) {
-          // the score pass has no registers for C and S next to its operands: every page runs the whole product.
-          // The two pages of a frame convert the same W': without the pin the conversions of the second page are
-          // done together with those of the first and their results held across a whole page.
+        if constexpr (mirrored) {
+          accC[0] = accC[1] = accS[0] = accS[1] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int rt = 0; rt < 2 * KS; ++rt)
-            asm volatile("" : "+v"(Wc[rt][0]), "+v"(Wc[rt][1]), "+v"(Ws[rt][0]), "+v"(Ws[rt][1]));
-          float4v accf[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
-          for (int s = 0; s < KS; ++s) {
-            half8 wb;
+          for (int j = 0; j < KS / 2; ++j) {
+            half8 wbc, wbs;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const float wv = (s & 1) ? Ws[4 * (s >> 1) + (e >> 1)][e & 1] : Wc[4 * (s >> 1) + (e >> 1)][e & 1];
-              wb[e] = (_Float16)((mirrored && (s & 1)) ? -wv : wv);   // offsets -(i + 1/2): the sines change sign
+              wbc[e] = (_Float16)Wc[4 * j + (e >> 1)][e & 1];
+              wbs[e] = (_Float16)Ws[4 * j + (e >> 1)][e & 1];
             }
-            accf[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][s], wb, accf[0], 0, 0, 0);
-            accf[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][s], wb, accf[1], 0, 0, 0);
+            accC[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j], wbc, accC[0], 0, 0, 0);
+            accC[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j], wbc, accC[1], 0, 0, 0);
+            accS[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j + 1], wbs, accS[0], 0, 0, 0);
+            accS[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j + 1], wbs, accS[1], 0, 0, 0);
           }
-          cd[0] = accf[0] * colscale + c0col;
-          cd[1] = accf[1] * colscale + c0col;
-        } else {
-          if constexpr (mirrored) {
-            accC[0] = accC[1] = accS[0] = accS[1] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < KS / 2; ++j) {
-              half8 wbc, wbs;
-#pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                wbc[e] = (_Float16)Wc[4 * j + (e >> 1)][e & 1];
-                wbs[e] = (_Float16)Ws[4 * j + (e >> 1)][e & 1];
-              }
-              accC[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j], wbc, accC[0], 0, 0, 0);
-              accC[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j], wbc, accC[1], 0, 0, 0);
-              accS[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[0][2 * j + 1], wbs, accS[0], 0, 0, 0);
-              accS[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ea[1][2 * j + 1], wbs, accS[1], 0, 0, 0);
-            }
-          }
-          // offsets -(i + 1/2) on the mirrored page: the sines change sign
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
-            cd[rb] = (mirrored ? accC[rb] - accS[rb] : accC[rb] + accS[rb]) * colscale + c0col;
         }
+        // offsets -(i + 1/2) on the mirrored page: the sines change sign
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+          cd[rb] = (mirrored ? accC[rb] - accS[rb] : accC[rb] + accS[rb]) * colscale + c0col;
         // behind the second page of a frame: W' moves on to the centre of the next frame
         if constexpr (!mirrored) rot_apply_in_place_from<2 * KS, 0>(rot_lane, rc, Wc, Ws);
         float4v accm[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
@@ -606,7 +596,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int v = 0; v < 4; ++v) o[v] = cd[rb][v] + accm[rb][v] * p.sm_log2e;
           *(float4v*)&s_part[it & 1][sl][lc * kPart + rb * 16 + 4 * lg] = o;
         }
-      } else if (it > 0) {
+      } else if (n_it > 0) {   // (the trip after the last page)
         flush_scores(it - 1);
       }
       if (MODE == 0 || it < n_it) barrier_lds_only();

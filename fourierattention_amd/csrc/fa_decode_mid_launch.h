@@ -28,11 +28,11 @@ template <typename E>
 void launch_mid_mfma_two_pass(const MidParams<E>& mp, const MidLaunch& ml, hipStream_t st) {
   dim3 grid(ml.n_wg, ml.n_groups), flat(ml.n_wg * ml.n_groups);
   if (ml.wide) {
-    decode_mid_mfma_kernel<E, 8, 4, 8, 2, 1><<<grid, 512, 0, st>>>(mp);
+    decode_mid_mfma_kernel<E, 8, 4, 8, 3, 1><<<grid, 512, 0, st>>>(mp);
     if (ml.fused) decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2, true><<<flat, 512, 0, st>>>(mp);
     else decode_mid_mfma_kernel<E, 8, 4, 8, 3, 2><<<grid, 512, 0, st>>>(mp);
   } else {
-    decode_mid_mfma_kernel<E, 8, 2, 4, 2, 1><<<grid, 512, 0, st>>>(mp);
+    decode_mid_mfma_kernel<E, 8, 2, 4, 4, 1><<<grid, 512, 0, st>>>(mp);
     if (ml.fused) decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2, true><<<flat, 512, 0, st>>>(mp);
     else decode_mid_mfma_kernel<E, 8, 2, 4, 4, 2><<<grid, 512, 0, st>>>(mp);
   }
