@@ -115,10 +115,17 @@ def attn_step_bench(name, device, steps=100, warmup=10):
     from fourierattention_amd import _lib
     w = WORKLOADS[name]
     cache, q, kn, vn = build_cache(w, torch.bfloat16, device)
-    for _ in range(warmup):
-        out = cache.decode_attention(q, 0, w["Hq"], w["Hkv"])
-    torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # warm-up by time: at least ``warmup`` steps and 40 ms of them (the first tens of milliseconds after an idle
+    # period run slower than the steady state of a decode loop)
+    done_ms = 0.0
+    while done_ms < 40.0:
+        e0.record()
+        for _ in range(warmup):
+            out = cache.decode_attention(q, 0, w["Hq"], w["Hkv"])
+        e1.record()
+        torch.cuda.synchronize()
+        done_ms += e0.elapsed_time(e1)
     e0.record()
     for _ in range(steps):
         out = cache.decode_attention(q, 0, w["Hq"], w["Hkv"])
@@ -451,7 +458,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # (a device that has been idle runs its first 30 ms or so of work about 8 % slower than it does in the steady state of a
+    # decode loop; 300 steps are 35 ms at this workload)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--workload", default="config3_decode_attn_8b_32k", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the leg that uses the CPU restatement: the parity check before the timed region and the "
