@@ -34,7 +34,15 @@ def dtype_code(dt: torch.dtype) -> int:
         raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> int:
+    """Handle of the stream the caller's tensor work is queued on (torch's current stream of ``device``).  Looked up
+    on every call: the caller may switch streams, or capture into a graph, between two operators."""
+    if _raw_stream is not None:     # the bare handle, without building a torch.cuda.Stream object around it
+        idx = device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -309,6 +317,7 @@ class PackedLinearWeight:
         assert weight.dim() == 2 and weight.is_contiguous() and weight.dtype in (torch.bfloat16, torch.float16)
         self.n_out, self.k = int(weight.shape[0]), int(weight.shape[1])
         self.dtype = weight.dtype
+        self._rows_ok = {}     # row count -> whether the kernel takes it (asked once per count)
         self.data = torch.empty_like(weight)
         check(_lib.load().fa_linear_pack(weight.data_ptr(), self.data.data_ptr(), self.n_out, self.k, dtype_code(weight.dtype),
                                          _stream(weight.device)))
@@ -317,9 +326,13 @@ class PackedLinearWeight:
         return self.stamp.changed()
 
     def covers(self, x: torch.Tensor) -> bool:
-        rows = x.numel() // max(x.shape[-1], 1)
-        return (x.is_cuda and x.dtype == self.dtype and x.shape[-1] == self.k and x.stride(-1) == 1
-                and bool(_lib.load().fa_linear_packed_ok(rows, self.k, self.n_out)))
+        if not (x.is_cuda and x.dtype == self.dtype and x.shape[-1] == self.k and x.stride(-1) == 1):
+            return False
+        rows = x.numel() // max(self.k, 1)
+        ok = self._rows_ok.get(rows)
+        if ok is None:
+            ok = self._rows_ok[rows] = bool(_lib.load().fa_linear_packed_ok(rows, self.k, self.n_out))
+        return ok
 
 
 def linear_packed(x: torch.Tensor, w: PackedLinearWeight) -> torch.Tensor:
