@@ -458,9 +458,10 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    # (a device that has been idle runs its first 30 ms or so of work about 8 % slower than it does in the steady state of a
-    # decode loop; 300 steps are 35 ms at this workload)
-    ap.add_argument("--warmup", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-priming", action="store_true",
+                    help="skip the 60 ms of untimed steps that bring an idle device to the state of a running decode loop "
+                         "before the warm-up steps (comparison: the first 30 ms or so after an idle period run about 8 %% slower)")
     ap.add_argument("--workload", default="config3_decode_attn_8b_32k", choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the leg that uses the CPU restatement: the parity check before the timed region and the "
@@ -530,10 +531,22 @@ def main():
     cache.fuse_decode = not args.no_fuse
     cache.sub_splits = not args.no_sub_splits
     Hq, Hkv = w["Hq"], w["Hkv"]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # A decode loop runs for thousands of steps; a device that has been idle takes its first 30 ms or so of work
+    # about 8 % slower (both launches of the step, by the kernel trace) and a few hundred steps to settle.  The figure
+    # of merit is the settled one, so the same step first runs untimed for 60 ms, whatever --warmup and --steps say.
+    priming = {"steps": 0, "ms": 0.0}
+    while not args.no_priming and priming["ms"] < 60.0:
+        start.record()
+        for _ in range(50):
+            out = cache.decode_attention(q, 0, Hq, Hkv)
+        stop.record()
+        torch.cuda.synchronize()
+        priming["steps"] += 50
+        priming["ms"] = round(priming["ms"] + start.elapsed_time(stop), 2)
     for _ in range(args.warmup):
         out = cache.decode_attention(q, 0, Hq, Hkv)
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
     for _ in range(args.steps):
@@ -593,6 +606,7 @@ def main():
         "algorithmic_bytes_per_step": nbytes,
         "parity_max_abs_err": parity,
         "wall_ms_per_step": round(wall * 1e3 / args.steps, 5),
+        "untimed_steps_before_warmup": priming,
         "kernel_ms": {k: round(float(v), 5) for k, v in kernel_ms.items()},
         "merge_inside_mid_row_launch": merge_in_mid_rows,
         # each launch of kernel_ms sits between its own pair of HIP events; the pairs cost a few microseconds each,
