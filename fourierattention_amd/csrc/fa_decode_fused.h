@@ -429,11 +429,15 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
 #pragma unroll
     for (int u = 0; u < kPre; ++u) il_pre[u] = *(const float4v*)(il_src + (int64_t)min(x_cls + 4 * u, n_il - 1) * D);
   }
-  // (SUB: class j takes all splits of sub-split j, whose partials are those of virtual batch element 4 b0 + j)
-  const bool on_on = x_cl < ncol && 4 * x_d4 < vn_len;
-  const int on_first = SUB ? 0 : x_cls, on_step = SUB ? 1 : 4;
-  const int on_slot = SUB ? 4 * x_cls + c16_0 + x_cl : c16_0 + x_cl;
-  const float* on_src = p.pon + (SUB ? prow_of(on_slot) : qrow0 + x_cl) * NS * D + 4 * x_d4;
+  // (SUB: class j takes all splits of sub-split j, whose partials are those of virtual batch element 4 b0 + j - up to
+  // 32 of them, a chain of dependent loads if one thread walks them all.  A workgroup with one or two columns has
+  // threads for four: the spare ones help, thread column x_cl working for column x_cl % ncol on every on_h-th split.)
+  const int on_h = (SUB && (ncol == 1 || ncol == 2)) ? 4 / ncol : 1;
+  const int on_col = on_h > 1 ? x_cl % ncol : x_cl, on_hlp = on_h > 1 ? x_cl / ncol : 0;
+  const bool on_on = on_col < ncol && 4 * x_d4 < vn_len;
+  const int on_first = SUB ? on_hlp : x_cls, on_step = SUB ? on_h : 4;
+  const int on_slot = SUB ? 4 * x_cls + c16_0 + on_col : c16_0 + on_col;
+  const float* on_src = p.pon + (SUB ? prow_of(on_slot) : qrow0 + on_col) * NS * D + 4 * x_d4;
   if (on_on) {
 #pragma unroll
     for (int u = 0; u < kPre; ++u) on_pre[u] = *(const float4v*)(on_src + (int64_t)min(on_first + on_step * u, n_s - 1) * D);
@@ -559,10 +563,13 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
   float o_val = (s_red[((0 * 4 + o_cl) * 32) * 4 + o_d] + s_red[((1 * 4 + o_cl) * 32) * 4 + o_d]) +
                 (s_red[((2 * 4 + o_cl) * 32) * 4 + o_d] + s_red[((3 * 4 + o_cl) * 32) * 4 + o_d]);
   const int o_src = s_src[o_d];
-  if (o_src >= 128) {   // a stored dim: its sum
+  if (o_src >= 128) {   // a stored dim: its sum (over the classes, and over the helpers of the column)
     const int jj = o_src - 128;
-    o_val += (s_g[((0 * 4 + o_cl) * 32) * 4 + jj] + s_g[((1 * 4 + o_cl) * 32) * 4 + jj]) +
-             (s_g[((2 * 4 + o_cl) * 32) * 4 + jj] + s_g[((3 * 4 + o_cl) * 32) * 4 + jj]);
+    for (int hh = 0; hh < on_h; ++hh) {
+      const int sl = min(o_cl + hh * ncol, 3);
+      o_val += (s_g[((0 * 4 + sl) * 32) * 4 + jj] + s_g[((1 * 4 + sl) * 32) * 4 + jj]) +
+               (s_g[((2 * 4 + sl) * 32) * 4 + jj] + s_g[((3 * 4 + sl) * 32) * 4 + jj]);
+    }
   }
   __syncthreads();
   // the row classes of the product meet -> the row share's partial output per column, by position in the head's list
@@ -576,14 +583,41 @@ __device__ __forceinline__ void fused_merge_tail(const P& p, float* sm, float* s
     float* pc = pc_team + (int64_t)split * 16 * 128;
     // (SUB: the row classes hold four slots each, those of the query heads)
     constexpr int kSlots = SUB ? 4 : 16;
-    for (int idx = tid; idx < kSlots * f.nqp; idx += 512) {
-      const int c16 = idx >> f.lq, q = idx & (f.nqp - 1);
-      if (4 * q < f.vc_len && slot_ok(c16)) {
+    const int n_out = kSlots * f.nqp;
+    // the row classes [r0, r1) of one output (column slot, four dims) added up: four reads in flight, fixed order
+    // (the number of classes is a power of two, at least four)
+    auto class_sum = [&](int c16, int q, int r0, int r1) -> float4v {
+      float4v a4 = float4v{0.f, 0.f, 0.f, 0.f};
+      for (int rc = r0; rc < r1; rc += 4) {
+        float4v t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = *(const float4v*)(s_red + ((rc + u) * kSlots + c16) * 4 * f.nqp + 4 * q);
+        a4 += (t[0] + t[1]) + (t[2] + t[3]);
+      }
+      return a4;
+    };
+    // A head with few compressed dims has few outputs and many row classes (256 for eight dims of a single sequence):
+    // one thread per output walking them all is a chain of n_rc / 4 LDS round trips, 6 us there.  Then the classes are
+    // added up in `parts` pieces by as many threads per output, and the pieces by one (through s_g, free by now).
+    const int parts = f.n_rc >= 256 ? 16 : f.n_rc >= 64 ? 8 : f.n_rc >= 32 ? 4 : 1;
+    if (parts == 1) {
+      for (int idx = tid; idx < n_out; idx += 512) {
+        const int c16 = idx >> f.lq, q = idx & (f.nqp - 1);
+        if (4 * q < f.vc_len && slot_ok(c16)) *(float4v*)(pc + c16 * 128 + 4 * q) = class_sum(c16, q, 0, f.n_rc);
+      }
+    } else {
+      const int per = f.n_rc / parts;
+      const int o = tid & (n_out - 1), part = tid / n_out;   // (parts * n_out <= n_rc / 4 * n_out = 512)
+      const int c16 = o >> f.lq, q = o & (f.nqp - 1);
+      const bool live = 4 * q < f.vc_len && slot_ok(c16);
+      if (part < parts && live) *(float4v*)(s_g + (part * n_out + o) * 4) = class_sum(c16, q, part * per, (part + 1) * per);
+      __syncthreads();
+      if (part == 0 && live) {
         float4v a4 = float4v{0.f, 0.f, 0.f, 0.f};
-        for (int rc = 0; rc < f.n_rc; rc += 4) {   // (a power of two, at least four; four reads in flight, fixed order)
+        for (int pp = 0; pp < parts; pp += 4) {
           float4v t[4];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) t[u] = *(const float4v*)(s_red + ((rc + u) * kSlots + c16) * 4 * f.nqp + 4 * q);
+          for (int u = 0; u < 4; ++u) t[u] = *(const float4v*)(s_g + ((pp + u) * n_out + o) * 4);
           a4 += (t[0] + t[1]) + (t[2] + t[3]);
         }
         *(float4v*)(pc + c16 * 128 + 4 * q) = a4;
