@@ -31,6 +31,9 @@ CASES = [
     (torch.bfloat16, 4, 32, 4, 64, 1024, 3000, U, U, 1),                                   # a full group of four
     (torch.bfloat16, 8, 32, 4, 64, 512, 1500, [64, 0, 128, 30, 64, 64, 100, 64], [1, 64, 2, 3, 128, 64, 0, 64], 1),
     (torch.float16, 2, 16, 4, 40, 512, 2500, U, U, 1),                                     # two sequences: no sub-splits
+    # heads with few compressed V dims (8, 3, 0, 16, 64, 1, 28, 12): few outputs and many row classes in the tail's product
+    (torch.bfloat16, 4, 32, 4, 64, 512, 2500, U, [120, 125, 128, 112, 64, 127, 100, 116], 1),
+    (torch.bfloat16, 1, 32, 4, 64, 1024, 6000, U, [120, 125, 128, 112, 64, 127, 100, 116], 2),
     # 1024 frequencies: the value pass of the two merges its own partials
     (torch.bfloat16, 4, 24, 4, 40, 2048, 6000, U, U, 1),
     (torch.float16, 2, 32, 4, 64, 2048, 5000, [64, 0, 128, 30, 64, 64, 100, 64], [1, 64, 2, 3, 128, 64, 0, 64], 1),
