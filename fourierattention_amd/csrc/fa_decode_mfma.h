@@ -45,6 +45,7 @@ __device__ __forceinline__ int freq_of(int rt, int lg, int fi2) { return rt * 8 
 
 constexpr float kLazyLog2 = 8.0f;   // slack of the running softmax reference, in powers of two
 constexpr int kFreqWaves = 4;  // the coefficient rows are split four ways (one slice per SIMD)
+constexpr int kScoreFrames = 4;  // value pass: frames (two pages) of scores a workgroup keeps in LDS
 
 // ---------------------------------------------------------------------------
 // constant operand tables (depend on T and N only); KS = N / (16 * slices) ksteps per frequency slice
@@ -270,7 +271,8 @@ struct MidParams {
 // MODE 1, scores: eight partials per page meet in LDS, their sum (the complete score of the page) goes to
 //         memory (2 KiB per page and workgroup, against 16 KiB of K/V);
 // MODE 2, values: every wave reads the page's scores back, runs the softmax and keeps its slice of the g
-//         history; waves 0-3 stream V.  No exchange between the waves at all.
+//         history; waves 0-3 stream V, waves 4-7 bring the scores of a frame into LDS for all eight; one meeting
+//         per frame.
 // FUSE (MODE 0 and the value pass, MODE 2): the launch merges its own partials and writes the output rows, see fa_decode_fused.h; the
 // workgroups are then numbered through p.fz.wg_map so that the splits of a (batch group, KV head) share one die.
 // SUB (FUSE only, a batch of one sequence, at most four query heads per KV head): a single batch element would
@@ -297,10 +299,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // in the two-pass modes only waves 0-3 stream pages
   __shared__ __attribute__((aligned(16))) unsigned char s_stage[MODE == 0 ? 8 : 4][NST][kFragsMax * 1024];
   __shared__ float s_part[MODE == 2 ? 1 : 2][MODE == 2 ? 1 : NSL][16 * kPart];
-  // value pass: the scores of a page travel like its V fragments, memory -> LDS without registers, every wave its own
-  // copy (two fragments: positions 8 lg .. 8 lg + 3 and 8 lg + 4 .. 8 lg + 7 of column lc at lane * 16), so that
-  // the only accesses to vector memory inside the loop are page requests, whose arrival can be counted
-  __shared__ __attribute__((aligned(16))) unsigned char s_sc[MODE == 2 ? 8 : 1][MODE == 2 ? NST : 1][MODE == 2 ? 2048 : 16];
+  // value pass: the scores of a page travel like its V fragments, memory -> LDS without registers (two fragments per
+  // page: positions 8 lg .. 8 lg + 3 and 8 lg + 4 .. 8 lg + 7 of column lc at lane * 16), so that the only accesses
+  // to vector memory inside the loop are page requests, whose arrival can be counted.  One copy per workgroup, frame
+  // by frame: waves 4-7, which stream no V, bring one of the frame's four fragments each, and the workgroup meets
+  // once per frame.
+  __shared__ __attribute__((aligned(16))) unsigned char s_sc[MODE == 2 ? kScoreFrames : 1][MODE == 2 ? 4096 : 16];
   // frame-to-frame rotation constants, float4 = (c, s) of two neighbouring frequencies, [slice][unit][lane group]:
   // for the score waves unit = row tile rt, frequencies freq_of(rt, lg, 0 / 1); for the value waves unit u covers
   // the frequencies 16 (u / 2) + 4 lg + 2 (u % 2) + 0 / 1, the rows 4 lg + 2 (u % 2) + 0 / 1 of tile pair u / 2
@@ -624,23 +628,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     half8 ETa[2 * KS];   // tile 2j: cosines, tile 2j + 1: sines of the frequencies 16j .. 16j + 15 of the slice
 #pragma unroll
     for (int rt = 0; rt < 2 * KS; ++rt) ETa[rt] = p.tabET[(sl * 2 * KS + rt) * 64 + lane];
-    // value pass: the scores of page pgi of the split, into this wave's stage of that page
-    auto issue_sc = [&](int pgi) {
+    // value pass: the scores of frame fi of the split (pages 2 fi, 2 fi + 1) into the workgroup's stage of that frame;
+    // wave 4 + j brings fragment j of the four (a split with an odd number of pages: the second page of its last
+    // frame repeats the first and is never read)
+    const int n_fr = (n_it + 1) >> 1;
+    auto issue_sc = [&](int fi) {
       if constexpr (MODE == 2) {
-        const float* src = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pgi) * 512 + lc * 32 + 8 * lg;
-        unsigned char* st = &s_sc[w][pgi % NST][0];
-        load_frag_to_lds<0>(src, st);
-        load_frag_to_lds<0>(src + 4, st + 1024);
+        if (w >= 4) {
+          const int j = w - 4;
+          const int pgi = min(2 * fi + (j >> 1), n_it - 1);
+          const float* src = p.scores + ((int64_t)(grp * p.Hkv + h) * n_tiles + t_beg + pgi) * 512 + lc * 32 + 8 * lg + 4 * (j & 1);
+          load_frag_to_lds<0>(src, &s_sc[fi % kScoreFrames][j * 1024]);
+        }
       }
     };
     // first pages requested behind the table (see the score waves); page by page, so that the requests of a page
     // sit together in the order of arrival
 #pragma unroll
     for (int i = 0; i < NST - 1; ++i)
-      if (i < n_it) {
-        if (streams_v) issue_v(t_beg_w + i, (i & 1) == 0);
-        issue_sc(i);
-      }
+      if (i < n_it && streams_v) issue_v(t_beg_w + i, (i & 1) == 0);
+    if constexpr (MODE == 2) {
+#pragma unroll
+      for (int i = 0; i < kScoreFrames - 1; ++i)
+        if (i < n_fr) issue_sc(i);
+    }
     rot_store();
     float4v hacc[2 * KS], oacc[VMAX];
 #pragma unroll
@@ -675,16 +686,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           if (RCB == 2 && 2 * KS > 4) rot_issue<1>(rot_lane, rc[RCB - 1]);
         }
         float sc[8];
-        if constexpr (MODE == 2) {
-          // a page of this wave is its V fragments (if it streams V) and its two fragments of scores
-          if (pg + NST - 2 < n_it) wait_pages_in_flight<NST - 2, VMAX + 2, 1>((has_v ? ndg : 0) + 2);
-          else wait_vmcnt<0>();
-          // refills the stages read one page ago
-          if (pg + NST - 1 < n_it) {
-            if constexpr (has_v) issue_v(t + NST - 1, first_of_frame == (((NST - 1) & 1) == 0));
-            issue_sc(pg + NST - 1);
-          }
-        } else if constexpr (has_v) {
+        // (value pass: the scores of the frame have landed before the workgroup's meeting at the top of the frame)
+        if constexpr (has_v) {
           if (pg + NST - 2 < n_it) wait_pages_in_flight<NST - 2, VMAX, 1>(ndg);
           else wait_vmcnt<0>();
           // refills the stage read one page ago
@@ -731,7 +734,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         uint4v sraw[2];   // value pass: the scores of the page, column lc, positions 8*lg .. 8*lg + 7
         if constexpr (MODE == 2) {
-          const unsigned sst = lds_addr_of(&s_sc[w][pg % NST][0]) + lane * 16;
+          const unsigned sst = lds_addr_of(&s_sc[(pg >> 1) % kScoreFrames][(pg & 1) * 2048]) + lane * 16;
           sraw[0] = lds_read_b128_async_at<0>(sst);
           sraw[1] = lds_read_b128_async_at<1024>(sst);
         }
@@ -831,7 +834,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     };
     auto value_loop = [&](auto stream_tag) {
       if constexpr (MODE == 2) {
+        // One meeting per frame.  It hands over the frame's scores (every loading wave has seen its fragment land) and
+        // frees the stage of the frame before for the next request.  It also keeps the waves of a workgroup - and with
+        // them the workgroups of the launch - in step: without any meeting the page streams drift apart, some
+        // workgroups end a fifth later than the median one and the launch ends with them.
         for (int it = 1; it <= n_it; it += 2) {
+          const int fr = (it - 1) >> 1;
+          if (w >= 4) {
+            if (fr + kScoreFrames - 2 < n_fr) wait_vmcnt<kScoreFrames - 2>();
+            else wait_vmcnt<0>();
+          }
+          barrier_lds_only();
+          if (fr + kScoreFrames - 1 < n_fr) issue_sc(fr + kScoreFrames - 1);
           value_page(it, std::true_type{}, stream_tag);
           if (it + 1 <= n_it) value_page(it + 1, std::false_type{}, stream_tag);
         }
